@@ -1,0 +1,136 @@
+"""Builds the HIP kernel library for gfx950 with hipcc: one object per source, compiled in
+parallel, linked into ``libburnlm_hip.so`` next to the sources.  No other build system and no
+torch headers are involved, so a first build takes about a minute."""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libburnlm_hip.so"
+ARCH = "gfx950"
+# packed-fp32 instructions are kept off for every device pass
+HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def sources():
+    return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
+
+
+def source_hash():
+    h = hashlib.sha256()
+    for name in sources() + sorted(f for f in os.listdir(HERE) if f.endswith(".h")):
+        h.update(name.encode())
+        with open(os.path.join(HERE, name), "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+def _writable(d):
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, f".probe{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def out_dir():
+    """In-tree when the checkout is writable, else a per-user folder under the temp dir."""
+    if _writable(os.path.join(HERE, "_build")):
+        return HERE
+    d = os.path.join(tempfile.gettempdir(), f"burnlm_amd_{os.getuid()}_{source_hash()[:12]}")
+    os.makedirs(os.path.join(d, "_build"), exist_ok=True)
+    return d
+
+
+def lib_path():
+    return os.path.join(out_dir(), LIB_NAME)
+
+
+def _hash_path():
+    return os.path.join(out_dir(), "_build", "source.sha256")
+
+
+def is_current():
+    try:
+        with open(_hash_path()) as f:
+            return os.path.exists(lib_path()) and f.read().strip() == source_hash()
+    except OSError:
+        return False
+
+
+def find_hipcc():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): the HIP kernel "
+                       "library cannot be built, and there is no fallback path without it")
+
+
+def build(verbose=True, jobs=None):
+    """Compile every source and link the library.  Always compiles; returns the library path."""
+    hipcc = find_hipcc()
+    od = out_dir()
+    bdir = os.path.join(od, "_build")
+    srcs = sources()
+    jobs = jobs or min(len(srcs), 8)
+    log = (lambda *a: print("[burn-lm_amd build]", *a, file=sys.stderr, flush=True)) if verbose else (lambda *a: None)
+    log(f"compiling {len(srcs)} HIP sources for {ARCH} with {hipcc} ({jobs} at a time)")
+    t0 = time.time()
+    pending = list(srcs)
+    running = {}
+    objs = []
+    last_note = time.time()
+    while pending or running:
+        while pending and len(running) < jobs:
+            s = pending.pop(0)
+            o = os.path.join(bdir, s[:-4] + ".o")
+            objs.append(o)
+            p = subprocess.Popen([hipcc, *HIPCC_FLAGS, "-I", HERE, "-c", os.path.join(HERE, s), "-o", o],
+                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+            running[s] = p
+        for s, p in list(running.items()):
+            if p.poll() is not None:
+                out = p.stdout.read()
+                del running[s]
+                if p.returncode != 0:
+                    for q in running.values():
+                        q.kill()
+                    raise RuntimeError(f"hipcc failed on {s}:\n{out}")
+                log(f"  {s} done ({time.time() - t0:.0f} s)")
+        if running and time.time() - last_note > 15:
+            log(f"  still compiling: {', '.join(sorted(running))} ({time.time() - t0:.0f} s)")
+            last_note = time.time()
+        time.sleep(0.05)
+    tmp = os.path.join(bdir, LIB_NAME + f".{os.getpid()}.tmp")
+    r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc link failed:\n{r.stdout}")
+    os.replace(tmp, os.path.join(od, LIB_NAME))
+    with open(_hash_path(), "w") as f:
+        f.write(source_hash())
+    log(f"built {os.path.join(od, LIB_NAME)} in {time.time() - t0:.0f} s")
+    return os.path.join(od, LIB_NAME)
+
+
+def ensure_built(verbose=True):
+    """Path of a library that matches the sources, building it first if there is none."""
+    if is_current():
+        return lib_path()
+    return build(verbose=verbose)
+
+
+if __name__ == "__main__":
+    print(build())

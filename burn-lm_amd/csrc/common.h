@@ -1,0 +1,88 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, reductions.
+// Every kernel is a template over the storage type (float or bf16) and computes in float.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define BLM_WAVE 64
+
+struct bf16 {
+  uint16_t v;
+};
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16 x) { return __uint_as_float(((uint32_t)x.v) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_float(float f);
+template <>
+__device__ __forceinline__ float from_float<float>(float f) { return f; }
+template <>
+__device__ __forceinline__ bf16 from_float<bf16>(float f) { return bf16{f32_to_bf16_bits(f)}; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = BLM_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, BLM_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = BLM_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, BLM_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result. `red` holds 17 floats.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  const int lane = threadIdx.x & (BLM_WAVE - 1), w = threadIdx.x / BLM_WAVE;
+  const int nw = (blockDim.x + BLM_WAVE - 1) / BLM_WAVE;
+  v = wave_sum(v);
+  __syncthreads();  // red may still be read from an earlier call
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  if (w == 0) {
+    float t = lane < nw ? red[lane] : 0.f;
+    t = wave_sum(t);
+    if (lane == 0) red[16] = t;
+  }
+  __syncthreads();
+  return red[16];
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  const int lane = threadIdx.x & (BLM_WAVE - 1), w = threadIdx.x / BLM_WAVE;
+  const int nw = (blockDim.x + BLM_WAVE - 1) / BLM_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  if (w == 0) {
+    float t = lane < nw ? red[lane] : -INFINITY;
+    t = wave_max(t);
+    if (lane == 0) red[16] = t;
+  }
+  __syncthreads();
+  return red[16];
+}
+
+// Error reporting shared by the host entry points (defined in api.hip).
+int blm_fail(const char* fmt, ...);
+#define BLM_REQUIRE(cond, ...)            \
+  do {                                    \
+    if (!(cond)) return blm_fail(__VA_ARGS__); \
+  } while (0)
+#define BLM_LAUNCH_CHECK(name)                                                        \
+  do {                                                                                \
+    hipError_t e__ = hipGetLastError();                                               \
+    if (e__ != hipSuccess) return blm_fail("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+  } while (0)
+
+// dtype codes of the C ABI
+#define BLM_F32 0
+#define BLM_BF16 1

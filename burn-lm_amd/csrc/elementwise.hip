@@ -1,0 +1,193 @@
+// Row-wise kernels: embedding gather, residual add + RMS norm, rotary encoding with the write
+// of keys and values into the paged cache, SwiGLU gating.  All arithmetic is in float; inputs
+// and outputs are float or bf16.  The residual stream `h` is always float.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------
+// embedding: h[t, :] = table[ids[t], :]
+// ---------------------------------------------------------------------------------------
+template <typename TW>
+__global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ h, int D) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const TW* row = table + (size_t)id * D;
+  float* out = h + (size_t)t * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) out[d] = to_float(row[d]);
+}
+
+extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* ids, float* h,
+                                int T, int D, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && D > 0, "embed_gather: bad sizes T=%d D=%d", T, D);
+  dim3 grid(T), block(256);
+  if (table_dtype == BLM_F32)
+    hipLaunchKernelGGL(embed_gather_kernel<float>, grid, block, 0, stream, (const float*)table, ids, h, D);
+  else if (table_dtype == BLM_BF16)
+    hipLaunchKernelGGL(embed_gather_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, h, D);
+  else
+    return blm_fail("embed_gather: unsupported table dtype %d", table_dtype);
+  BLM_LAUNCH_CHECK("embed_gather");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// residual add + RMS norm
+//   v = h[r] (+ delta[r]);  if write_h: h[r] = v;  out[i] = v / sqrt(mean(v^2) + eps) * gamma
+//   r = rows ? rows[i] : i
+// ---------------------------------------------------------------------------------------
+template <typename TA, typename TG>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+                                   const TG* __restrict__ gamma, TA* __restrict__ out,
+                                   const int* __restrict__ rows, int D, float eps, int write_h) {
+  __shared__ float red[17];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* hr = h + (size_t)r * D;
+  const TA* dr = delta ? delta + (size_t)r * D : nullptr;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float v = hr[d];
+    if (dr) {
+      v += to_float(dr[d]);
+      if (write_h) hr[d] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+  TA* o = out + (size_t)i * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float v = hr[d];
+    if (dr && !write_h) v += to_float(dr[d]);
+    o[d] = from_float<TA>(v * inv * to_float(gamma[d]));
+  }
+}
+
+extern "C" int blm_add_rmsnorm(float* h, const void* delta, const void* gamma, int gamma_dtype,
+                               void* out, int act_dtype, const int* rows, int n_out, int D,
+                               float eps, int write_h, hipStream_t stream) {
+  BLM_REQUIRE(n_out > 0 && D > 0, "add_rmsnorm: bad sizes n=%d D=%d", n_out, D);
+  dim3 grid(n_out), block(D >= 2048 ? 512 : 256);
+#define BLM_NORM_CASE(TA, TG)                                                                  \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG>), grid, block, 0, stream, h, (const TA*)delta, \
+                     (const TG*)gamma, (TA*)out, rows, D, eps, write_h)
+  if (act_dtype == BLM_F32 && gamma_dtype == BLM_F32) BLM_NORM_CASE(float, float);
+  else if (act_dtype == BLM_BF16 && gamma_dtype == BLM_BF16) BLM_NORM_CASE(bf16, bf16);
+  else if (act_dtype == BLM_BF16 && gamma_dtype == BLM_F32) BLM_NORM_CASE(bf16, float);
+  else if (act_dtype == BLM_F32 && gamma_dtype == BLM_BF16) BLM_NORM_CASE(float, bf16);
+  else return blm_fail("add_rmsnorm: unsupported dtypes act=%d gamma=%d", act_dtype, gamma_dtype);
+#undef BLM_NORM_CASE
+  BLM_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// rotary encoding of q (in place) and k, and the write of k, v into the paged cache
+//   qkv row layout: [q: nh*hd | k: nkv*hd | v: nkv*hd]
+//   cache plane layout: [page][kv head][slot in page][hd]
+//   pairing 0: lanes (2i, 2i+1) form a pair; pairing 1: lanes (i, i + hd/2)
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict__ positions,
+                                     const int* __restrict__ token_seq,
+                                     const int* __restrict__ block_table, int table_width,
+                                     const float2* __restrict__ cos_sin, TA* __restrict__ kcache,
+                                     TA* __restrict__ vcache, int page_size, int nh, int nkv,
+                                     int hd, int pairing, int write_kv) {
+  const int t = blockIdx.x;
+  const int b = token_seq[t];
+  if (b < 0) return;  // padding token
+  const int pos = positions[t];
+  const int half = hd >> 1;
+  TA* row = qkv + (size_t)t * (size_t)(nh + 2 * nkv) * hd;
+  const float2* cs = cos_sin + (size_t)pos * half;
+  const int page = block_table[(size_t)b * table_width + pos / page_size];
+  const int slot = pos % page_size;
+  const bool store = write_kv && page >= 0;
+
+  // rotations: heads 0..nh-1 are queries, nh..nh+nkv-1 keys
+  const int n_rot = (nh + nkv) * half;
+  for (int w = threadIdx.x; w < n_rot; w += blockDim.x) {
+    const int head = w / half, i = w - head * half;
+    const int i0 = pairing == 0 ? 2 * i : i;
+    const int i1 = pairing == 0 ? 2 * i + 1 : i + half;
+    TA* x = row + (size_t)head * hd;
+    const float x0 = to_float(x[i0]), x1 = to_float(x[i1]);
+    const float2 c = cs[i];
+    const TA y0 = from_float<TA>(x0 * c.x - x1 * c.y);
+    const TA y1 = from_float<TA>(x0 * c.y + x1 * c.x);
+    if (head < nh) {
+      x[i0] = y0;
+      x[i1] = y1;
+    } else if (store) {
+      TA* kd = kcache + (((size_t)page * nkv + (head - nh)) * page_size + slot) * hd;
+      kd[i0] = y0;
+      kd[i1] = y1;
+    }
+  }
+  if (store) {
+    const TA* v = row + (size_t)(nh + nkv) * hd;
+    for (int w = threadIdx.x; w < nkv * hd; w += blockDim.x) {
+      const int head = w / hd, d = w - head * hd;
+      vcache[(((size_t)page * nkv + head) * page_size + slot) * hd + d] = v[w];
+    }
+  }
+}
+
+extern "C" int blm_rope_kv_write(void* qkv, int act_dtype, const int* positions,
+                                 const int* token_seq, const int* block_table, int table_width,
+                                 const float* cos_sin, void* kcache, void* vcache, int page_size,
+                                 int T, int nh, int nkv, int hd, int pairing, int write_kv,
+                                 hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && hd > 0 && (hd % 2) == 0,
+              "rope_kv_write: bad sizes T=%d nh=%d nkv=%d head_dim=%d (head_dim must be even)", T, nh, nkv, hd);
+  BLM_REQUIRE(page_size > 0 && table_width > 0, "rope_kv_write: bad cache geometry");
+  BLM_REQUIRE(pairing == 0 || pairing == 1, "rope_kv_write: pairing %d unknown", pairing);
+  dim3 grid(T), block(256);
+  if (act_dtype == BLM_F32)
+    hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)qkv, positions, token_seq,
+                       block_table, table_width, (const float2*)cos_sin, (float*)kcache, (float*)vcache,
+                       page_size, nh, nkv, hd, pairing, write_kv);
+  else if (act_dtype == BLM_BF16)
+    hipLaunchKernelGGL(rope_kv_write_kernel<bf16>, grid, block, 0, stream, (bf16*)qkv, positions, token_seq,
+                       block_table, table_width, (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache,
+                       page_size, nh, nkv, hd, pairing, write_kv);
+  else
+    return blm_fail("rope_kv_write: unsupported dtype %d", act_dtype);
+  BLM_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// SwiGLU gating: out[t, i] = silu(gu[t, i]) * gu[t, I + i]
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void swiglu_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I) {
+  const int t = blockIdx.y;
+  const TA* g = gu + (size_t)t * 2 * I;
+  TA* o = out + (size_t)t * I;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < I; i += gridDim.x * blockDim.x) {
+    const float z = to_float(g[i]), u = to_float(g[I + i]);
+    o[i] = from_float<TA>(z / (1.0f + expf(-z)) * u);
+  }
+}
+
+extern "C" int blm_swiglu(const void* gu, void* out, int act_dtype, int T, int I, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && I > 0 && T <= 65535 * 64, "swiglu: bad sizes T=%d I=%d", T, I);
+  int gx = (I + 255) / 256;
+  if (gx > 64) gx = 64;
+  for (int t0 = 0; t0 < T; t0 += 65535) {
+    int tn = T - t0 < 65535 ? T - t0 : 65535;
+    dim3 grid(gx, tn), block(256);
+    if (act_dtype == BLM_F32)
+      hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)gu + (size_t)t0 * 2 * I,
+                         (float*)out + (size_t)t0 * I, I);
+    else if (act_dtype == BLM_BF16)
+      hipLaunchKernelGGL(swiglu_kernel<bf16>, grid, block, 0, stream, (const bf16*)gu + (size_t)t0 * 2 * I,
+                         (bf16*)out + (size_t)t0 * I, I);
+    else
+      return blm_fail("swiglu: unsupported dtype %d", act_dtype);
+  }
+  BLM_LAUNCH_CHECK("swiglu");
+  return 0;
+}

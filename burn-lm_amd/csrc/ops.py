@@ -1,0 +1,257 @@
+"""Python face of the HIP kernel library: loads ``libburnlm_hip.so`` through ctypes and wraps
+each entry point with checks of device, dtype, shape and contiguity.  Kernels run on torch's
+current HIP stream.  There is no fallback: without the library, or off the GPU, calls raise."""
+from __future__ import annotations
+
+import ctypes
+import threading
+
+import torch
+
+from . import build as _build
+
+ABI_VERSION = 1
+_lib = None
+_lock = threading.Lock()
+
+_c_int, _c_float, _c_void_p = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or failed to launch."""
+
+
+_SIGNATURES = {
+    "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int,
+                        _c_int, _c_float, _c_int, _c_void_p],
+    "blm_rope_kv_write": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
+                          _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_attn_paged": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                       _c_void_p],
+    "blm_gemm_tiled": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_void_p],
+    "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                        _c_int, _c_int, _c_void_p],
+    "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
+}
+
+
+def library():
+    """The loaded kernel library; built from source at the first call if it is not there."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                path = _build.ensure_built()
+                lib = ctypes.CDLL(path)
+                lib.blm_last_error.restype = ctypes.c_char_p
+                lib.blm_abi_version.restype = _c_int
+                if lib.blm_abi_version() != ABI_VERSION:
+                    raise KernelError(f"{path} has ABI {lib.blm_abi_version()}, expected {ABI_VERSION}: rebuild it")
+                for name, sig in _SIGNATURES.items():
+                    fn = getattr(lib, name)
+                    fn.argtypes = sig
+                    fn.restype = _c_int
+                _lib = lib
+    return _lib
+
+
+def library_file():
+    return _build.lib_path()
+
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _code(t):
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"dtype {t.dtype} is not supported by the kernels (float32 or bfloat16)") from None
+
+
+def _gpu(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError("the kernels run on the GPU only: got a tensor on " + str(t.device))
+
+
+def _contig(name, t):
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+
+
+def _i32(name, t, n=None):
+    if t.dtype != torch.int32:
+        raise KernelError(f"{name} must be int32, got {t.dtype}")
+    _contig(name, t)
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name} has {t.numel()} elements, needs {n}")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _call(name, *args):
+    lib = library()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise KernelError(lib.blm_last_error().decode())
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+# ------------------------------------------------------------------------------------------
+def embed_gather(table, ids, out_h):
+    """out_h[t, :] = table[ids[t], :] as float32.  ids must already be checked against the vocabulary."""
+    _gpu(table, ids, out_h)
+    T, D = out_h.shape
+    _i32("ids", ids, T)
+    _contig("table", table); _contig("h", out_h)
+    if out_h.dtype != torch.float32 or table.shape[1] != D:
+        raise KernelError("embed_gather: h must be float32 [T, D] with D the table's width")
+    _call("blm_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out_h.data_ptr(), T, D, _stream())
+    return out_h
+
+
+def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True):
+    """v = h[r] (+ delta[r]); h[r] = v if write_h; out[i] = v / sqrt(mean(v^2) + eps) * gamma,
+    with r = rows[i] if rows is given, else i.  h is the float32 residual stream."""
+    _gpu(h, delta, gamma, out, rows)
+    D = h.shape[1]
+    n_out = out.shape[0]
+    if h.dtype != torch.float32:
+        raise KernelError("add_rmsnorm: the residual stream must be float32")
+    _contig("h", h); _contig("out", out); _contig("gamma", gamma)
+    if gamma.numel() != D or out.shape[1] != D:
+        raise KernelError(f"add_rmsnorm: width mismatch h={D} gamma={gamma.numel()} out={out.shape[1]}")
+    if delta is not None:
+        _contig("delta", delta)
+        if delta.shape != h.shape or delta.dtype != out.dtype:
+            raise KernelError("add_rmsnorm: delta must match h in shape and out in dtype")
+    if rows is not None:
+        _i32("rows", rows, n_out)
+    elif n_out != h.shape[0]:
+        raise KernelError("add_rmsnorm: out needs one row per row of h when rows is not given")
+    _call("blm_add_rmsnorm", h.data_ptr(), _ptr(delta), gamma.data_ptr(), _code(gamma), out.data_ptr(), _code(out),
+          _ptr(rows), n_out, D, float(eps), 1 if write_h else 0, _stream())
+    return out
+
+
+def rope_kv_write(qkv, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,
+                  nh, nkv, hd, pairing, write_kv=True):
+    """Rotate q (in place) and k of each token by its position's angles and store k, v in the
+    paged cache.  cos_sin: float32 [positions, hd/2, 2].  Cache planes: [pages, nkv, page, hd]."""
+    _gpu(qkv, positions, token_seq, block_table, cos_sin, kcache, vcache)
+    T = qkv.shape[0]
+    _contig("qkv", qkv); _contig("cos_sin", cos_sin); _contig("kcache", kcache); _contig("vcache", vcache)
+    if qkv.shape[1] != (nh + 2 * nkv) * hd:
+        raise KernelError(f"rope_kv_write: qkv row is {qkv.shape[1]}, expected {(nh + 2 * nkv) * hd}")
+    _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
+    if cos_sin.dtype != torch.float32 or cos_sin.shape[1:] != (hd // 2, 2):
+        raise KernelError("rope_kv_write: cos_sin must be float32 [positions, head_dim/2, 2]")
+    if kcache.dtype != qkv.dtype or vcache.dtype != qkv.dtype:
+        raise KernelError("rope_kv_write: cache and activations must share a dtype")
+    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or kcache.shape != vcache.shape:
+        raise KernelError(f"rope_kv_write: cache plane shape {tuple(kcache.shape)} does not fit "
+                          f"[pages, {nkv}, {page_size}, {hd}]")
+    _call("blm_rope_kv_write", qkv.data_ptr(), _code(qkv), positions.data_ptr(), token_seq.data_ptr(),
+          block_table.data_ptr(), block_table.shape[1], cos_sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
+          page_size, T, nh, nkv, hd, pairing, 1 if write_kv else 0, _stream())
+
+
+def swiglu(gate_up, out):
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _gpu(gate_up, out)
+    T, I = out.shape
+    _contig("gate_up", gate_up); _contig("out", out)
+    if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype:
+        raise KernelError("swiglu: gate_up must be [T, 2I] of out's dtype")
+    _call("blm_swiglu", gate_up.data_ptr(), out.data_ptr(), _code(out), T, I, _stream())
+    return out
+
+
+def attn_paged(q, q_row_stride, out, positions, token_seq, block_table, kcache, vcache, page_size,
+               nh, nkv, hd, scale, window=0):
+    """Attention of every query token over its sequence's cached keys (generic kernel).
+    q: first nh*hd columns of rows with stride q_row_stride; out: [T, nh*hd]."""
+    _gpu(q, out, positions, token_seq, block_table, kcache, vcache)
+    T = out.shape[0]
+    _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
+    if out.shape[1] != nh * hd or out.dtype != q.dtype or kcache.dtype != q.dtype:
+        raise KernelError("attn_paged: out must be [T, heads*head_dim] and share q's dtype with the cache")
+    if q.stride(-1) != 1 or q_row_stride < nh * hd:
+        raise KernelError("attn_paged: q rows must be contiguous and at least heads*head_dim long")
+    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or kcache.shape != vcache.shape:
+        raise KernelError("attn_paged: cache plane shape does not fit [pages, kv_heads, page, head_dim]")
+    _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
+    _call("blm_attn_paged", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
+          token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
+          page_size, T, nh, nkv, hd, float(scale), int(window), _stream())
+    return out
+
+
+def _check_mm(a, w, out):
+    _gpu(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or out.shape != (M, N):
+        raise KernelError(f"matrix product: shapes a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)} do not fit")
+    if a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("matrix product: a and out need unit stride along their rows")
+    _contig("w", w)
+    return M, N, K
+
+
+def gemm_tiled(a, w, out):
+    """out[M,N] = a[M,K] @ w[N,K]^T with float accumulation by plain fused multiply-adds."""
+    M, N, K = _check_mm(a, w, out)
+    _call("blm_gemm_tiled", a.data_ptr(), _code(a), w.data_ptr(), _code(w), out.data_ptr(), _code(out),
+          M, N, K, a.stride(0), out.stride(0), _stream())
+    return out
+
+
+def gemv_skinny(a, w, out):
+    """The same product for M <= 8 rows; streams w once."""
+    M, N, K = _check_mm(a, w, out)
+    _call("blm_gemv_skinny", a.data_ptr(), _code(a), w.data_ptr(), _code(w), out.data_ptr(), _code(out),
+          M, N, K, a.stride(0), out.stride(0), _stream())
+    return out
+
+
+def argmax(logits, out=None):
+    """First index of each row's maximum of float32 logits [R, V] -> int32 [R]."""
+    _gpu(logits, out)
+    R, V = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("argmax: logits must be float32 with unit stride along the vocabulary")
+    if out is None:
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    _i32("out", out, R)
+    _call("blm_argmax", logits.data_ptr(), out.data_ptr(), R, V, logits.stride(0), _stream())
+    return out
+
+
+def sample(logits, uniforms, temperature, top_p=1.0, out=None):
+    """Pick from softmax(logits / temperature) cut to the top-p nucleus at the given uniforms."""
+    _gpu(logits, uniforms, out)
+    R, V = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be float32 with unit stride along the vocabulary")
+    if uniforms.dtype != torch.float32 or uniforms.numel() < R or not uniforms.is_contiguous():
+        raise KernelError("sample: uniforms must be contiguous float32 with one value per row")
+    if out is None:
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    _i32("out", out, R)
+    _call("blm_sample", logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), R, V, logits.stride(0),
+          float(temperature), float(top_p), _stream())
+    return out

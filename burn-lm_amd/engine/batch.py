@@ -1,0 +1,73 @@
+"""One step's batch: the tokens of several sequences packed into one run, with everything the
+kernels need to know about where each token belongs."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Sequence
+
+import torch
+
+
+@dataclass
+class Step:
+    n_tokens: int
+    n_seqs: int
+    n_wanted: int
+    token_ids: torch.Tensor      # int32 [tokens]
+    positions: torch.Tensor      # int32 [tokens]  absolute position of each token in its sequence
+    token_seq: torch.Tensor      # int32 [tokens]  index of the token's sequence in this step (-1: padding)
+    seq_slots: torch.Tensor      # int32 [seqs]    cache slot of each sequence (-1: padding)
+    cu_seqlens: torch.Tensor     # int32 [seqs+1]  first token of each sequence in the packed run
+    lens_after: torch.Tensor     # int32 [seqs]    length of each sequence once this step has run
+    want_rows: torch.Tensor      # int32 [wanted]  packed rows whose logits are asked for
+    block_tables: Dict[int, torch.Tensor] = field(default_factory=dict)  # group -> int32 [seqs, width]
+    max_new: int = 1             # most tokens any sequence brings
+    max_position: int = 0        # largest position in the step
+    max_len_after: int = 0
+    is_decode: bool = False      # every sequence brings exactly one token
+    host_slots: List[int] = field(default_factory=list)
+    host_new: List[int] = field(default_factory=list)
+
+
+def build_step(entries: Sequence, lengths: Sequence[int], cache, device) -> Step:
+    """entries: (slot, tokens, want) per sequence; lengths: what each already holds.  All index
+    arrays go to the device in one copy."""
+    tok, pos, seq, rows, cu, after, slots = [], [], [], [], [0], [], []
+    for b, ((slot, tokens, want), past) in enumerate(zip(entries, lengths)):
+        n = len(tokens)
+        base = len(tok)
+        tok.extend(tokens)
+        pos.extend(range(past, past + n))
+        seq.extend([b] * n)
+        rows.extend(base + w for w in want)
+        cu.append(base + n)
+        after.append(past + n)
+        slots.append(slot)
+    T, B, R = len(tok), len(entries), len(rows)
+    max_after = max(after)
+    width = max(1, (max_after + cache.page_size - 1) // cache.page_size)
+    tables = [cache.page_table(gi, slots, width) for gi in range(len(cache.groups))]
+    flat = tok + pos + seq + slots + cu + after + rows
+    for t in tables:
+        for r in t:
+            flat.extend(r)
+    host = torch.tensor(flat, dtype=torch.int32)
+    if device.type == "cuda":
+        host = host.pin_memory()
+    dev = host.to(device, non_blocking=True)
+    o = 0
+
+    def take(n):
+        nonlocal o
+        v = dev[o:o + n]
+        o += n
+        return v
+
+    token_ids, positions, token_seq = take(T), take(T), take(T)
+    seq_slots, cu_seqlens, lens_after, want_rows = take(B), take(B + 1), take(B), take(R)
+    block_tables = {gi: take(B * width).view(B, width) for gi in range(len(tables))}
+    news = [len(e[1]) for e in entries]
+    return Step(n_tokens=T, n_seqs=B, n_wanted=R, token_ids=token_ids, positions=positions, token_seq=token_seq,
+                seq_slots=seq_slots, cu_seqlens=cu_seqlens, lens_after=lens_after, want_rows=want_rows,
+                block_tables=block_tables, max_new=max(news), max_position=max_after - 1, max_len_after=max_after,
+                is_decode=all(n == 1 for n in news), host_slots=slots, host_new=news)

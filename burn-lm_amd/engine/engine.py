@@ -1,0 +1,84 @@
+"""The step function: a model, its cache, and one call that runs exactly the tokens it is given.
+
+``step(entries)`` takes, per sequence, its slot, its next tokens and the places among them whose
+logits are wanted.  The sequences of a call may have different lengths and different pasts; the
+tokens run as one packed batch, each attending to its own sequence's cache, and the logits of
+the wanted rows come back as float32 ``[wanted, vocab]`` in the order of the entries and of
+their ``want`` lists.  Position of the t-th new token of a sequence = tokens it already holds + t
+(crates/burn-lm-llama/src/nn/pos_encoding.rs:66-79).  Everything is checked before anything
+changes: a refused step leaves cache and sequences as they were.  One iteration body of the
+reference's loop (crates/burn-lm-llama/src/generation/generate.rs:66-85) is one such step.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.cache import Cache, CacheError
+
+
+class StepError(ValueError):
+    pass
+
+
+class Engine:
+    def __init__(self, model, rt, max_tokens: int, max_seqs: Optional[int] = None,
+                 max_context: Optional[int] = None, page_size: int = 64):
+        self.model, self.rt = model, rt
+        plan_max = model.plan.max_positions
+        n_pages = (max_tokens + page_size - 1) // page_size
+        max_context = min(max_context or plan_max, plan_max, n_pages * page_size)
+        max_seqs = max_seqs or min(n_pages, 4096)
+        self.cache = Cache(model.cache_needs(), model.reads_from(), max_tokens=n_pages * page_size,
+                           max_seqs=max_seqs, max_context=max_context, page_size=page_size,
+                           dtype=rt.dtype, device=rt.device)
+        model.prepare_positions(max_context)
+        self.max_context = max_context
+        self.vocab_size = model.vocab_size
+
+    # ---- sequences ---------------------------------------------------------------------------
+    def open(self) -> int:
+        return self.cache.open()
+
+    def close(self, slot: int) -> None:
+        self.cache.close(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    def clear(self) -> None:
+        """Close every live sequence."""
+        for s in self.cache.live_slots:
+            self.cache.close(s)
+
+    # ---- the step ----------------------------------------------------------------------------
+    def _check(self, entries):
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        V = self.vocab_size
+        for slot, tokens, want in entries:
+            n = len(tokens)
+            if n == 0:
+                raise StepError(f"slot {slot}: a step must bring at least one token per sequence")
+            for t in tokens:
+                if not (isinstance(t, int) and 0 <= t < V):
+                    raise StepError(f"slot {slot}: token {t!r} is outside the vocabulary of {V}")
+            for w in want:
+                if not (isinstance(w, int) and 0 <= w < n):
+                    raise StepError(f"slot {slot}: wanted place {w!r} is outside this step's {n} tokens")
+
+    def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> Optional[torch.Tensor]:
+        entries = [(int(s), list(t), list(w)) for s, t, w in entries]
+        self._check(entries)
+        lengths = [self.cache.length(s) for s, _, _ in entries]
+        self.cache.reserve([(s, len(t)) for s, t, _ in entries])  # raises before any change
+        step = self.build_step(entries, lengths)
+        logits = self.model.forward(step, self.cache)
+        for s, t, _ in entries:
+            self.cache.advance(s, len(t))
+        return logits
+
+    def build_step(self, entries, lengths):
+        from .batch import build_step
+        return build_step(entries, lengths, self.cache, self.rt.device)

@@ -1,0 +1,66 @@
+"""From a model folder to an engine: read config.json, find the architecture in the registry,
+plan the parts, load the tensors by name, build the cache."""
+from __future__ import annotations
+
+import json
+import os
+import time
+
+import torch
+
+from .. import models, parts, registry  # noqa: F401  (registration happens at import)
+from ..config.llama import ConfigError
+from ..weights import loader, safetensors_io
+from .engine import Engine
+from .model import Model
+from .runtime import Runtime
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
+          "fp32": torch.float32}
+
+
+def parse_dtype(name):
+    if isinstance(name, torch.dtype):
+        return name
+    try:
+        return DTYPES[str(name).lower()]
+    except KeyError:
+        raise ValueError(f"dtype {name!r} unknown; one of bfloat16, float32") from None
+
+
+def read_config(folder):
+    path = os.path.join(folder, "config.json")
+    try:
+        with open(path) as f:
+            d = json.load(f)
+    except FileNotFoundError:
+        raise ConfigError(f"{path} not found: a model folder holds config.json and model.safetensors") from None
+    except json.JSONDecodeError as e:
+        raise ConfigError(f"{path} is not valid JSON: {e}") from None
+    arch = registry.architecture_of(d)
+    return arch, arch.read_config(d)
+
+
+def load_model(folder, dtype="bfloat16", device="cuda:0"):
+    """-> (Model bound to its tensors, Runtime, typed configuration)."""
+    dtype = parse_dtype(dtype)
+    arch, cfg = read_config(folder)
+    rt = Runtime(dtype=dtype, device=device)
+    available = safetensors_io.open_folder(folder)
+    plan = arch.plan(cfg, set(available))
+    model = Model(plan)
+    tensors = loader.load(folder, model.tensor_specs(), dtype, rt.device, plan.ignorable_tensors, available)
+    model.bind(tensors, rt)
+    model.config = cfg
+    model.architecture = arch
+    return model, rt, cfg
+
+
+def load_engine(folder, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_context=None, device="cuda:0",
+                page_size=64):
+    t0 = time.time()
+    model, rt, cfg = load_model(folder, dtype, device)
+    eng = Engine(model, rt, max_tokens=max_tokens, max_seqs=max_seqs, max_context=max_context, page_size=page_size)
+    eng.config = cfg
+    eng.load_seconds = time.time() - t0
+    return eng

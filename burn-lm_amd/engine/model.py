@@ -1,0 +1,80 @@
+"""Builds a runnable model from a plan: instantiates the parts by their registered kinds,
+collects the tensors they ask for, binds the loaded tensors, and runs a step through the places
+of the layer order."""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from .. import registry
+from ..models.plan import ModelPlan
+from ..parts.base import TensorSpec
+
+
+class Model:
+    def __init__(self, plan: ModelPlan):
+        self.plan = plan
+        self.positions = {k: registry.part("position", s.kind)(s.params, s.names) for k, s in plan.positions.items()}
+        self.embedding = registry.part("embedding", plan.embedding.kind)(plan.embedding.params, plan.embedding.names)
+        self.final_norm = registry.part("norm", plan.final_norm.kind)(plan.final_norm.params, plan.final_norm.names)
+        self.head = registry.part("head", plan.head.kind)(plan.head.params, plan.head.names)
+        self.blocks = []
+        for lp in plan.layers:
+            mp = dict(lp.mixer.params)
+            if lp.position is not None:
+                mp["position"] = self.positions[lp.position]
+            mixer = registry.part("mixer", lp.mixer.kind)(mp, lp.mixer.names)
+            ffn = registry.part("feed_forward", lp.feed_forward.kind)(lp.feed_forward.params, lp.feed_forward.names)
+            n1 = registry.part("norm", lp.mixer_norm.kind)(lp.mixer_norm.params, lp.mixer_norm.names)
+            n2 = registry.part("norm", lp.ffn_norm.kind)(lp.ffn_norm.params, lp.ffn_norm.names)
+            self.blocks.append(registry.part("block", lp.block)(mixer, ffn, n1, n2))
+        for i, place in enumerate(plan.order):
+            if not 0 <= place.layer < len(self.blocks):
+                raise ValueError(f"place {i} of the layer order names layer {place.layer}, "
+                                 f"but there are {len(self.blocks)} layers")
+        self.vocab_size = plan.vocab_size
+        self.rt = None
+
+    def all_parts(self):
+        yield self.embedding
+        for b in self.blocks:
+            yield from b.parts()
+        yield self.final_norm
+        yield self.head
+        yield from self.positions.values()
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+        for p in self.all_parts():
+            for name, spec in p.tensor_specs().items():
+                if name in specs and specs[name] != spec:
+                    raise ValueError(f"tensor {name} is asked for with two shapes: {specs[name].shape} and {spec.shape}")
+                specs[name] = spec
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor], rt) -> None:
+        self.rt = rt
+        for p in self.all_parts():
+            p.bind(tensors, rt)
+
+    def cache_needs(self) -> List:
+        return [self.blocks[pl.layer].mixer.cache_need() for pl in self.plan.order]
+
+    def reads_from(self) -> List:
+        return [pl.reads_cache_of for pl in self.plan.order]
+
+    def prepare_positions(self, n_positions: int) -> None:
+        for p in self.positions.values():
+            p.prepare(n_positions, self.rt)
+
+    def forward(self, step, cache):
+        """Logits (float32, [wanted rows, vocab]) of one step, or None when no row is wanted."""
+        h = self.embedding.forward(step.token_ids)
+        delta = None
+        for i, place in enumerate(self.plan.order):
+            delta = self.blocks[place.layer].forward(h, delta, step, cache.views[i])
+        if step.n_wanted == 0:
+            return None
+        x = self.final_norm.add_norm(h, delta, rows=step.want_rows, write_h=False)
+        return self.head.forward(x)

@@ -1,0 +1,54 @@
+"""Grouped-query attention over the paged cache.
+
+``q, k, v = x Wq, x Wk, x Wv`` without bias, heads split as ``feature j -> head j // head_dim``
+(crates/burn-lm-llama/src/nn/attention/mha.rs:121-140); position encoding of q and k, append to
+the cache (mha.rs:91-95); query head h reads key-value head ``h // (heads / kv_heads)``
+(mha.rs:174-185); ``softmax(q k^T * scale + causal mask) v`` (mha.rs:143-171, scale
+``1/sqrt(head_dim)`` at :159); output projection (mha.rs:118).  The three projections run as
+one product on the stacked weight.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import KVNeed, Mixer, TensorSpec
+
+
+class Attention(Mixer):
+    """params: width, heads, kv_heads, head_dim, scale, window (0 = all keys), position (the
+    position-encoding object, given by the model builder).  names: q, k, v, o."""
+
+    def tensor_specs(self):
+        p = self.params
+        d, hd = p["width"], p["head_dim"]
+        return {self.names["q"]: TensorSpec((p["heads"] * hd, d)),
+                self.names["k"]: TensorSpec((p["kv_heads"] * hd, d)),
+                self.names["v"]: TensorSpec((p["kv_heads"] * hd, d)),
+                self.names["o"]: TensorSpec((d, p["heads"] * hd))}
+
+    def cache_need(self):
+        p = self.params
+        return KVNeed(p["kv_heads"], p["head_dim"], int(p.get("window", 0)))
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        p = self.params
+        self.heads, self.kv_heads, self.head_dim = p["heads"], p["kv_heads"], p["head_dim"]
+        self.scale = float(p["scale"])
+        self.window = int(p.get("window", 0))
+        self.position = p["position"]
+        ws = [tensors[self.names[r]] for r in ("q", "k", "v")]
+        if len({w.dtype for w in ws}) != 1:
+            ws = [w.float() for w in ws]
+        self.w_qkv = torch.cat(ws, dim=0).contiguous()
+        self.w_o = tensors[self.names["o"]].contiguous()
+
+    def forward(self, x, step, view):
+        rt = self.rt
+        nh, nkv, hd = self.heads, self.kv_heads, self.head_dim
+        qkv = rt.linear(x, self.w_qkv)
+        self.position.encode_and_store(qkv, step, view, nh, nkv, hd, store=view.store)
+        out = torch.empty(x.shape[0], nh * hd, dtype=rt.dtype, device=x.device)
+        rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, view.block_table(step),
+                          view.k, view.v, view.page_size, nh, nkv, hd, self.scale, self.window)
+        return rt.linear(out, self.w_o)

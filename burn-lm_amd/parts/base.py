@@ -1,0 +1,107 @@
+"""What every part of a model is to the framework.
+
+A model is put together from parts chosen by name: a *mixer* (attention, or anything else that
+moves information between the tokens of a sequence), a *feed-forward*, a *norm*, a *position
+encoding*, and a *block* that arranges them.  A part gets its sizes and constants as
+parameters, names the checkpoint tensors it wants, and never learns which model it is in.
+
+Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the activation dtype,
+``h`` the float32 residual stream of the same shape):
+
+* ``Part.tensor_specs() -> {checkpoint name: TensorSpec}`` and ``Part.bind(tensors, rt)``.
+* ``Norm.add_norm(h, delta, rows=None, write_h=True) -> x``: ``h += delta`` (if given), then
+  the normalised rows (all rows, or the rows listed in ``rows``).
+* ``Mixer.cache_need() -> KVNeed | StateNeed | None`` and
+  ``Mixer.forward(x, step, view) -> delta``; ``view`` is what the cache holds for this place
+  in the layer order (``KVView``, ``StateView`` or ``None``).
+* ``FeedForward.forward(x, step) -> delta``.
+* ``PositionEncoding.prepare(n_positions, rt)`` and, for encodings that act on queries and keys,
+  ``encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store)``.
+* ``Block.forward(h, delta, step, view) -> delta``: runs its parts; the returned delta has not
+  been added to ``h`` yet (the next norm adds it, in float32).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    shape: Tuple[int, ...]
+    kind: str = "float"  # "float": kept in bfloat16 / float32; "int": kept as int32
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """Choice of a part: its registered kind, its parameters, and the checkpoint tensor name of
+    each of its roles."""
+    kind: str
+    params: dict = field(default_factory=dict)
+    names: Dict[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values per token.  window = 0 keeps every key; window = w keeps the last w."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """State of fixed size per sequence, zeroed when a sequence starts."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    def __init__(self, params: dict, names: Dict[str, str]):
+        self.params = dict(params)
+        self.names = dict(names)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], rt) -> None:
+        self.rt = rt
+
+
+class Norm(Part):
+    def add_norm(self, h, delta, rows=None, write_h=True):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        return None
+
+    def forward(self, x, step, view):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, step):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, n_positions: int, rt) -> None:
+        pass
+
+
+class Block:
+    """Arrangement of a layer's parts."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+
+    def parts(self):
+        return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+
+    def forward(self, h, delta, step, view):
+        raise NotImplementedError

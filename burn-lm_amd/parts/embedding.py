@@ -1,0 +1,40 @@
+"""Token embedding and output head.
+
+``h = table[ids]`` with no scaling (crates/burn-lm-llama/src/nn/transformer.rs:95) into the
+float32 residual stream; ``logits = x W_out^T`` without bias in float32 (transformer.rs:102).
+A tied head uses the embedding table itself: the ``[vocab, width]`` table is the head's
+``[d_out, d_in]`` matrix (the reference leaves tying as a TODO, transformer.rs:82-84)."""
+from __future__ import annotations
+
+import torch
+
+from .base import Part, TensorSpec
+
+
+class Embedding(Part):
+    """params: vocab, width.  names: weight."""
+
+    def tensor_specs(self):
+        return {self.names["weight"]: TensorSpec((self.params["vocab"], self.params["width"]))}
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.table = tensors[self.names["weight"]].contiguous()
+
+    def forward(self, ids):
+        h = torch.empty(ids.shape[0], self.params["width"], dtype=torch.float32, device=ids.device)
+        return self.rt.ops.embed_gather(self.table, ids, h)
+
+
+class LMHead(Part):
+    """params: vocab, width.  names: weight (the embedding's name when tied)."""
+
+    def tensor_specs(self):
+        return {self.names["weight"]: TensorSpec((self.params["vocab"], self.params["width"]))}
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.weight = tensors[self.names["weight"]].contiguous()
+
+    def forward(self, x):
+        return self.rt.linear(x, self.weight, out_dtype=torch.float32)

@@ -1,0 +1,62 @@
+"""Rotary position encoding with optional llama3 frequency scaling.
+
+Angles: ``theta_i = theta^(-2i/head_dim)``, scaled "by parts" as in
+crates/burn-lm-llama/src/nn/pos_encoding.rs:107-138; a token at absolute position p has its
+pairs turned by ``p * theta_i`` (pos_encoding.rs:66-79, vector :165-174).  The table of cosines
+and sines is computed once in float64 on the host and kept in float32; the rotation itself is
+float32 in the kernel, rounded once.
+
+Pairing: the reference pairs adjacent lanes ``(2i, 2i+1)`` and permutes Hugging Face q/k rows
+into that order when it imports them (nn/llama/import.rs:94-127).  ``pairing="half"`` pairs
+``(i, i + head_dim/2)`` instead, which is the same function on un-permuted Hugging Face rows,
+so such checkpoints load without a re-layout.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+from .base import PositionEncoding
+
+PAIRING = {"interleaved": 0, "half": 1}
+
+
+def rope_frequencies(head_dim, theta, scaling=None):
+    """float64 [head_dim/2].  scaling: None or (factor, low_freq_factor, high_freq_factor, old_context)."""
+    i = np.arange(0, head_dim, 2, dtype=np.float64)
+    f = np.power(float(theta), -i / head_dim)
+    if scaling is not None:
+        factor, low, high, old = (float(v) for v in scaling)
+        wavelen = 2.0 * math.pi / f
+        smooth = (old / wavelen - low) / (high - low)
+        mid = (1.0 - smooth) * f / factor + smooth * f
+        f = np.where(wavelen < old / high, f, np.where(wavelen > old / low, f / factor, mid))
+    return f
+
+
+class RotaryEncoding(PositionEncoding):
+    """params: head_dim, theta, scaling (None or 4 numbers), pairing ("half" | "interleaved")."""
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.head_dim = int(self.params["head_dim"])
+        if self.params["pairing"] not in PAIRING:
+            raise ValueError(f"rotary pairing {self.params['pairing']!r} unknown; one of {list(PAIRING)}")
+        self.pairing = PAIRING[self.params["pairing"]]
+        self.freqs = rope_frequencies(self.head_dim, self.params["theta"], self.params.get("scaling"))
+        self.table = None
+
+    def prepare(self, n_positions, rt):
+        ang = np.arange(n_positions, dtype=np.float64)[:, None] * self.freqs[None, :]
+        cs = np.stack([np.cos(ang), np.sin(ang)], axis=-1).astype(np.float32)
+        self.table = torch.from_numpy(cs).to(rt.device)
+        self.n_positions = n_positions
+
+    def encode_and_store(self, qkv, step, view, heads, kv_heads, head_dim, store=True):
+        if step.max_position >= self.n_positions:
+            raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
+        self.rt.ops.rope_kv_write(qkv, step.positions, step.token_seq, view.block_table(step), self.table,
+                                  view.k, view.v, view.page_size, heads, kv_heads, head_dim, self.pairing,
+                                  write_kv=store)

@@ -1,0 +1,34 @@
+"""Dense SwiGLU feed-forward: ``(silu(x W1) * (x W3)) W2`` without bias
+(crates/burn-lm-llama/src/nn/fftn.rs:44-46; W1 = gate, W3 = up, W2 = down,
+nn/llama/import.rs:22-31).  Gate and up run as one product on the stacked weight; silu and the
+product are float32 in the kernel."""
+from __future__ import annotations
+
+import torch
+
+from .base import FeedForward, TensorSpec
+
+
+class SwiGLU(FeedForward):
+    """params: width, inner.  names: gate, up, down."""
+
+    def tensor_specs(self):
+        d, i = self.params["width"], self.params["inner"]
+        return {self.names["gate"]: TensorSpec((i, d)), self.names["up"]: TensorSpec((i, d)),
+                self.names["down"]: TensorSpec((d, i))}
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        self.w_down = tensors[self.names["down"]].contiguous()
+        self.inner = self.params["inner"]
+
+    def forward(self, x, step):
+        rt = self.rt
+        gu = rt.linear(x, self.w_gate_up)
+        act = torch.empty(x.shape[0], self.inner, dtype=rt.dtype, device=x.device)
+        rt.ops.swiglu(gu, act)
+        return rt.linear(act, self.w_down)
