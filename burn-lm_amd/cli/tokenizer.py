@@ -1,0 +1,53 @@
+"""Text <-> token ids for the command line.
+
+``ByteTokenizer``: a token is a byte value, as the reference's test tokenizer
+(crates/burn-lm-llama/src/tokenizer/byte.rs:3-49: bos 0, eos 1, stop ids [2]); it needs a
+vocabulary of at least 256.  Where the reference prints the id list on decode (byte.rs:34-36),
+this one gives the bytes back as text.  A ``tokenizer.json`` in the model folder is used instead
+when the ``tokenizers`` package can read it."""
+from __future__ import annotations
+
+import os
+from typing import List
+
+
+class ByteTokenizer:
+    bos_id, eos_id = 0, 1
+
+    def encode(self, text: str, bos: bool = False, eos: bool = False) -> List[int]:
+        ids = list(text.encode("utf-8"))
+        return ([self.bos_id] if bos else []) + ids + ([self.eos_id] if eos else [])
+
+    def decode(self, tokens) -> str:
+        return bytes(t for t in tokens if 0 <= t < 256).decode("utf-8", errors="replace")
+
+    def stop_ids(self):
+        return [2]
+
+
+class FileTokenizer:
+    def __init__(self, path):
+        from tokenizers import Tokenizer
+        self._tok = Tokenizer.from_file(path)
+
+    def encode(self, text, bos=False, eos=False):
+        return self._tok.encode(text, add_special_tokens=False).ids
+
+    def decode(self, tokens):
+        return self._tok.decode(list(tokens), skip_special_tokens=True)
+
+    def stop_ids(self):
+        return []
+
+
+def for_folder(folder: str, vocab_size: int):
+    path = os.path.join(folder, "tokenizer.json")
+    if os.path.exists(path):
+        try:
+            return FileTokenizer(path)
+        except Exception as e:  # unreadable file: say so and fall back to bytes
+            print(f"warning: {path} could not be read ({e}); using the byte tokenizer")
+    if vocab_size < 256:
+        raise ValueError(f"the byte tokenizer needs a vocabulary of at least 256, the model has {vocab_size}; "
+                         f"pass token ids instead of text")
+    return ByteTokenizer()

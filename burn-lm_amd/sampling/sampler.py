@@ -1,0 +1,66 @@
+"""Choice of the next token from float32 logits.
+
+The reference picks ``argmax`` when the temperature is 0 and otherwise draws from
+``softmax(logits / temperature)`` cut to the top-p nucleus (crates/burn-lm-llama/src/server/
+llama3.rs:454-462, generation/generate.rs:87-91, generation/sampling.rs:9-71), with a seeded
+generator and "seed 0 = a fresh seed for each request".  Here both run as HIP kernels on the
+whole batch; the random number of a draw depends only on (seed, request, index of the token in
+that request), so a request samples the same tokens whatever else is in its batch."""
+from __future__ import annotations
+
+import os
+from typing import List, Sequence
+
+import torch
+
+_MASK = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & _MASK
+    return x ^ (x >> 31)
+
+
+def uniform(seed: int, request: int, index: int) -> float:
+    """Counter-based uniform number in [0, 1) with 24 bits, a pure function of its arguments."""
+    x = _splitmix64(seed & _MASK)
+    x = _splitmix64(x ^ ((request + 1) * 0xD1B54A32D192ED03 & _MASK))
+    x = _splitmix64(x ^ ((index + 1) * 0x8CB92BA72F3D8DD7 & _MASK))
+    return (x >> 40) / float(1 << 24)
+
+
+class Sampler:
+    """temperature == 0: greedy, lowest index wins ties.  temperature > 0: temperature softmax,
+    nucleus of mass top_p (1.0 keeps everything), inverse-CDF draw."""
+
+    def __init__(self, temperature: float = 0.0, top_p: float = 0.9, seed: int = 0, ops=None):
+        if temperature < 0:
+            raise ValueError(f"temperature must be >= 0, got {temperature}")
+        if not 0 < top_p <= 1:
+            raise ValueError(f"top_p must be in (0, 1], got {top_p}")
+        self.temperature, self.top_p = float(temperature), float(top_p)
+        # seed 0 means a fresh random seed (crates/burn-lm-llama/src/server/llama3.rs:454-457)
+        self.seed = int(seed) if seed else int.from_bytes(os.urandom(8), "little")
+        self._ops = ops
+
+    @property
+    def greedy(self):
+        return self.temperature == 0.0
+
+    def uniforms(self, requests: Sequence[int], indices: Sequence[int]) -> List[float]:
+        return [uniform(self.seed, r, i) for r, i in zip(requests, indices)]
+
+    def pick(self, logits: torch.Tensor, requests: Sequence[int], indices: Sequence[int]) -> List[int]:
+        """logits float32 [rows, vocab] on the GPU -> one token per row, as host integers."""
+        ops = self._ops
+        if ops is None:
+            from ..csrc import ops
+            self._ops = ops
+        if self.greedy:
+            out = ops.argmax(logits)
+        else:
+            u = torch.tensor(self.uniforms(requests, indices), dtype=torch.float32).to(logits.device)
+            out = ops.sample(logits, u, self.temperature, self.top_p)
+        return out.tolist()

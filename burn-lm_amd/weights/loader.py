@@ -74,7 +74,7 @@ def load(folder: str, specs: Dict[str, TensorSpec], run_dtype: torch.dtype, devi
     for name, spec in specs.items():
         f = available[name]
         t = f.tensor(name)
-        out[name] = t.to(device=device, dtype=stored_dtype_to_kept(t.dtype, spec.kind, run_dtype)).contiguous()
+        out[name] = t.to(device=device, dtype=stored_dtype_to_kept(t.dtype, spec.kind, run_dtype), copy=True).contiguous()
     for f in {id(f): f for f in available.values()}.values():
         f.close()
     return out

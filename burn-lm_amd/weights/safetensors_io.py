@@ -9,6 +9,7 @@ import json
 import mmap
 import os
 import struct
+import warnings
 from typing import Dict, Iterable, Tuple
 
 import torch
@@ -72,15 +73,15 @@ class SafetensorsFile:
             count *= s
         if count == 0:
             return torch.empty(e["shape"], dtype=DTYPES[e["dtype"]])
-        t = torch.frombuffer(self._mm, dtype=DTYPES[e["dtype"]], count=count, offset=self._data_start + a)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", UserWarning)  # the map is read-only; nothing writes through the view
+            t = torch.frombuffer(self._mm, dtype=DTYPES[e["dtype"]], count=count, offset=self._data_start + a)
         return t.reshape(e["shape"])
 
     def close(self):
-        try:
-            if self._mm is not None:
-                self._mm.close()
-        except BufferError:
-            pass  # a view is still alive; the map goes with it
+        # The map is not closed by hand: tensors made by tensor() may still view it, and each of
+        # them keeps the map alive; it is unmapped when the last of them is gone.
+        self._mm = None
         self._f.close()
 
 

@@ -1,0 +1,166 @@
+"""The cache's bookkeeping (no GPU): no slot or page is lost, held twice or freed twice; pages
+follow each sequence's own length; groups have pools of their own; a refused step changes nothing."""
+import random
+
+import pytest
+import torch
+
+from burn_lm_amd.cache.cache import Cache, CacheError, CacheFull, ContextOverflow, KVView, PagePool, StateView
+from burn_lm_amd.parts.base import KVNeed, StateNeed
+
+
+def make(needs=None, reads=None, max_tokens=256, max_seqs=4, max_context=128, page=16):
+    needs = needs if needs is not None else [KVNeed(2, 8)] * 3
+    reads = reads if reads is not None else [None] * len(needs)
+    return Cache(needs, reads, max_tokens, max_seqs, max_context, page_size=page, dtype=torch.float32, device="cpu")
+
+
+def held_pages(c, gi=0):
+    return [p for t in c.groups[gi].tables.values() for p in t if p >= 0]
+
+
+def check_invariants(c):
+    for gi, g in enumerate(c.groups):
+        held = held_pages(c, gi)
+        assert len(held) == len(set(held)), "a page is held twice"
+        assert set(held) == g.pool._out, "pool and tables disagree"
+        assert sorted(held + g.pool._free) == list(range(g.pool.n_pages)), "a page is lost"
+    assert sorted(c.live_slots + c._free_slots) == list(range(c.max_seqs)), "a slot is lost"
+
+
+def test_pool_refuses_double_free_and_over_take():
+    p = PagePool(4)
+    a = p.take(3)
+    assert len(set(a)) == 3 and p.n_free == 1
+    with pytest.raises(CacheFull):
+        p.take(2)
+    p.give(a[:1])
+    with pytest.raises(CacheError, match="freed twice"):
+        p.give(a[:1])
+    assert p.n_free == 2
+
+
+def test_pages_follow_each_sequences_own_length():
+    c = make()
+    a, b = c.open(), c.open()
+    c.reserve([(a, 5), (b, 33)])
+    c.advance(a, 5); c.advance(b, 33)
+    assert c.length(a) == 5 and c.length(b) == 33
+    assert len(c.groups[0].tables[a]) == 1 and len(c.groups[0].tables[b]) == 3
+    c.reserve([(a, 11), (b, 1)])          # a: 16 tokens, still 1 page; b: 34, still 3
+    c.advance(a, 11); c.advance(b, 1)
+    assert len(c.groups[0].tables[a]) == 1 and len(c.groups[0].tables[b]) == 3
+    c.reserve([(a, 1)]); c.advance(a, 1)  # 17 tokens -> second page
+    assert len(c.groups[0].tables[a]) == 2
+    check_invariants(c)
+    assert c.page_table(0, [b, a], 4) == [c.groups[0].tables[b] + [-1], c.groups[0].tables[a] + [-1, -1]]
+
+
+def test_layers_of_one_need_share_a_group_and_planes_are_their_own():
+    c = make()
+    assert len(c.groups) == 1 and c.groups[0].storage.shape == (3, 2, 16, 2, 16, 8)
+    v0, v2 = c.views[0], c.views[2]
+    assert isinstance(v0, KVView) and v0.k.data_ptr() != v2.k.data_ptr() and v0.k.data_ptr() != v0.v.data_ptr()
+    assert v0.store and v0.k.shape == (16, 2, 16, 8)
+
+
+def test_groups_with_different_needs_have_storage_and_pools_of_their_own():
+    needs = [KVNeed(2, 8), KVNeed(2, 8, window=20), KVNeed(1, 4), KVNeed(2, 8, window=20)]
+    c = make(needs)
+    assert len(c.groups) == 3
+    assert [c.views[i].group_index for i in range(4)] == [0, 1, 2, 1]
+    s = c.open()
+    c.reserve([(s, 70)]); c.advance(s, 70)
+    # all keys: 5 pages held; window 20: next query (position 70) sees keys 51.., so pages 0..2 are gone
+    assert len(held_pages(c, 0)) == 5 and len(held_pages(c, 2)) == 5
+    assert c.groups[1].tables[s][:3] == [-1, -1, -1] and len(held_pages(c, 1)) == 2
+    check_invariants(c)
+    c.close(s)
+    assert c.pages_in_use() == 0
+    check_invariants(c)
+
+
+def test_a_place_may_read_an_earlier_places_cache():
+    c = make([KVNeed(2, 8), KVNeed(2, 8), KVNeed(2, 8)], [None, None, 0])
+    assert c.groups[0].storage.shape[0] == 2
+    assert c.views[2].k.data_ptr() == c.views[0].k.data_ptr() and not c.views[2].store
+    with pytest.raises(CacheError, match="earlier place"):
+        make([KVNeed(2, 8), KVNeed(2, 8)], [1, None])
+    with pytest.raises(CacheError, match="differ"):
+        make([KVNeed(2, 8), KVNeed(1, 8)], [None, 0])
+
+
+def test_fixed_size_state_is_per_slot_and_zeroed_when_a_slot_opens():
+    c = make([KVNeed(2, 8), StateNeed((3, 5)), None])
+    assert isinstance(c.views[1], StateView) and c.views[1].tensor.shape == (4, 3, 5) and c.views[2] is None
+    s = c.open()
+    c.views[1].tensor[s] += 7
+    c.close(s)
+    s2 = c.open()
+    assert s2 == s and float(c.views[1].tensor[s2].abs().sum()) == 0.0
+
+
+def test_slots_are_given_back_and_used_again():
+    c = make(max_seqs=2)
+    a, b = c.open(), c.open()
+    with pytest.raises(CacheFull, match="slots"):
+        c.open()
+    c.close(a)
+    with pytest.raises(CacheError, match="closed twice"):
+        c.close(a)
+    assert c.open() == a
+    with pytest.raises(CacheError, match="not open"):
+        c.length(99)
+
+
+def test_a_refused_step_changes_nothing():
+    c = make(max_tokens=64, max_context=48)   # 4 pages of 16
+    a, b = c.open(), c.open()
+    c.reserve([(a, 20)]); c.advance(a, 20)    # 2 pages
+    before = (list(c.groups[0].pool._free), {k: list(v) for k, v in c.groups[0].tables.items()})
+    with pytest.raises(CacheFull, match="pages"):
+        c.reserve([(a, 1), (b, 40)])          # would need 3 more
+    with pytest.raises(ContextOverflow) as e:
+        c.reserve([(a, 29)])
+    assert (e.value.actual, e.value.maximum) == (49, 48)
+    with pytest.raises(CacheError, match="twice"):
+        c.reserve([(b, 1), (b, 1)])
+    with pytest.raises(CacheError, match="at least one"):
+        c.reserve([(b, 0)])
+    assert before == (list(c.groups[0].pool._free), {k: list(v) for k, v in c.groups[0].tables.items()})
+    assert c.length(a) == 20 and c.length(b) == 0 and c.room(a) == 28
+    check_invariants(c)
+
+
+def test_random_traffic_keeps_the_books():
+    rnd = random.Random(0)
+    c = make([KVNeed(2, 8), KVNeed(2, 8, window=24)], max_tokens=320, max_seqs=5, max_context=96)
+    live = {}
+    for _ in range(600):
+        r = rnd.random()
+        if r < 0.25 and c.free_slots:
+            live[c.open()] = 0
+        elif r < 0.4 and live:
+            s = rnd.choice(list(live))
+            c.close(s); del live[s]
+        elif live:
+            group = rnd.sample(list(live), rnd.randint(1, len(live)))
+            growth = [(s, rnd.choice([1, 1, 1, 7, 30])) for s in group]
+            try:
+                c.reserve(growth)
+            except (CacheFull, ContextOverflow):
+                check_invariants(c)
+                continue
+            for s, n in growth:
+                c.advance(s, n); live[s] += n
+        check_invariants(c)
+        for s, n in live.items():
+            assert c.length(s) == n
+            t = c.groups[0].tables[s]
+            assert len(t) == (n + 15) // 16 and all(p >= 0 for p in t)
+            tw = c.groups[1].tables[s]
+            first_key = max(0, n - 24 + 1)
+            assert all((p >= 0) == (i >= first_key // 16) for i, p in enumerate(tw))
+    for s in list(live):
+        c.close(s)
+    assert c.pages_in_use() == 0 and c.free_slots == 5

@@ -1,0 +1,116 @@
+"""Configuration and registry (no GPU)."""
+import json
+
+import pytest
+
+import burn_lm_amd  # noqa: F401
+from burn_lm_amd import registry
+from burn_lm_amd.config.llama import ConfigError, LlamaConfig, RopeScaling
+from burn_lm_amd.config.presets import preset, presets
+from helpers import TINY_A, TINY_B
+
+
+def test_reads_every_size_from_its_keys():
+    c = LlamaConfig.from_dict(TINY_B)
+    assert (c.hidden_size, c.intermediate_size, c.num_hidden_layers) == (144, 384, 3)
+    assert (c.num_attention_heads, c.num_key_value_heads, c.head_dim) == (6, 1, 24)
+    assert (c.vocab_size, c.max_position_embeddings) == (384, 384)
+    assert c.rms_norm_eps == 1e-6 and c.rope_theta == 500000.0 and c.tie_word_embeddings is False
+    assert c.rope_scaling == RopeScaling(8.0, 1.0, 4.0, 32)
+
+
+def test_defaults_are_the_references():
+    # crates/burn-lm-llama/src/nn/llama/base.rs:54-62,254; nn/attention/mha.rs:191; nn/pos_encoding.rs:91-101
+    d = {k: v for k, v in TINY_A.items() if k not in ("num_key_value_heads", "rms_norm_eps", "rope_theta",
+                                                      "tie_word_embeddings")}
+    c = LlamaConfig.from_dict(d)
+    assert c.num_key_value_heads == c.num_attention_heads == 4
+    assert c.head_dim == 16 and c.rms_norm_eps == 1e-5 and c.rope_theta == 10000.0
+    assert c.tie_word_embeddings is False and c.rope_scaling is None
+    c = LlamaConfig.from_dict({**TINY_A, "rope_scaling": {"rope_type": "llama3"}})
+    assert c.rope_scaling == RopeScaling(8.0, 1.0, 4.0, 8192)
+
+
+@pytest.mark.parametrize("key", ["hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
+                                 "vocab_size", "max_position_embeddings"])
+def test_missing_size_names_the_key(key):
+    d = dict(TINY_A)
+    del d[key]
+    with pytest.raises(ConfigError, match=key):
+        LlamaConfig.from_dict(d)
+
+
+@pytest.mark.parametrize("patch,word", [
+    ({"num_key_value_heads": 3}, "num_key_value_heads"),
+    ({"head_dim": 15}, "head_dim"),
+    ({"hidden_size": "64"}, "hidden_size"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "yarn"),
+    ({"attention_bias": True}, "attention_bias"),
+    ({"mlp_bias": True}, "mlp_bias"),
+    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"eos_token_id": 999}, "999"),
+    ({"rms_norm_eps": 0}, "rms_norm_eps"),
+    ({"hidden_size": 66, "head_dim": None}, "head_dim"),
+])
+def test_bad_values_are_refused_with_their_key(patch, word):
+    with pytest.raises(ConfigError, match=word):
+        LlamaConfig.from_dict({**TINY_A, **patch})
+
+
+def test_eos_may_be_one_id_or_a_list_and_round_trips():
+    c = LlamaConfig.from_dict({**TINY_A, "eos_token_id": [1, 2]})
+    assert c.eos_token_ids == (1, 2)
+    assert LlamaConfig.from_dict({**TINY_A, "eos_token_id": 7}).eos_token_ids == (7,)
+    assert LlamaConfig.from_dict(c.to_dict()) == c
+    assert LlamaConfig.from_dict(LlamaConfig.from_dict(TINY_B).to_dict()) == LlamaConfig.from_dict(TINY_B)
+
+
+def test_folder_errors(tmp_path):
+    with pytest.raises(ConfigError, match="config.json"):
+        LlamaConfig.from_folder(str(tmp_path))
+    (tmp_path / "config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="JSON"):
+        LlamaConfig.from_folder(str(tmp_path))
+    (tmp_path / "config.json").write_text(json.dumps(TINY_A))
+    assert LlamaConfig.from_folder(str(tmp_path)).hidden_size == 64
+
+
+def test_registry_maps_names_to_the_architecture():
+    a = registry.architecture_of(TINY_A)
+    assert a is registry.architecture("llama") is registry.architecture("LlamaForCausalLM")
+    with pytest.raises(registry.RegistryError, match="LlamaForCausalLM"):
+        registry.architecture("MambaForCausalLM")
+    with pytest.raises(registry.RegistryError, match="names no architecture"):
+        registry.architecture_of({"hidden_size": 1})
+    assert registry.architecture_of({"architectures": ["Nope"], "model_type": "llama"}) is a
+    with pytest.raises(registry.RegistryError, match="attention"):
+        registry.part("mixer", "nope")
+
+
+def test_plan_follows_the_configuration():
+    a = registry.architecture("llama")
+    cfg = a.read_config(TINY_B)
+    plan = a.plan(cfg, None)
+    assert len(plan.layers) == 3 and [p.layer for p in plan.order] == [0, 1, 2]
+    m = plan.layers[1].mixer
+    assert m.kind == "attention" and m.params["heads"] == 6 and m.params["kv_heads"] == 1 and m.params["head_dim"] == 24
+    assert abs(m.params["scale"] - 24 ** -0.5) < 1e-15
+    assert plan.layers[0].mixer_norm.params["eps"] == 1e-6
+    assert plan.positions["rope"].params["pairing"] == "half"
+    assert plan.head.names["weight"] == "lm_head.weight"
+    tied = a.plan(a.read_config(TINY_A), None)
+    assert tied.head.names["weight"] == tied.embedding.names["weight"]
+    meta = a.plan(cfg, {"tok_embeddings.weight"})
+    assert meta.positions["rope"].params["pairing"] == "interleaved"
+    assert meta.layers[0].feed_forward.names["gate"] == "layers.0.feed_forward.w1.weight"
+
+
+def test_presets_are_valid_configurations():
+    for name in presets():
+        c = LlamaConfig.from_dict(preset(name))
+        assert c.num_hidden_layers > 0
+    c = LlamaConfig.from_dict(preset("llama3.2-1b"))
+    # crates/burn-lm-llama/src/nn/llama/base.rs:103-113
+    assert (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads,
+            c.intermediate_size, c.vocab_size) == (2048, 16, 32, 8, 8192, 128256)
+    assert c.rope_scaling.factor == 32.0 and c.rope_theta == 500000.0

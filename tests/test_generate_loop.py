@@ -1,0 +1,168 @@
+"""The generation loop's decisions, on a stand-in engine without a GPU: batches of unequal
+prompts, stop tokens, sequences that end earlier, one batch after another on the same slots."""
+import pytest
+import torch
+
+from burn_lm_amd.cache.cache import Cache
+from burn_lm_amd.engine.generate import generate, plan_batches
+from burn_lm_amd.parts.base import KVNeed
+from burn_lm_amd.sampling.sampler import Sampler, uniform
+
+
+class ToyEngine:
+    """Next token = (sum of the sequence so far) mod vocab, told through one-hot logits.  Uses the
+    real cache bookkeeping, and records every step it is asked to run."""
+
+    def __init__(self, vocab=50, max_tokens=256, max_seqs=4, max_context=64, page=16):
+        self.vocab_size, self.max_context = vocab, max_context
+        self.cache = Cache([KVNeed(1, 2)], [None], max_tokens, max_seqs, max_context, page, torch.float32, "cpu")
+        self.sums, self.steps, self.opened = {}, [], []
+
+    def open(self):
+        s = self.cache.open()
+        self.sums[s] = 0
+        self.opened.append(s)
+        return s
+
+    def close(self, s):
+        self.cache.close(s)
+        del self.sums[s]
+
+    def length(self, s):
+        return self.cache.length(s)
+
+    def step(self, entries):
+        self.cache.reserve([(s, len(t)) for s, t, _ in entries])
+        self.steps.append([(s, len(t)) for s, t, _ in entries])
+        rows = []
+        for s, toks, want in entries:
+            assert want == [len(toks) - 1]
+            self.sums[s] += sum(toks)
+            self.cache.advance(s, len(toks))
+            row = torch.zeros(self.vocab_size)
+            row[self.sums[s] % self.vocab_size] = 1.0
+            rows.append(row)
+        return torch.stack(rows)
+
+
+class HostArgmax:
+    def pick(self, logits, requests, indices):
+        self.last = (list(requests), list(indices))
+        return [int(i) for i in logits.argmax(1)]
+
+
+def expected(prompt, n, vocab=50, stop=()):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = sum(toks) % vocab
+        out.append(t); toks.append(t)
+        if t in stop:
+            break
+    return out
+
+
+def test_unequal_prompts_one_prefill_then_one_token_each():
+    eng = ToyEngine()
+    prompts = [[1, 2, 3], [4] * 9, [7]]
+    res, stats = generate(eng, prompts, HostArgmax(), sample_len=5, batch_size=4)
+    assert [r.tokens for r in res] == [expected(p, 5) for p in prompts]
+    assert all(r.finish_reason == "length" for r in res)
+    assert [n for _, n in eng.steps[0]] == [3, 9, 1]                 # all prompts in one step
+    assert all(n == 1 for st in eng.steps[1:] for _, n in st)        # then one token each
+    assert len(eng.steps) == 5                                       # the 5th token needs no further step
+    assert stats.prompt_tokens == 13 and stats.generated_tokens == 15 and stats.decode_tokens == 12
+    assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 4
+
+
+def test_stop_token_ends_a_sequence_and_the_others_go_on():
+    eng = ToyEngine()
+    prompts = [[1, 2, 3], [5, 5], [9]]
+    free = [expected(p, 8) for p in prompts]
+    stop = free[1][2]                       # third token of request 1
+    want = [expected(p, 8, stop=(stop,)) for p in prompts]
+    res, _ = generate(eng, prompts, HostArgmax(), sample_len=8, stop_ids=[stop], batch_size=4)
+    assert [r.tokens for r in res] == want
+    assert res[1].finish_reason == "stop" and res[1].tokens[-1] == stop and len(res[1].tokens) == 3
+    sizes = [len(s) for s in eng.steps]
+    assert sizes[0] == 3 and min(sizes) < 3, "the ended sequence must leave the batch"
+    # no step runs for a sequence after its stop token
+    slot1 = eng.opened[1]
+    assert sum(1 for st in eng.steps for s, _ in st if s == slot1) == 3
+
+
+def test_batches_run_one_after_another_on_the_same_slots():
+    eng = ToyEngine(max_seqs=2)
+    prompts = [[i + 1] * (i + 1) for i in range(5)]
+    res, _ = generate(eng, prompts, HostArgmax(), sample_len=3, batch_size=2)
+    assert [r.tokens for r in res] == [expected(p, 3) for p in prompts]
+    assert len(eng.opened) == 5 and set(eng.opened) == {0, 1}, "slots are used again"
+    assert [len(s) for s in eng.steps if s[0][1] > 1 or len(s) == 2][:1] == [2]
+    assert eng.cache.pages_in_use() == 0
+
+
+def test_batches_are_cut_to_what_the_cache_holds():
+    # 4 pages of 16: each request may reach 10 + 20 = 30 tokens = 2 pages -> two per batch
+    assert plan_batches([10, 10, 10], 20, batch_size=8, max_context=64, page_size=16, n_pages=4, n_slots=8) == [[0, 1], [2]]
+    assert plan_batches([10] * 5, 20, batch_size=2, max_context=64, page_size=16, n_pages=64, n_slots=8) == [[0, 1], [2, 3], [4]]
+    assert plan_batches([10] * 3, 20, batch_size=8, max_context=64, page_size=16, n_pages=64, n_slots=1) == [[0], [1], [2]]
+    # the context bounds what a request can come to hold
+    assert plan_batches([10, 10], 1000, batch_size=8, max_context=32, page_size=16, n_pages=4, n_slots=8) == [[0, 1]]
+    eng = ToyEngine(max_tokens=64)
+    res, _ = generate(eng, [[1] * 10, [2] * 10, [3] * 10], HostArgmax(), sample_len=20, batch_size=8)
+    assert [len(r.tokens) for r in res] == [20, 20, 20]
+    assert [len(s) for s in eng.steps if s[0][1] == 10] == [2, 1]
+
+
+def test_context_end_and_refused_prompts():
+    eng = ToyEngine(max_context=12, max_tokens=64)
+    res, _ = generate(eng, [[1] * 10, [2] * 13, [], [3]], HostArgmax(), sample_len=50, batch_size=4)
+    # 10 prompt tokens + 2 fed-back tokens fill the context; the token predicted from the full context is the last
+    assert res[0].finish_reason == "length" and len(res[0].tokens) == 3
+    assert res[0].tokens == expected([1] * 10, 3)
+    assert res[1].finish_reason == "error" and "exceeds maximum context window (12" in res[1].error
+    assert res[2].finish_reason == "error" and not res[2].tokens
+    assert res[3].finish_reason == "length" and len(res[3].tokens) == 12
+    assert eng.cache.pages_in_use() == 0
+
+
+def test_sample_len_zero_and_callback_order():
+    eng = ToyEngine()
+    res, _ = generate(eng, [[1, 2]], HostArgmax(), sample_len=0)
+    assert res[0].tokens == [] and res[0].finish_reason == "length" and not eng.steps
+    seen = []
+    res, _ = generate(eng, [[1, 2], [3]], HostArgmax(), sample_len=3, on_token=lambda r, t: seen.append((r, t)))
+    assert [t for r, t in seen if r == 0] == res[0].tokens and [t for r, t in seen if r == 1] == res[1].tokens
+    assert [r for r, _ in seen[:2]] == [0, 1]
+
+
+def test_slots_are_returned_when_a_step_fails():
+    eng = ToyEngine()
+
+    def boom(entries):
+        raise RuntimeError("kernel failed")
+    eng.step = boom
+    with pytest.raises(RuntimeError, match="kernel failed"):
+        generate(eng, [[1], [2]], HostArgmax(), sample_len=2)
+    assert eng.cache.free_slots == 4
+
+
+def test_sampler_numbers_depend_on_seed_request_and_index_only():
+    a = Sampler(0.8, 0.9, seed=5)
+    assert a.uniforms([3, 4], [0, 0]) == [uniform(5, 3, 0), uniform(5, 4, 0)]
+    assert a.uniforms([3], [7]) == a.uniforms([9, 3], [1, 7])[1:]       # batch mates do not matter
+    assert uniform(5, 3, 0) != uniform(6, 3, 0) != uniform(5, 3, 1)
+    us = [uniform(1, r, i) for r in range(40) for i in range(50)]
+    assert all(0.0 <= u < 1.0 for u in us) and abs(sum(us) / len(us) - 0.5) < 0.02
+    assert Sampler(0.0).greedy and not a.greedy
+    assert Sampler(0.7, seed=0).seed != Sampler(0.7, seed=0).seed       # 0 = a fresh seed each time
+    with pytest.raises(ValueError):
+        Sampler(-1.0)
+    with pytest.raises(ValueError):
+        Sampler(1.0, top_p=0.0)
+
+
+def test_sampler_is_told_request_and_token_index():
+    eng = ToyEngine()
+    s = HostArgmax()
+    generate(eng, [[1], [20], [3]], s, sample_len=4, stop_ids=[expected([20], 4)[1]], batch_size=4)
+    assert s.last == ([0, 2], [3, 3])
