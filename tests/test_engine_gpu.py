@@ -1,0 +1,192 @@
+"""The engine on the GPU against the plain implementation: long decoding, the first tokens of a
+sequence, greedy generation through the entry point, faults that random weights would hide."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from helpers import TINIES, TINY_A, TINY_B, TOL, make_folder, random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {k: make_folder(tmp_path_factory.mktemp("m" + k), cfg, seed) for k, (cfg, seed) in TINIES.items()}
+
+
+def load(folder, dtype, **kw):
+    from burn_lm_amd.engine.loading import load_engine
+    kw.setdefault("max_tokens", 1024)
+    return load_engine(folder, dtype=dtype, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding(folders, name, dtype):
+    """7 prompt tokens, then 300 tokens one by one: five pages, every page edge crossed in decode."""
+    cfg, seed = TINIES[name]
+    toks = random_tokens(seed + 50, cfg["vocab_size"], 307)
+    want = P.transformer_forward([toks], P.load_model_folder(folders[name]))[0]
+    eng = load(folders[name], dtype)
+    s = eng.open()
+    got = [eng.step([(s, toks[:7], list(range(7)))])]
+    for t in toks[7:]:
+        got.append(eng.step([(s, [t], [0])]))
+    got = torch.cat(got).double().cpu().numpy()
+    errs = [rel_err(got[p], want[p]) for p in range(len(toks))]
+    bad = [p for p, e in enumerate(errs) if e > TOL[dtype]]
+    assert not bad, f"first wrong position {bad[0]} (page edge every 64), error {errs[bad[0]]:.3g}"
+    assert eng.length(s) == 307
+    eng.close(s)
+    assert eng.cache.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(folders, dtype):
+    """Prompts of one and two tokens (one token = no mask at all in the reference,
+    crates/burn-lm-llama/src/nn/transformer.rs:169-171), then their first decoded tokens."""
+    cfg, seed = TINIES["B"]
+    plain = P.load_model_folder(folders["B"])
+    eng = load(folders["B"], dtype)
+    toks = random_tokens(3, cfg["vocab_size"], 6)
+    want = P.transformer_forward([toks], plain)[0]
+    a, b = eng.open(), eng.open()
+    got = eng.step([(a, toks[:1], [0]), (b, toks[:2], [0, 1])]).double().cpu().numpy()
+    for row, p in zip(got, [0, 0, 1]):
+        assert rel_err(row, want[p]) <= TOL[dtype]
+    got = eng.step([(a, [toks[1]], [0]), (b, [toks[2]], [0])]).double().cpu().numpy()
+    assert rel_err(got[0], want[1]) <= TOL[dtype] and rel_err(got[1], want[2]) <= TOL[dtype]
+    got = eng.step([(b, toks[3:6], [2]), (a, [toks[2]], [0])]).double().cpu().numpy()   # a chunk and a single token
+    assert rel_err(got[0], want[5]) <= TOL[dtype] and rel_err(got[1], want[2]) <= TOL[dtype]
+
+
+def test_a_far_key_among_hundreds_is_found(folders, tmp_path):
+    """One early key is made to stand out for the last query (its embedding row scaled up), so an
+    attention that loses keys far back, or a page of the table, changes the logits visibly."""
+    from burn_lm_amd.weights import safetensors_io as st
+    cfg, seed = TINIES["A"]
+    f = st.open_folder(folders["A"])
+    tensors = {n: f[n].tensor(n).clone() for n in f}
+    emb = tensors["model.embed_tokens.weight"].float()
+    emb[255] *= 12.0
+    tensors["model.embed_tokens.weight"] = emb.bfloat16()
+    folder = str(tmp_path / "m")
+    os.makedirs(folder)
+    st.write_file(os.path.join(folder, "model.safetensors"), tensors.items())
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    plain = P.load_model_folder(folder)
+    toks = [t % 255 for t in random_tokens(11, 255, 400)]
+    toks[3] = 255
+    want = P.transformer_forward([toks], plain)[0]
+    without = list(toks)
+    without[3] = 7
+    moved = P.transformer_forward([without], plain)[0]
+    assert rel_err(moved[399], want[399]) > 0.05, "the test's own premise: the far key matters"
+    for dtype in ("float32", "bfloat16"):
+        eng = load(folder, dtype)
+        s = eng.open()
+        eng.step([(s, toks[:330], [])])
+        got = torch.cat([eng.step([(s, [t], [0])]) for t in toks[330:]]).double().cpu().numpy()
+        for i, p in enumerate(range(330, 400)):
+            assert rel_err(got[i], want[p]) <= TOL[dtype], f"{dtype}: position {p}"
+
+
+def test_logits_do_not_depend_on_batch_mates_or_on_where_in_the_cache(folders):
+    cfg, seed = TINIES["A"]
+    eng = load(folders["A"], "float32", max_tokens=2048)
+    toks = random_tokens(21, cfg["vocab_size"], 90)
+    s = eng.open()
+    alone = eng.step([(s, toks, list(range(90)))]).cpu()
+    eng.close(s)
+    # fill and free pages so that the same request lands on other pages and another slot
+    junk = [eng.open() for _ in range(3)]
+    eng.step([(j, random_tokens(30 + i, cfg["vocab_size"], 70 + 40 * i), []) for i, j in enumerate(junk)])
+    eng.cache.views[0].k.fill_(float("nan"))   # what is left in pages must never be read
+    eng.cache.views[1].v.fill_(float("nan"))
+    for j in junk[:2]:
+        eng.close(j)
+    s = eng.open()
+    other = eng.open()
+    assert eng.cache.groups[0].tables[s] == []
+    both = eng.step([(other, random_tokens(40, cfg["vocab_size"], 33), [32]), (s, toks, list(range(90)))]).cpu()
+    assert torch.isfinite(both).all()
+    assert rel_err(both[1:].double().numpy(), alone.double().numpy()) <= 2e-6
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(folders, name):
+    """Unequal prompts, more requests than batch places, a stop token that ends one early: the
+    32-bit engine gives the plain implementation's tokens."""
+    from burn_lm_amd.server import InferenceServer
+    cfg, seed = TINIES[name]
+    plain = P.load_model_folder(folders[name])
+    lens = [5, 11, 17, 1, 33, 7, 20]
+    prompts = [random_tokens(60 + i, cfg["vocab_size"], n) for i, n in enumerate(lens)]
+    free = [P.greedy_generate(plain, p, 10) for p in prompts]
+    stop = free[1][3]
+    want = [P.greedy_generate(plain, p, 10, stop_ids=(stop,)) for p in prompts]
+    server = InferenceServer(folders[name], dtype="float32", batch_size=3)
+    server.config.update(max_seq_len=128, sample_len=10, temperature=0.0)
+    results, stats = server.generate(prompts, stop_ids=[stop])
+    assert [r.tokens for r in results] == want
+    assert results[1].finish_reason == "stop" and len(results[1].tokens) == 4
+    assert stats.generated_tokens == sum(len(w) for w in want) and stats.prompt_tokens == sum(lens)
+    assert "Tokens Per Second" in stats.display_stats() and "##### BurnLM Stats" in stats.display_stats()
+    # statelessness: the same request after others gives the same tokens (generate.rs:163-226)
+    again, _ = server.generate([prompts[4]], stop_ids=[stop])
+    assert again[0].tokens == want[4]
+    assert server.engine.cache.pages_in_use() == 0
+
+
+def test_temperature_sampling_is_seeded_and_independent_of_batch_mates(folders):
+    from burn_lm_amd.server import InferenceServer
+    cfg, seed = TINIES["B"]
+    prompts = [random_tokens(80 + i, cfg["vocab_size"], n) for i, n in enumerate([1, 7, 20, 33])]
+    server = InferenceServer(folders["B"], dtype="float32", batch_size=4)
+    server.config.update(max_seq_len=128, sample_len=12, temperature=0.8, top_p=0.9, seed=11)
+    a, _ = server.generate(prompts, stop_ids=[])
+    b, _ = server.generate(prompts, stop_ids=[])
+    assert [r.tokens for r in a] == [r.tokens for r in b]
+    solo, _ = server.generate(prompts[:1], stop_ids=[])
+    assert solo[0].tokens == a[0].tokens
+    c, _ = server.generate(prompts, stop_ids=[], seed=12)
+    assert [r.tokens for r in c] != [r.tokens for r in a]
+    greedy, _ = server.generate(prompts, stop_ids=[], temperature=0.0)
+    assert [r.tokens for r in greedy] != [r.tokens for r in a]
+
+
+def test_a_refused_step_leaves_the_engine_as_it_was(folders):
+    from burn_lm_amd.cache.cache import CacheFull, ContextOverflow
+    from burn_lm_amd.engine.engine import StepError
+    cfg, _ = TINIES["A"]
+    eng = load(folders["A"], "float32", max_tokens=128)
+    s = eng.open()
+    eng.step([(s, [1, 2, 3], [])])
+    for bad in ([(s, [], [])], [(s, [256], [0])], [(s, [1], [1])], [(s, [-1], [])], []):
+        with pytest.raises(StepError):
+            eng.step(bad)
+    with pytest.raises(CacheFull):
+        eng.step([(s, [1] * 200, [])])
+    t = eng.open()
+    with pytest.raises(CacheFull):
+        eng.step([(s, [1], [0]), (t, [1] * 100, [])])
+    assert eng.length(s) == 3 and eng.length(t) == 0
+    small = load(folders["A"], "float32", max_tokens=1024, max_context=64)
+    u = small.open()
+    with pytest.raises(ContextOverflow):
+        small.step([(u, [1] * 65, [])])
+
+
+def test_command_line_runs_a_prompt(folders, capsys):
+    from burn_lm_amd.cli.main import main
+    main(["-d", "f32", "run", folders["A"], "--sample-len", "6", "--tokens", "5,17,3"])
+    out = capsys.readouterr().out
+    plain = P.load_model_folder(folders["A"])
+    assert ",".join(str(t) for t in P.greedy_generate(plain, [5, 17, 3], 6)) in out
+    assert "##### BurnLM Stats" in out and "Tokens Per Second" in out
+    main(["run", folders["A"], "--sample-len", "4", "--temperature", "0.7", "--seed", "3", "--no-stats", "hi"])
+    assert "BurnLM Stats" not in capsys.readouterr().out

@@ -1,0 +1,312 @@
+"""Each HIP kernel alone against a plain float32 / float64 torch expression of the same
+operation, at sizes other than the engine's (widths and vocabularies that are no powers of two,
+odd head counts, several head sizes), in float32 and bfloat16."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# one rounding to the storage type, relative to the largest value of the row
+EPS = {"float32": 2e-6, "bfloat16": 6e-3}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from burn_lm_amd.csrc import ops
+    ops.library()
+    return ops
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def close(got, want, tol):
+    got, want = got.double().cpu(), want.double().cpu()
+    err = float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+    assert err <= tol, f"relative error {err:.3g} > {tol}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed_gather(ops, dtype):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(1000, 200, generator=g).to(DT[dtype])
+    ids = torch.tensor([0, 999, 5, 5, 123], dtype=torch.int32)
+    h = torch.empty(5, 200, dtype=torch.float32, device="cuda")
+    ops.embed_gather(dev(table), dev(ids), h)
+    assert torch.equal(h.cpu(), table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("gamma_dtype", ["float32", "bfloat16"])
+def test_add_rmsnorm(ops, dtype, gamma_dtype):
+    g = torch.Generator().manual_seed(1)
+    T, D, eps = 7, 200, 1e-3
+    h = torch.randn(T, D, generator=g) * 0.02          # small, so eps matters
+    delta = (torch.randn(T, D, generator=g) * 0.02).to(DT[dtype])
+    gamma = (1 + 0.3 * torch.randn(D, generator=g)).to(DT[gamma_dtype])
+
+    def ref(v):
+        v = v.double()
+        return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * gamma.double()
+
+    hd = dev(h.clone())
+    out = torch.empty(T, D, dtype=DT[dtype], device="cuda")
+    ops.add_rmsnorm(hd, dev(delta), dev(gamma), eps, out)
+    summed = h + delta.float()
+    assert torch.equal(hd.cpu(), summed), "the residual sum is float32 and written back"
+    close(out, ref(summed), EPS[dtype])
+    # eps inside the root: leaving it out changes these small rows a lot
+    assert float((ref(summed) - summed.double() / summed.double().pow(2).mean(-1, keepdim=True).sqrt() * gamma.double()).abs().max()) > 0.05
+    # no delta; rows gathered; h untouched
+    hd = dev(h.clone())
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    out = torch.empty(3, D, dtype=DT[dtype], device="cuda")
+    ops.add_rmsnorm(hd, None, dev(gamma), eps, out, rows=dev(rows))
+    close(out, ref(h[rows.long()]), EPS[dtype])
+    ops.add_rmsnorm(hd, dev(delta), dev(gamma), eps, out, rows=dev(rows), write_h=False)
+    close(out, ref(summed[rows.long()]), EPS[dtype])
+    assert torch.equal(hd.cpu(), h)
+
+
+def _rope_ref(x, pos, freqs, pairing):
+    """x [T, heads, hd] double; complex multiplication on the pairs."""
+    ang = pos.double()[:, None] * freqs[None, :]
+    rot = torch.polar(torch.ones_like(ang), ang)[:, None, :]
+    hd = x.shape[-1]
+    if pairing == "interleaved":
+        z = torch.complex(x[..., 0::2], x[..., 1::2]) * rot
+        out = torch.empty_like(x)
+        out[..., 0::2], out[..., 1::2] = z.real, z.imag
+    else:
+        z = torch.complex(x[..., : hd // 2], x[..., hd // 2:]) * rot
+        out = torch.cat([z.real, z.imag], -1)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("pairing", ["interleaved", "half"])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 3, 32), (5, 5, 24), (8, 1, 80)])
+def test_rope_kv_write(ops, dtype, pairing, nh, nkv, hd):
+    from burn_lm_amd.parts.rope import PAIRING, rope_frequencies
+    g = torch.Generator().manual_seed(2)
+    page, n_pages = 16, 12
+    # two sequences: 5 new tokens at positions 30..34 (crossing a page edge), 1 new token at position 3
+    positions = torch.tensor([30, 31, 32, 33, 34, 3], dtype=torch.int32)
+    token_seq = torch.tensor([0, 0, 0, 0, 0, 1], dtype=torch.int32)
+    table = torch.tensor([[7, 2, 9, -1], [4, -1, -1, -1]], dtype=torch.int32)
+    T = 6
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=g).to(DT[dtype])
+    freqs = torch.from_numpy(rope_frequencies(hd, 500000.0, (8, 1, 4, 32)))
+    ang = torch.arange(64).double()[:, None] * freqs[None, :]
+    cs = torch.stack([ang.cos(), ang.sin()], -1).float()
+    k = torch.full((n_pages, nkv, page, hd), 99.0).to(DT[dtype])
+    v = torch.full((n_pages, nkv, page, hd), 99.0).to(DT[dtype])
+    qd, kd, vd = dev(qkv.clone()), dev(k), dev(v)
+    ops.rope_kv_write(qd, dev(positions), dev(token_seq), dev(table), dev(cs), kd, vd, page, nh, nkv, hd,
+                      PAIRING[pairing])
+    x = qkv.double()
+    q_ref = _rope_ref(x[:, : nh * hd].reshape(T, nh, hd), positions, freqs, pairing)
+    k_ref = _rope_ref(x[:, nh * hd: (nh + nkv) * hd].reshape(T, nkv, hd), positions, freqs, pairing)
+    v_ref = x[:, (nh + nkv) * hd:].reshape(T, nkv, hd)
+    close(qd[:, : nh * hd].reshape(T, nh, hd), q_ref, EPS[dtype])
+    assert torch.equal(qd[:, nh * hd:].cpu(), qkv[:, nh * hd:]), "k and v in the activation buffer stay as they were"
+    kc, vc = kd.cpu().double(), vd.cpu().double()
+    written = torch.zeros(n_pages, page, dtype=torch.bool)
+    for t in range(T):
+        p = int(positions[t])
+        pg = int(table[int(token_seq[t]), p // page])
+        written[pg, p % page] = True
+        close(kc[pg, :, p % page], k_ref[t], EPS[dtype])
+        assert torch.equal(vc[pg, :, p % page], v_ref[t].to(DT[dtype]).double())
+    untouched = ~written[:, None, :, None].expand(n_pages, nkv, page, hd)
+    assert bool((kc[untouched] == 99).all()) and bool((vc[untouched] == 99).all()), "nothing else is written"
+    # a place that reads another's cache rotates q only
+    qd2, kd2 = dev(qkv.clone()), dev(k)
+    ops.rope_kv_write(qd2, dev(positions), dev(token_seq), dev(table), dev(cs), kd2, dev(v), page, nh, nkv, hd,
+                      PAIRING[pairing], write_kv=False)
+    assert torch.equal(qd2.cpu(), qd.cpu()) and bool((kd2.cpu() == 99).all())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu(ops, dtype):
+    g = torch.Generator().manual_seed(3)
+    T, I = 5, 300
+    gu = (torch.randn(T, 2 * I, generator=g) * 3).to(DT[dtype])
+    out = torch.empty(T, I, dtype=DT[dtype], device="cuda")
+    ops.swiglu(dev(gu), out)
+    x = gu.double()
+    close(out, torch.nn.functional.silu(x[:, :I]) * x[:, I:], EPS[dtype])
+
+
+def _attn_ref(q, keys, values, pos, scale, window, n_rep):
+    """q [nh, hd]; keys/values [S, nkv, hd] of the whole sequence; query at position pos."""
+    lo = max(0, pos - window + 1) if window else 0
+    k = keys[lo: pos + 1].double().repeat_interleave(n_rep, 1)
+    v = values[lo: pos + 1].double().repeat_interleave(n_rep, 1)
+    s = torch.einsum("hd,shd->hs", q.double(), k) * scale
+    return torch.einsum("hs,shd->hd", torch.softmax(s, -1), v)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (6, 1, 24, 0), (5, 5, 64, 0), (8, 2, 128, 0),
+                                               (3, 1, 200, 0), (4, 2, 32, 37)])
+def test_attn_paged(ops, dtype, nh, nkv, hd, window):
+    g = torch.Generator().manual_seed(4)
+    page, n_pages = 16, 40
+    lens = [150, 1, 70]          # cached length of three sequences after this step
+    new = [4, 1, 70]             # the last `new` positions are this step's queries
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = 10
+    table = torch.full((3, width), -1, dtype=torch.int32)
+    keys, values = [], []
+    kc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    vc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    for b, L in enumerate(lens):
+        kb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
+        vb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
+        if L > 100:   # a far key that the last queries must find: scale it up
+            kb[5] *= 6.0
+        keys.append(kb); values.append(vb)
+        for i in range((L + page - 1) // page):
+            pg = perm.pop()
+            table[b, i] = pg
+            n = min(page, L - i * page)
+            kc[pg, :, :n] = kb[i * page: i * page + n].transpose(0, 1).float()
+            vc[pg, :, :n] = vb[i * page: i * page + n].transpose(0, 1).float()
+    positions, token_seq = [], []
+    for b, (L, n) in enumerate(zip(lens, new)):
+        positions += list(range(L - n, L)); token_seq += [b] * n
+    positions.append(0); token_seq.append(-1)     # a padding token
+    T = len(positions)
+    stride = (nh + 2 * nkv) * hd
+    qkv = torch.randn(T, stride, generator=g).to(DT[dtype])
+    out = torch.full((T, nh * hd), 7.0, dtype=DT[dtype], device="cuda")
+    scale = 1.0 / math.sqrt(hd)
+    ops.attn_paged(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
+                   dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc.to(DT[dtype])),
+                   dev(vc.to(DT[dtype])), page, nh, nkv, hd, scale, window)
+    got = out.cpu().double().reshape(T, nh, hd)
+    assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
+    for t in range(T - 1):
+        b = token_seq[t]
+        want = _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[b], values[b], positions[t], scale, window, nh // nkv)
+        close(got[t], want, EPS[dtype] * 2)
+    assert bool((got[T - 1] == 0).all()), "a padding token gives zeros"
+
+
+def test_attn_paged_refuses_what_it_cannot_do(ops):
+    from burn_lm_amd.csrc.ops import KernelError
+    z = torch.zeros(1, 3 * 258, device="cuda")
+    i = torch.zeros(1, dtype=torch.int32, device="cuda")
+    c = torch.zeros(1, 1, 16, 258, device="cuda")
+    with pytest.raises(KernelError, match="head_dim 258"):
+        ops.attn_paged(z, 3 * 258, torch.zeros(1, 258, device="cuda"), i, i, i.view(1, 1), c, c, 16, 1, 1, 258, 1.0)
+    with pytest.raises(KernelError, match="GPU only"):
+        ops.swiglu(torch.zeros(1, 4), torch.zeros(1, 2))
+
+
+@pytest.mark.parametrize("a,w,c", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
+                                   ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
+def test_gemm_tiled(ops, a, w, c):
+    g = torch.Generator().manual_seed(5)
+    M, N, K = 70, 130, 50
+    A = torch.randn(M, K, generator=g).to(DT[a])
+    W = torch.randn(N, K, generator=g).to(DT[w])
+    out = torch.empty(M, N, dtype=DT[c], device="cuda")
+    ops.gemm_tiled(dev(A), dev(W), out)
+    close(out, A.double() @ W.double().T, EPS[c] * 2)
+    # rows taken from a wider buffer (unit stride along rows is all that is asked)
+    wide = torch.randn(M, K + 14, generator=g).to(DT[a])
+    ops.gemm_tiled(dev(wide)[:, :K], dev(W), out)
+    close(out, wide[:, :K].double() @ W.double().T, EPS[c] * 2)
+
+
+def test_float32_product_is_true_32_bit(ops):
+    """Operands with 21 significant bits: a matrix mode that rounds its inputs to bfloat16 or to a
+    19-bit format returns 16, true float32 returns 16 * (1 + 2^-20); every partial sum is exact."""
+    K = 16
+    A = torch.full((3, K), 1.0 + 2.0 ** -20)
+    W = torch.ones(65, K)
+    for fn in (ops.gemm_tiled, ops.gemv_skinny):
+        out = torch.empty(3, 65, device="cuda")
+        fn(dev(A), dev(W), out)
+        assert torch.equal(out.cpu(), torch.full((3, 65), 16.0 + 2.0 ** -16))
+
+
+@pytest.mark.parametrize("dtype,out_dtype", [("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")])
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8])
+def test_gemv_skinny(ops, dtype, out_dtype, M):
+    from burn_lm_amd.csrc.ops import KernelError
+    g = torch.Generator().manual_seed(6)
+    N, K = 1001, 264
+    A = torch.randn(M, K, generator=g).to(DT[dtype])
+    W = torch.randn(N, K, generator=g).to(DT[dtype])
+    out = torch.empty(M, N, dtype=DT[out_dtype], device="cuda")
+    ops.gemv_skinny(dev(A), dev(W), out)
+    close(out, A.double() @ W.double().T, EPS[out_dtype] * 2)
+    with pytest.raises(KernelError, match="multiples of 8"):
+        ops.gemv_skinny(dev(A)[:, :260].contiguous(), dev(W)[:, :260].contiguous(), out)
+    with pytest.raises(KernelError, match="1..8"):
+        ops.gemv_skinny(dev(torch.zeros(9, K).to(DT[dtype])), dev(W), torch.empty(9, N, dtype=DT[out_dtype], device="cuda"))
+
+
+def test_argmax_first_maximum_wins(ops):
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(6, 1000, generator=g)
+    x[1, 17] = x[1, 900] = 50.0
+    x[2, 999] = 60.0
+    x[3, 0] = 60.0
+    x[4] = 0.0
+    wide = torch.randn(6, 1200, generator=g)
+    wide[:, :1000] = x
+    wide[:, 1000:] = 100.0                       # beyond the vocabulary: must not be looked at
+    got = ops.argmax(dev(wide)[:, :1000]).cpu().tolist()
+    assert got == [int(x[0].argmax()), 17, 999, 0, 0, int(x[5].argmax())]
+
+
+def test_sample_follows_the_temperature_distribution(ops):
+    g = torch.Generator().manual_seed(8)
+    V, R, T = 37, 40000, 0.7
+    logits = torch.randn(V, generator=g) * 2
+    probs = torch.softmax(logits.double() / T, 0)
+    u = torch.rand(R, generator=g)
+    got = ops.sample(dev(logits.expand(R, V).contiguous()), dev(u), T, 1.0).cpu()
+    counts = torch.bincount(got.long(), minlength=V).double()
+    chi2 = float(((counts - R * probs) ** 2 / (R * probs)).sum())
+    assert chi2 < 80, f"chi-square {chi2:.1f} with 36 degrees of freedom"
+    # inverse CDF in index order: the same u gives the same token, and u = 0 gives the first token with mass
+    cdf = torch.cumsum(probs, 0)
+    want = torch.searchsorted(cdf, u.double().clamp(max=float(cdf[-1]) - 1e-12), right=True)
+    assert float((want == got).double().mean()) > 0.999
+    # very low temperature is argmax
+    cold = ops.sample(dev(logits.expand(50, V).contiguous()), dev(u[:50]), 1e-3, 1.0).cpu()
+    assert bool((cold == int(logits.argmax())).all())
+
+
+def test_sample_top_p_keeps_the_nucleus_only(ops):
+    import plain_llama as P
+    g = torch.Generator().manual_seed(9)
+    V, R, T, p = 200, 20000, 1.3, 0.6
+    logits = torch.randn(V, generator=g) * 1.5
+    probs = P.temperature_softmax(logits.numpy(), T)
+    kept = P.top_p_keep(probs, p)                 # crates/burn-lm-llama/src/generation/sampling.rs:50-63
+    u = torch.rand(R, generator=g)
+    got = ops.sample(dev(logits.expand(R, V).contiguous()), dev(u), T, p).cpu()
+    seen = set(got.tolist())
+    assert seen <= set(kept), f"tokens outside the nucleus were drawn: {sorted(seen - set(kept))}"
+    assert seen == set(kept) or len(kept) - len(seen) <= 1
+    sub = torch.tensor([probs[i] for i in kept]).double()
+    sub = sub / sub.sum()
+    counts = torch.tensor([(got == i).sum() for i in kept]).double()
+    chi2 = float(((counts - R * sub) ** 2 / (R * sub)).sum())
+    assert chi2 < 3 * len(kept) + 30
+    # rows are independent: different logits per row, large vocabulary that is no power of two
+    big = torch.randn(5, 50257, generator=g)
+    big[3, 40000] = 30.0
+    out = ops.sample(dev(big), dev(torch.full((5,), 0.5)), 0.8, 0.9).cpu()
+    assert int(out[3]) == 40000 and all(0 <= int(t) < 50257 for t in out)

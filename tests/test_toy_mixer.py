@@ -1,0 +1,171 @@
+"""A mixer with state of its own, and the architecture that uses it, are defined here, in the
+test: registered, built from a model folder through the registry, and stepped, without a change
+to the framework's files.  The toy is no model of anyone's: layer 0 is the framework's attention,
+layer 1 a running decayed sum ``s_t = a * s_{t-1} + x_t W`` kept as fixed-size state per sequence,
+and the order runs layer 0 twice, the second time reading the first run's keys and values."""
+import json
+import math
+import os
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+TOY = dict(architectures=["ToyDecayLM"], width=48, inner=80, heads=4, kv_heads=2, head_dim=12, vocab=97,
+           eps=1e-5, theta=10000.0, decay=0.8, max_positions=256)
+
+
+def register_toy():
+    from burn_lm_amd import registry
+    from burn_lm_amd.models.plan import LayerPlan, ModelPlan, Place
+    from burn_lm_amd.parts.base import Mixer, PartSpec, StateNeed, TensorSpec
+
+    class DecayMixer(Mixer):
+        """params: width, decay.  names: w.  State: one float32 vector per sequence."""
+
+        def tensor_specs(self):
+            return {self.names["w"]: TensorSpec((self.params["width"],) * 2)}
+
+        def cache_need(self):
+            return StateNeed((self.params["width"],), torch.float32)
+
+        def bind(self, tensors, rt):
+            self.rt, self.w, self.a = rt, tensors[self.names["w"]], float(self.params["decay"])
+
+        def forward(self, x, step, view):
+            u = self.rt.linear(x, self.w).float()
+            out = torch.empty_like(u)
+            row = 0
+            for slot, n in zip(step.host_slots, step.host_new):   # tokens of a sequence run in order
+                s = view.tensor[slot]
+                for t in range(row, row + n):
+                    s = self.a * s + u[t]
+                    out[t] = s
+                view.tensor[slot] = s
+                row += n
+            return out.to(self.rt.dtype)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        d: dict
+
+        def __getattr__(self, k):
+            return self.d[k]
+
+    def plan(cfg, names=None):
+        D = cfg.width
+        norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=cfg.eps), dict(weight=n))
+        ffn = lambda i: PartSpec("swiglu", dict(width=D, inner=cfg.inner),
+                                 dict(gate=f"l{i}.gate", up=f"l{i}.up", down=f"l{i}.down"))
+        attn = PartSpec("attention", dict(width=D, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim,
+                                          scale=1 / math.sqrt(cfg.head_dim)),
+                        dict(q="l0.q", k="l0.k", v="l0.v", o="l0.o"))
+        layers = [LayerPlan("pre_norm", attn, ffn(0), norm("l0.n1"), norm("l0.n2"), position="rope"),
+                  LayerPlan("pre_norm", PartSpec("toy_decay", dict(width=D, decay=cfg.decay), dict(w="l1.w")),
+                            ffn(1), norm("l1.n1"), norm("l1.n2"))]
+        return ModelPlan(vocab_size=cfg.vocab, width=D, max_positions=cfg.max_positions,
+                         embedding=PartSpec("table", dict(vocab=cfg.vocab, width=D), dict(weight="emb")),
+                         layers=layers, order=[Place(0), Place(1), Place(0, reads_cache_of=0)],
+                         final_norm=norm("norm"), head=PartSpec("linear", dict(vocab=cfg.vocab, width=D), dict(weight="emb")),
+                         positions={"rope": PartSpec("rope", dict(head_dim=cfg.head_dim, theta=cfg.theta,
+                                                                  pairing="interleaved", scaling=None))})
+
+    registry.register_part("mixer", "toy_decay", DecayMixer)
+    registry.register_architecture(registry.Architecture("ToyDecayLM", read_config=lambda d: ToyConfig(d), plan=plan))
+
+
+def toy_weights(seed=3):
+    c = TOY
+    g = torch.Generator().manual_seed(seed)
+    m = lambda *s: (torch.randn(*s, generator=g) * 0.15).bfloat16()
+    n = lambda: (1 + 0.1 * torch.randn(c["width"], generator=g)).bfloat16()
+    D, I, hd = c["width"], c["inner"], c["head_dim"]
+    t = {"emb": m(c["vocab"], D), "norm": n(), "l1.w": m(D, D),
+         "l0.q": m(c["heads"] * hd, D), "l0.k": m(c["kv_heads"] * hd, D), "l0.v": m(c["kv_heads"] * hd, D),
+         "l0.o": m(D, c["heads"] * hd)}
+    for i in (0, 1):
+        t.update({f"l{i}.gate": m(I, D), f"l{i}.up": m(I, D), f"l{i}.down": m(D, I), f"l{i}.n1": n(), f"l{i}.n2": n()})
+    return t
+
+
+def toy_plain(tokens, t):
+    """The toy's whole-sequence forward in float64, from the plain parts."""
+    c = TOY
+    w = {k: v.double().numpy() for k, v in t.items()}
+    freqs = P.rope_base_frequencies(c["head_dim"], c["theta"])
+    ffn = lambda i, x: P.swiglu_feed_forward(x, w[f"l{i}.gate"], w[f"l{i}.up"], w[f"l{i}.down"])
+    attn = lambda x: P.attention_layer(x, w["l0.q"], w["l0.k"], w["l0.v"], w["l0.o"], c["heads"], c["kv_heads"],
+                                       c["head_dim"], freqs)
+    h = w["emb"][np.asarray(tokens)][None]
+    # place 0: attention layer
+    x0 = P.rms_norm(h, w["l0.n1"], c["eps"])
+    h = h + attn(x0)
+    h = h + ffn(0, P.rms_norm(h, w["l0.n2"], c["eps"]))
+    # place 1: decayed running sum
+    u = P.rms_norm(h, w["l1.n1"], c["eps"]) @ w["l1.w"].T
+    s, outs = np.zeros(c["width"]), []
+    for i in range(u.shape[1]):
+        s = c["decay"] * s + u[0, i]
+        outs.append(s)
+    h = h + np.stack(outs)[None]
+    h = h + ffn(1, P.rms_norm(h, w["l1.n2"], c["eps"]))
+    # place 2: layer 0 again, queries from the new stream, keys and values of place 0
+    x2 = P.rms_norm(h, w["l0.n1"], c["eps"])
+    b, T = 1, x2.shape[1]
+    q = (x2 @ w["l0.q"].T).reshape(b, T, c["heads"], c["head_dim"]).swapaxes(1, 2)
+    k = (x0 @ w["l0.k"].T).reshape(b, T, c["kv_heads"], c["head_dim"]).swapaxes(1, 2)
+    v = (x0 @ w["l0.v"].T).reshape(b, T, c["kv_heads"], c["head_dim"]).swapaxes(1, 2)
+    pos = np.arange(T)
+    o = P.scaled_attention(P.rope_interleaved(q, pos, freqs), P.rope_interleaved(k, pos, freqs), v, P.hidden_mask(T, T))
+    h = h + o.swapaxes(1, 2).reshape(b, T, -1) @ w["l0.o"].T
+    h = h + ffn(0, P.rms_norm(h, w["l0.n2"], c["eps"]))
+    return (P.rms_norm(h, w["norm"], c["eps"]) @ w["emb"].T)[0]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype, tol):
+    from burn_lm_amd.cache.cache import KVView, StateView
+    from burn_lm_amd.engine.loading import load_engine
+    from burn_lm_amd.weights import safetensors_io as st
+    register_toy()
+    t = toy_weights()
+    json.dump(TOY, open(tmp_path / "config.json", "w"))
+    st.write_file(str(tmp_path / "model.safetensors"), t.items())
+    eng = load_engine(str(tmp_path), dtype=dtype, max_tokens=512, max_seqs=4)
+    views = eng.cache.views
+    assert isinstance(views[0], KVView) and isinstance(views[1], StateView) and isinstance(views[2], KVView)
+    assert views[2].k.data_ptr() == views[0].k.data_ptr() and not views[2].store
+    assert eng.cache.groups[0].storage.shape[0] == 1 and views[1].tensor.shape == (4, 48)
+    rng = np.random.default_rng(0)
+    reqs = [[int(x) for x in rng.integers(0, 97, n)] for n in (70, 9, 33)]
+    want = [toy_plain(r, t) for r in reqs]
+    err = lambda got, w: float(np.abs(got.double().cpu().numpy() - w).max() / np.abs(w).max())
+    # whole, each alone
+    for r, w in zip(reqs, want):
+        s = eng.open()
+        assert err(eng.step([(s, r, list(range(len(r))))]), w) <= tol
+        eng.close(s)
+    # unequal batch: prompts in one step, then one token each; the shortest ends first; state and
+    # slots are used again by a second batch
+    for _ in range(2):
+        slots = [eng.open() for _ in reqs]
+        cut = [len(r) - 8 for r in reqs]
+        got = eng.step([(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cut)])
+        o = 0
+        for r, c, w in zip(reqs, cut, want):
+            assert err(got[o:o + c], w[:c]) <= tol
+            o += c
+        for k in range(8):
+            live = [i for i in range(3) if not (i == 1 and k >= 4)]
+            got = eng.step([(slots[i], [reqs[i][cut[i] + k]], [0]) for i in live])
+            for row, i in enumerate(live):
+                assert err(got[row], want[i][cut[i] + k]) <= tol, f"request {i}, decode step {k}"
+            if k == 3:
+                eng.close(slots[1])
+        eng.close(slots[0]); eng.close(slots[2])
+    assert eng.cache.pages_in_use() == 0
