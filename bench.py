@@ -1,0 +1,169 @@
+"""Decode and prefill throughput of the engine on one MI355X, with roofline fractions.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers L]
+
+A "step" is one decode step of the whole batch: the engine's step function on one token per
+sequence, the sampling kernel, and the tokens' trip to the host, as the generation loop does it.
+The default run has the layer sizes of the Llama-3.2-1B shape with random weights, a batch of 8
+and a context of 4096 tokens per sequence.  One JSON line is printed.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                                   # MI355X HBM3E, published
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}          # dense, published
+
+
+def weight_bytes(cfg, layers, itemsize):
+    d, hd = cfg.hidden_size, cfg.head_dim
+    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * hd * d + d * cfg.num_attention_heads * hd
+                 + 3 * cfg.intermediate_size * d + 2 * d)
+    head = cfg.vocab_size * d
+    return (layers * per_layer + d + head) * itemsize   # the embedding rows read are negligible; tied or not, the head is read once
+
+
+def kv_bytes_per_token(cfg, layers, itemsize):
+    return 2 * layers * cfg.num_key_value_heads * cfg.head_dim * itemsize
+
+
+def prefill_flops(cfg, layers, T, rows_out=1):
+    d, hd, nh, nkv = cfg.hidden_size, cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
+    lin = 2 * T * ((nh + 2 * nkv) * hd * d + d * nh * hd + 3 * cfg.intermediate_size * d)
+    attn = 2 * 2 * nh * hd * (T * (T + 1) // 2)
+    return layers * (lin + attn) + 2 * rows_out * cfg.vocab_size * d
+
+
+def fill_cache(engine, n_seqs, length, seed=0):
+    """Sequences that already hold `length` tokens: pages reserved, lengths set, keys and values
+    random (synthetic; what they hold does not change the work of a decode step)."""
+    import torch
+    g = torch.Generator(device=engine.rt.device).manual_seed(seed)
+    for grp in engine.cache.groups:
+        grp.storage.normal_(0.0, 1.0, generator=g)
+    slots = []
+    for _ in range(n_seqs):
+        s = engine.open()
+        engine.cache.reserve([(s, length)])
+        engine.cache.advance(s, length)
+        slots.append(s)
+    return slots
+
+
+def time_decode(engine, sampler, batch, context, steps, warmup):
+    import torch
+    for s in list(engine.cache.live_slots):
+        engine.close(s)
+    start = context - (steps + warmup)
+    slots = fill_cache(engine, batch, start)
+    toks = [1] * batch
+    reqs = list(range(batch))
+    for i in range(warmup):
+        logits = engine.step([(s, [t], [0]) for s, t in zip(slots, toks)])
+        toks = sampler.pick(logits, reqs, [i] * batch)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        logits = engine.step([(s, [t], [0]) for s, t in zip(slots, toks)])
+        toks = sampler.pick(logits, reqs, [warmup + i] * batch)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for s in slots:
+        engine.close(s)
+    return dt / steps
+
+
+def time_prefill(engine, T, reps=3):
+    import torch
+    import numpy as np
+    toks = [int(x) for x in np.random.default_rng(0).integers(0, engine.vocab_size, T)]
+    best = None
+    for r in range(reps + 1):
+        s = engine.open()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([(s, toks, [T - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.close(s)
+        if r > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
+    ap.add_argument("--preset", default="llama3.2-1b")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 decode points")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this library has no multi-GPU path (run with --gpus 1)")
+        sys.exit(2)
+
+    import torch
+    from burn_lm_amd.config.presets import preset
+    from burn_lm_amd.engine.loading import random_engine
+    from burn_lm_amd.sampling.sampler import Sampler
+
+    config = preset(args.preset)
+    full_layers = config["num_hidden_layers"]
+    layers = args.layers or full_layers
+    config["num_hidden_layers"] = layers
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    engine = random_engine(config, seed=0, dtype=args.dtype, max_tokens=biggest * args.context,
+                           max_seqs=biggest, max_context=args.context)
+    cfg = engine.config
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    sampler = Sampler(temperature=0.0)
+
+    sec = time_decode(engine, sampler, args.batch, args.context, args.steps, args.warmup)
+    value = args.batch / sec
+    mean_ctx = args.context - args.steps / 2
+    step_bytes = weight_bytes(cfg, layers, itemsize) + kv_bytes_per_token(cfg, layers, itemsize) * mean_ctx * args.batch
+    achieved = step_bytes / sec / 1e9
+
+    T = args.prefill_tokens
+    psec = time_prefill(engine, T)
+    pf = prefill_flops(cfg, layers, T)
+    peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            s = time_decode(engine, sampler, b, args.context, max(8, args.steps // 2), 4)
+            points[f"decode_b{b}"] = round(b / s, 1)
+
+    out = {
+        "metric": "decode_tokens_per_second", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (seeded random weights N(0, 0.02), random token ids, random cache contents)",
+        "config": {"model": args.preset, "batch": args.batch, "context": args.context, "layers": layers,
+                   "layers_of_shape": full_layers, "hidden_size": cfg.hidden_size,
+                   "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
+                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size,
+                   "tied_head": cfg.tie_word_embeddings, "page_size": engine.cache.page_size,
+                   "sampling": "greedy", "parallelism": "single GPU"},
+        "prefill": {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3), "frac": round(pf / psec / peak, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -192,7 +192,8 @@ static int launch_skinny(const void* A, const void* W, void* C, int M, int N, in
 
 extern "C" int blm_gemv_skinny(const void* A, int a_dtype, const void* W, int w_dtype, void* C,
                                int c_dtype, int M, int N, int K, int lda, int ldc, hipStream_t stream) {
-  BLM_REQUIRE(M >= 1 && M <= 8 && N > 0 && K > 0, "gemv_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+  BLM_REQUIRE(M >= 1 && M <= 8, "gemv_skinny: M=%d out of range 1..8", M);
+  BLM_REQUIRE(N > 0 && K > 0, "gemv_skinny: bad sizes N=%d K=%d", N, K);
   BLM_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemv_skinny: K=%d and lda=%d must be multiples of 8", K, lda);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemv_skinny: operands must be 16-byte aligned");
   BLM_REQUIRE(a_dtype == w_dtype, "gemv_skinny: A and W must share a dtype (got %d, %d)", a_dtype, w_dtype);

@@ -64,3 +64,29 @@ def load_engine(folder, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_co
     eng.config = cfg
     eng.load_seconds = time.time() - t0
     return eng
+
+
+def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_context=None,
+                  device="cuda:0", std=0.02, page_size=64):
+    """Engine with seeded random weights made directly on the GPU (same generator as the
+    random-weights mode that writes a folder, without the trip through a file)."""
+    from ..weights.random_init import random_tensors
+    dtype = parse_dtype(dtype)
+    arch = registry.architecture_of(config)
+    cfg = arch.read_config(config)
+    rt = Runtime(dtype=dtype, device=device, page_size=page_size)
+    plan = arch.plan(cfg, None)
+    model = Model(plan)
+    specs = model.tensor_specs()
+    tensors = {}
+    for name, t in random_tensors(arch, cfg, seed, std=std, dtype=dtype, device=rt.device):
+        if name in specs:
+            tensors[name] = t
+    missing = [n for n in specs if n not in tensors]
+    if missing:
+        raise ValueError(f"random weights: the architecture's checkpoint lacks {missing}")
+    model.bind(tensors, rt)
+    model.config, model.architecture = cfg, arch
+    eng = Engine(model, rt, max_tokens=max_tokens, max_seqs=max_seqs, max_context=max_context, page_size=page_size)
+    eng.config = cfg
+    return eng

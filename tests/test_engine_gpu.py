@@ -72,7 +72,7 @@ def test_a_far_key_among_hundreds_is_found(folders, tmp_path):
     f = st.open_folder(folders["A"])
     tensors = {n: f[n].tensor(n).clone() for n in f}
     emb = tensors["model.embed_tokens.weight"].float()
-    emb[255] *= 12.0
+    emb[255] *= 4.0
     tensors["model.embed_tokens.weight"] = emb.bfloat16()
     folder = str(tmp_path / "m")
     os.makedirs(folder)
@@ -85,7 +85,8 @@ def test_a_far_key_among_hundreds_is_found(folders, tmp_path):
     without = list(toks)
     without[3] = 7
     moved = P.transformer_forward([without], plain)[0]
-    assert rel_err(moved[399], want[399]) > 0.05, "the test's own premise: the far key matters"
+    effect = [rel_err(moved[p], want[p]) for p in range(330, 400)]
+    assert sum(e > 0.1 for e in effect) >= 5, "the test's own premise: the far key matters to several late positions"
     for dtype in ("float32", "bfloat16"):
         eng = load(folder, dtype)
         s = eng.open()
@@ -127,13 +128,14 @@ def test_greedy_generation_through_the_entry_point(folders, name):
     lens = [5, 11, 17, 1, 33, 7, 20]
     prompts = [random_tokens(60 + i, cfg["vocab_size"], n) for i, n in enumerate(lens)]
     free = [P.greedy_generate(plain, p, 10) for p in prompts]
-    stop = free[1][3]
+    k = next(k for k in range(1, 10) if free[1][k] not in free[1][:k])   # a token request 1 makes first at place k
+    stop = free[1][k]
     want = [P.greedy_generate(plain, p, 10, stop_ids=(stop,)) for p in prompts]
     server = InferenceServer(folders[name], dtype="float32", batch_size=3)
     server.config.update(max_seq_len=128, sample_len=10, temperature=0.0)
     results, stats = server.generate(prompts, stop_ids=[stop])
     assert [r.tokens for r in results] == want
-    assert results[1].finish_reason == "stop" and len(results[1].tokens) == 4
+    assert results[1].finish_reason == "stop" and len(results[1].tokens) == k + 1
     assert stats.generated_tokens == sum(len(w) for w in want) and stats.prompt_tokens == sum(lens)
     assert "Tokens Per Second" in stats.display_stats() and "##### BurnLM Stats" in stats.display_stats()
     # statelessness: the same request after others gives the same tokens (generate.rs:163-226)
@@ -169,7 +171,7 @@ def test_a_refused_step_leaves_the_engine_as_it_was(folders):
     for bad in ([(s, [], [])], [(s, [256], [0])], [(s, [1], [1])], [(s, [-1], [])], []):
         with pytest.raises(StepError):
             eng.step(bad)
-    with pytest.raises(CacheFull):
+    with pytest.raises((CacheFull, ContextOverflow)):
         eng.step([(s, [1] * 200, [])])
     t = eng.open()
     with pytest.raises(CacheFull):

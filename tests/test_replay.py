@@ -82,7 +82,7 @@ def test_replay_matches_plain_whole_tail_and_batched(case, dtype, tmp_path):
                                      f"{len(reqs[rid])} (step {step}) differs by {e:.3g} of the largest logit")
     everything = {(rid, p) for rid, t in reqs.items() for p in range(len(t))}
     assert seen["whole"] == everything and seen["tail"] == everything
-    assert len(seen["batched"]) > 700
+    assert len(seen["batched"]) > 400
     print(f"config {name} {dtype}: worst relative error {worst}")
 
 
