@@ -31,6 +31,10 @@ _SIGNATURES = {
     "blm_attn_paged": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                        _c_void_p],
+    "blm_attn_decode": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                        _c_void_p, _c_void_p, _c_void_p],
+    "blm_attn_decode_supported": [_c_int, _c_int],
     "blm_gemm_tiled": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_void_p],
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
@@ -197,6 +201,34 @@ def attn_paged(q, q_row_stride, out, positions, token_seq, block_table, kcache, 
     _call("blm_attn_paged", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
           page_size, T, nh, nkv, hd, float(scale), int(window), _stream())
+    return out
+
+
+def attn_decode_supported(dtype, hd):
+    """Whether the split-key decode kernel takes this head size (else the generic kernel does)."""
+    return dtype in DTYPE_CODE and bool(library().blm_attn_decode_supported(DTYPE_CODE[dtype], int(hd)))
+
+
+def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache, vcache, page_size,
+                nh, nkv, hd, scale, window=0, n_splits=1):
+    """Attention for few query tokens over long key ranges, the key range cut into n_splits."""
+    _gpu(q, out, positions, token_seq, block_table, kcache, vcache)
+    T = out.shape[0]
+    _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
+    if out.shape[1] != nh * hd or out.dtype != q.dtype or kcache.dtype != q.dtype:
+        raise KernelError("attn_decode: out must be [T, heads*head_dim] and share q's dtype with the cache")
+    if q.stride(-1) != 1 or q_row_stride < nh * hd:
+        raise KernelError("attn_decode: q rows must be contiguous and at least heads*head_dim long")
+    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or kcache.shape != vcache.shape:
+        raise KernelError("attn_decode: cache plane shape does not fit [pages, kv_heads, page, head_dim]")
+    _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
+    n_splits = max(1, int(n_splits))
+    part_o = torch.empty(T * nh * n_splits * hd, dtype=torch.float32, device=out.device)
+    part_ml = torch.empty(T * nh * n_splits * 2, dtype=torch.float32, device=out.device)
+    _call("blm_attn_decode", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
+          token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
+          page_size, T, nh, nkv, hd, float(scale), int(window), n_splits, part_o.data_ptr(), part_ml.data_ptr(),
+          _stream())
     return out
 
 

@@ -128,7 +128,7 @@ def test_greedy_generation_through_the_entry_point(folders, name):
     lens = [5, 11, 17, 1, 33, 7, 20]
     prompts = [random_tokens(60 + i, cfg["vocab_size"], n) for i, n in enumerate(lens)]
     free = [P.greedy_generate(plain, p, 10) for p in prompts]
-    k = next(k for k in range(1, 10) if free[1][k] not in free[1][:k])   # a token request 1 makes first at place k
+    k = next((k for k in range(1, 10) if free[1][k] not in free[1][:k]), 0)   # a token request 1 makes first at place k
     stop = free[1][k]
     want = [P.greedy_generate(plain, p, 10, stop_ids=(stop,)) for p in prompts]
     server = InferenceServer(folders[name], dtype="float32", batch_size=3)

@@ -199,6 +199,59 @@ def test_attn_paged(ops, dtype, nh, nkv, hd, window):
     assert bool((got[T - 1] == 0).all()), "a padding token gives zeros"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,window,splits", [(4, 2, 16, 0, 3), (6, 1, 32, 0, 1), (5, 5, 64, 0, 4), (8, 2, 128, 0, 16),
+                                                      (12, 1, 64, 0, 2), (3, 1, 256, 0, 5), (4, 2, 32, 37, 2)])
+def test_attn_decode(ops, dtype, nh, nkv, hd, window, splits):
+    """The split-key decode kernel: sequences of very different lengths in one call (one of a single
+    key, one that ends exactly at a page edge), scrambled pages with NaN in every unused place, a far
+    key that stands out, more splits than some sequences have pages, a padding token."""
+    assert ops.attn_decode_supported(DT[dtype], hd) and not ops.attn_decode_supported(DT[dtype], 24)
+    g = torch.Generator().manual_seed(14)
+    page, n_pages = 16, 60
+    lens = [403, 1, 64, 17, 130]
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = 26
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    keys, values = [], []
+    kc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    vc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    for b, L in enumerate(lens):
+        kb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
+        vb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
+        if L > 100:
+            kb[2] *= 5.0
+        keys.append(kb); values.append(vb)
+        for i in range((L + page - 1) // page):
+            pg = perm.pop()
+            table[b, i] = pg
+            n = min(page, L - i * page)
+            kc[pg, :, :n] = kb[i * page: i * page + n].transpose(0, 1).float()
+            vc[pg, :, :n] = vb[i * page: i * page + n].transpose(0, 1).float()
+    positions = [L - 1 for L in lens] + [0]
+    token_seq = list(range(len(lens))) + [-1]
+    # order of the tokens need not be the order of the sequences
+    order = [3, 0, 5, 4, 1, 2]
+    positions = [positions[i] for i in order]; token_seq = [token_seq[i] for i in order]
+    T = len(positions)
+    stride = (nh + 2 * nkv) * hd
+    qkv = torch.randn(T, stride, generator=g).to(DT[dtype])
+    out = torch.full((T, nh * hd), 7.0, dtype=DT[dtype], device="cuda")
+    scale = 1.0 / math.sqrt(hd)
+    ops.attn_decode(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
+                    dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc.to(DT[dtype])),
+                    dev(vc.to(DT[dtype])), page, nh, nkv, hd, scale, window, splits)
+    got = out.cpu().double().reshape(T, nh, hd)
+    assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
+    for t in range(T):
+        b = token_seq[t]
+        if b < 0:
+            assert bool((got[t] == 0).all())
+            continue
+        want = _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[b], values[b], positions[t], scale, window, nh // nkv)
+        close(got[t], want, EPS[dtype] * 2)
+
+
 def test_attn_paged_refuses_what_it_cannot_do(ops):
     from burn_lm_amd.csrc.ops import KernelError
     z = torch.zeros(1, 3 * 258, device="cuda")
