@@ -39,6 +39,8 @@ _SIGNATURES = {
                        _c_int, _c_int, _c_void_p],
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                         _c_int, _c_int, _c_void_p],
+    "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
 }
@@ -257,6 +259,20 @@ def gemv_skinny(a, w, out):
     M, N, K = _check_mm(a, w, out)
     _call("blm_gemv_skinny", a.data_ptr(), _code(a), w.data_ptr(), _code(w), out.data_ptr(), _code(out),
           M, N, K, a.stride(0), out.stride(0), _stream())
+    return out
+
+
+def gemv_mfma_supported(M, N, K):
+    return bool(library().blm_gemv_mfma_supported(int(M), int(N), int(K)))
+
+
+def gemv_mfma(a, w, out):
+    """bfloat16 product for M <= 16 rows on the matrix cores; streams w once.  out: bfloat16 or float32."""
+    M, N, K = _check_mm(a, w, out)
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("gemv_mfma: operands must be bfloat16")
+    _call("blm_gemv_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
+          out.stride(0), _stream())
     return out
 
 

@@ -4,7 +4,8 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
 * float32 weights: the hand-written float kernels always (plain fused multiply-adds, no
   reduced-precision matrix mode), whatever the activation dtype.  This is the whole float32 path
   and also what keeps a tensor that a checkpoint stores in 32 bits exact in a bfloat16 run.
-* bfloat16 weights, few rows (decode): the hand-written skinny kernel that streams the weight once.
+* bfloat16 weights, up to 16 rows (decode): the hand-written skinny kernel on the matrix cores that
+  streams the weight once.
 * bfloat16 weights, many rows (prefill): the library product (hipBLASLt through torch), as the
   reference's engine leaves its matrix products to its tensor library
   (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).
@@ -16,6 +17,7 @@ import torch
 from ..csrc import ops
 
 SKINNY_MAX_ROWS = 8
+MFMA_SKINNY_MAX_ROWS = 16
 
 
 class Runtime:
@@ -47,7 +49,10 @@ class Runtime:
                     and x.stride(0) % 8 == 0:
                 return ops.gemv_skinny(x, w, out)
             return ops.gemm_tiled(x, w, out)
-        if M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+        aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+        if M <= MFMA_SKINNY_MAX_ROWS and aligned and ops.gemv_mfma_supported(M, N, K):
+            return ops.gemv_mfma(x, w, out)
+        if M <= SKINNY_MAX_ROWS and aligned:
             return ops.gemv_skinny(x, w, out)
         if out_dtype == torch.bfloat16:
             return torch.matmul(x, w.t(), out=out)

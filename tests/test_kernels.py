@@ -308,6 +308,40 @@ def test_gemv_skinny(ops, dtype, out_dtype, M):
         ops.gemv_skinny(dev(torch.zeros(9, K).to(DT[dtype])), dev(W), torch.empty(9, N, dtype=DT[out_dtype], device="cuda"))
 
 
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("M,N,K", [(1, 1001, 264), (8, 48, 64), (7, 130, 144), (16, 16, 512), (11, 333, 520),
+                                   (8, 257, 2048), (3, 40, 8192), (16, 100, 8200), (5, 31, 14336)])
+def test_gemv_mfma(ops, out_dtype, M, N, K):
+    """Matrix-core skinny product: every way K is cut among wavefronts, tails in N, K and M."""
+    g = torch.Generator().manual_seed(16)
+    A = torch.randn(M, K, generator=g).bfloat16()
+    W = torch.randn(N, K, generator=g).bfloat16()
+    # make one product term dominate a column so that a wrong operand layout cannot hide in the noise
+    W[N // 2, K - 8:] = 40.0
+    assert ops.gemv_mfma_supported(M, N, K)
+    out = torch.full((M, N), 7.0, dtype=DT[out_dtype], device="cuda")
+    ops.gemv_mfma(dev(A), dev(W), out)
+    want = A.double() @ W.double().T
+    got = out.double().cpu()
+    err = ((got - want).abs() / (want.abs() + want.abs().mean())).max()
+    assert float(err) <= (2e-5 if out_dtype == "float32" else 8e-3), f"error {float(err):.3g}"
+    # rows of a wider buffer, and an output with a row stride
+    wide = torch.randn(M, K + 24, generator=g).bfloat16()
+    big = torch.zeros(M, N + 5, dtype=DT[out_dtype], device="cuda")
+    ops.gemv_mfma(dev(wide)[:, 8:K + 8], dev(W), big[:, :N])
+    close(big[:, :N], wide[:, 8:K + 8].double() @ W.double().T, EPS[out_dtype] * 2)
+    assert bool((big[:, N:] == 0).all())
+
+
+def test_gemv_mfma_refuses_what_it_cannot_do(ops):
+    from burn_lm_amd.csrc.ops import KernelError
+    assert not ops.gemv_mfma_supported(17, 64, 64) and not ops.gemv_mfma_supported(4, 64, 60)
+    assert not ops.gemv_mfma_supported(4, 64, 16392)
+    with pytest.raises(KernelError, match="1..16"):
+        ops.gemv_mfma(dev(torch.zeros(17, 64).bfloat16()), dev(torch.zeros(8, 64).bfloat16()),
+                      torch.zeros(17, 8, dtype=torch.bfloat16, device="cuda"))
+
+
 def test_argmax_first_maximum_wins(ops):
     g = torch.Generator().manual_seed(7)
     x = torch.randn(6, 1000, generator=g)
