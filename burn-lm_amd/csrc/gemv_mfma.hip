@@ -14,8 +14,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 __device__ __forceinline__ uint4 ld16(const bf16* p) { return *reinterpret_cast<const uint4*>(p); }
 
-template <int KSTEPS, typename TC>
-__global__ void __launch_bounds__(1024)
+// KSTEPS: k-steps of 32 per wavefront.  MAXT: most threads of a block (sets the register budget).
+// KEEP_A: the activations' fragments stay in registers across the block's column tiles.
+template <int KSTEPS, int MAXT, bool KEEP_A, typename TC>
+__global__ void __launch_bounds__(MAXT)
     gemv_mfma_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, TC* __restrict__ C, int M, int N,
                      int K, int lda, int ldc, int n_tiles) {
   extern __shared__ float red[];  // [waves][256]
@@ -24,28 +26,50 @@ __global__ void __launch_bounds__(1024)
   const int row = lane & 15, kg = lane >> 4;
   const int kbase = wave * (KSTEPS * 32) + kg * 8;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  const int arow = row < M ? row : M - 1;   // rows >= M read a real row and are zeroed, so every load is in bounds
+  const bf16* ap = A + (size_t)arow * lda;
 
+  // Fragments of A beyond K or beyond M are zero, so whatever W holds there adds nothing; the
+  // weight loads can then be unconditional, with their addresses clamped into the matrix.
   uint4 a[KSTEPS];
+  if (KEEP_A) {
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) {
-    const int k = kbase + s * 32;
-    a[s] = (row < M && k < K) ? ld16(A + (size_t)row * lda + k) : zero;
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int k = kbase + s * 32;
+      const uint4 v = ld16(ap + (k < K ? k : K - 8));
+      a[s] = (row < M && k < K) ? v : zero;
+    }
   }
 
   for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     const int n = tile * 16 + row;
-    const bf16* wrow = W + (size_t)n * K;
-    uint4 w[KSTEPS];
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      const int k = kbase + s * 32;
-      w[s] = (n < N && k < K) ? ld16(wrow + k) : zero;
-    }
+    const bf16* wrow = W + (size_t)(n < N ? n : N - 1) * K;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    constexpr int CH = KSTEPS < 16 ? KSTEPS : 16;   // weight loads in flight per wavefront
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
-                                                    __builtin_bit_cast(bf16x8_t, w[s]), acc, 0, 0, 0);
+    for (int c = 0; c < KSTEPS; c += CH) {
+      uint4 w[CH];
+#pragma unroll
+      for (int s = 0; s < CH; ++s) {
+        const int k = kbase + (c + s) * 32;
+        w[s] = ld16(wrow + (k < K ? k : K - 8));
+      }
+      if (!KEEP_A) {
+#pragma unroll
+        for (int s = 0; s < CH; ++s) {
+          const int k = kbase + (c + s) * 32;
+          const uint4 v = ld16(ap + (k < K ? k : K - 8));
+          a[c + s] = (row < M && k < K) ? v : zero;
+        }
+      }
+      // All loads of the chunk are issued before its first MFMA: left alone, the scheduler reuses
+      // one register for every load and waits for each in turn, which makes the kernel latency-bound.
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < CH; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[c + s]),
+                                                      __builtin_bit_cast(bf16x8_t, w[s]), acc, 0, 0, 0);
+    }
     // acc[r] is C[m = kg*4 + r][n = tile*16 + row]
     if (n_waves == 1) {
 #pragma unroll
@@ -69,10 +93,14 @@ __global__ void __launch_bounds__(1024)
   }
 }
 
-// how K is cut: k-steps of 32 per wavefront and wavefronts per block; 0 if K is out of range
+// How K is cut: k-steps of 32 per wavefront and wavefronts per block; 0 if K is out of range.
+//   K <= 512          4 steps, up to 4 wavefronts
+//   K <= 2048        16 steps, up to 4 wavefronts   (256 threads: registers are plentiful)
+//   K <= 8192        32 steps, up to 8 wavefronts   (512 threads: 256 registers a lane)
+//   K <= 16384       32 steps, up to 16 wavefronts  (1024 threads: the A fragments are re-read per tile)
 static int plan_k(int K, int* ksteps) {
   if (K <= 512) { *ksteps = 4; return (K + 127) / 128; }
-  if (K <= 8192) { *ksteps = 16; return (K + 511) / 512; }
+  if (K <= 2048) { *ksteps = 16; return (K + 511) / 512; }
   if (K <= 16384) { *ksteps = 32; return (K + 1023) / 1024; }
   return 0;
 }
@@ -90,16 +118,17 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
   const int n_tiles = (N + 15) / 16;
   // enough blocks to fill the chip, few enough that a block reuses its activations
   int blocks = n_tiles;
-  const int cap = waves >= 8 ? 256 : 512;
+  const int cap = waves > 4 ? 256 : 512;
   if (blocks > cap) blocks = cap;
   dim3 grid(blocks), block(waves * BLM_WAVE);
   const size_t smem = waves > 1 ? (size_t)waves * 256 * sizeof(float) : 0;
-#define BLM_GM(KS)                                                                                          \
-  hipLaunchKernelGGL((gemv_mfma_kernel<KS, TC>), grid, block, smem, stream, (const bf16*)A, (const bf16*)W, \
-                     (TC*)C, M, N, K, lda, ldc, n_tiles)
-  if (ksteps == 4) BLM_GM(4);
-  else if (ksteps == 16) BLM_GM(16);
-  else BLM_GM(32);
+#define BLM_GM(KS, MAXT, KEEP)                                                                                  \
+  hipLaunchKernelGGL((gemv_mfma_kernel<KS, MAXT, KEEP, TC>), grid, block, smem, stream, (const bf16*)A,         \
+                     (const bf16*)W, (TC*)C, M, N, K, lda, ldc, n_tiles)
+  if (ksteps == 4) BLM_GM(4, 256, true);
+  else if (ksteps == 16) BLM_GM(16, 256, true);
+  else if (waves <= 8) BLM_GM(32, 512, true);
+  else BLM_GM(32, 1024, false);
 #undef BLM_GM
   BLM_LAUNCH_CHECK("gemv_mfma");
   return 0;

@@ -24,7 +24,7 @@ class StepError(ValueError):
 
 class Engine:
     def __init__(self, model, rt, max_tokens: int, max_seqs: Optional[int] = None,
-                 max_context: Optional[int] = None, page_size: int = 64):
+                 max_context: Optional[int] = None, page_size: int = 64, graphs: bool = True):
         self.model, self.rt = model, rt
         plan_max = model.plan.max_positions
         n_pages = (max_tokens + page_size - 1) // page_size
@@ -36,6 +36,8 @@ class Engine:
         model.prepare_positions(max_context)
         self.max_context = max_context
         self.vocab_size = model.vocab_size
+        from .graphs import DecodeGraphs
+        self.graphs = DecodeGraphs(self) if graphs else None
 
     # ---- sequences ---------------------------------------------------------------------------
     def open(self) -> int:
@@ -73,8 +75,13 @@ class Engine:
         self._check(entries)
         lengths = [self.cache.length(s) for s, _, _ in entries]
         self.cache.reserve([(s, len(t)) for s, t, _ in entries])  # raises before any change
-        step = self.build_step(entries, lengths)
-        logits = self.model.forward(step, self.cache)
+        key = self.graphs.key_for(entries, lengths) if self.graphs is not None else None
+        logits = self.graphs.run(key, entries, lengths) if key is not None else None
+        if logits is None:
+            step = self.build_step(entries, lengths)
+            logits = self.model.forward(step, self.cache)
+            if key is not None:
+                self.graphs.after_eager(key)
         for s, t, _ in entries:
             self.cache.advance(s, len(t))
         return logits

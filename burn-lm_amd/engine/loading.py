@@ -57,17 +57,18 @@ def load_model(folder, dtype="bfloat16", device="cuda:0"):
 
 
 def load_engine(folder, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_context=None, device="cuda:0",
-                page_size=64):
+                page_size=64, graphs=True):
     t0 = time.time()
     model, rt, cfg = load_model(folder, dtype, device)
-    eng = Engine(model, rt, max_tokens=max_tokens, max_seqs=max_seqs, max_context=max_context, page_size=page_size)
+    eng = Engine(model, rt, max_tokens=max_tokens, max_seqs=max_seqs, max_context=max_context, page_size=page_size,
+                 graphs=graphs)
     eng.config = cfg
     eng.load_seconds = time.time() - t0
     return eng
 
 
 def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_context=None,
-                  device="cuda:0", std=0.02, page_size=64):
+                  device="cuda:0", std=0.02, page_size=64, graphs=True):
     """Engine with seeded random weights made directly on the GPU (same generator as the
     random-weights mode that writes a folder, without the trip through a file)."""
     from ..weights.random_init import random_tensors
@@ -87,6 +88,7 @@ def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_s
         raise ValueError(f"random weights: the architecture's checkpoint lacks {missing}")
     model.bind(tensors, rt)
     model.config, model.architecture = cfg, arch
-    eng = Engine(model, rt, max_tokens=max_tokens, max_seqs=max_seqs, max_context=max_context, page_size=page_size)
+    eng = Engine(model, rt, max_tokens=max_tokens, max_seqs=max_seqs, max_context=max_context, page_size=page_size,
+                 graphs=graphs)
     eng.config = cfg
     return eng

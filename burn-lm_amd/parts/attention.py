@@ -17,6 +17,8 @@ from .base import KVNeed, Mixer, TensorSpec
 class Attention(Mixer):
     """params: width, heads, kv_heads, head_dim, scale, window (0 = all keys), position (the
     position-encoding object, given by the model builder).  names: q, k, v, o."""
+    graph_safe = True
+
 
     def tensor_specs(self):
         p = self.params

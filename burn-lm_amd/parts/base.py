@@ -59,6 +59,11 @@ class StateNeed:
 
 
 class Part:
+    # True if forward() only launches work on the current stream from device-side data, so that a
+    # decode step through this part can be captured into a HIP graph and replayed.  A part that
+    # reads the step's host-side lists (or syncs with the host) must leave this False.
+    graph_safe = False
+
     def __init__(self, params: dict, names: Dict[str, str]):
         self.params = dict(params)
         self.names = dict(names)

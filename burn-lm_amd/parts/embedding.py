@@ -13,6 +13,8 @@ from .base import Part, TensorSpec
 
 class Embedding(Part):
     """params: vocab, width.  names: weight."""
+    graph_safe = True
+
 
     def tensor_specs(self):
         return {self.names["weight"]: TensorSpec((self.params["vocab"], self.params["width"]))}
@@ -28,6 +30,8 @@ class Embedding(Part):
 
 class LMHead(Part):
     """params: vocab, width.  names: weight (the embedding's name when tied)."""
+    graph_safe = True
+
 
     def tensor_specs(self):
         return {self.names["weight"]: TensorSpec((self.params["vocab"], self.params["width"]))}

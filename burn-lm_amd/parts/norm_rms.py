@@ -13,6 +13,8 @@ from .base import Norm, TensorSpec
 
 class RMSNorm(Norm):
     """params: width, eps.  names: weight."""
+    graph_safe = True
+
 
     def tensor_specs(self):
         return {self.names["weight"]: TensorSpec((self.params["width"],))}

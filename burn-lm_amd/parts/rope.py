@@ -38,6 +38,8 @@ def rope_frequencies(head_dim, theta, scaling=None):
 
 class RotaryEncoding(PositionEncoding):
     """params: head_dim, theta, scaling (None or 4 numbers), pairing ("half" | "interleaved")."""
+    graph_safe = True
+
 
     def bind(self, tensors, rt):
         self.rt = rt

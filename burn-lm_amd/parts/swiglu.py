@@ -11,6 +11,8 @@ from .base import FeedForward, TensorSpec
 
 class SwiGLU(FeedForward):
     """params: width, inner.  names: gate, up, down."""
+    graph_safe = True
+
 
     def tensor_specs(self):
         d, i = self.params["width"], self.params["inner"]

@@ -12,7 +12,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # A: grouped heads (2 per group), head size 16, tied head, no frequency scaling
 TINY_A = dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=64, intermediate_size=176,
               num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
-              max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)
+              max_position_embeddings=1024, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)
 # B: one key-value head for six query heads, head size 24 (no power of two, not width/heads * anything
 # special), widths and vocabulary that are no powers of two, another eps, llama3 scaling whose three
 # branches are all hit at head size 24, separate head

@@ -192,3 +192,55 @@ def test_command_line_runs_a_prompt(folders, capsys):
     assert "##### BurnLM Stats" in out and "Tokens Per Second" in out
     main(["run", folders["A"], "--sample-len", "4", "--temperature", "0.7", "--seed", "3", "--no-stats", "hi"])
     assert "BurnLM Stats" not in capsys.readouterr().out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(folders, dtype):
+    """Decode steps replayed from a captured graph against the same steps run eagerly on a second
+    engine: several replays of one shape with eager work (prefills of other sequences, slot churn)
+    and synchronisations between them, batches that shrink below their bucket (padding), and a page
+    table that grows into the next width bucket."""
+    cfg, seed = TINIES["A"]
+    g = load(folders["A"], dtype, max_tokens=4096)
+    e = load(folders["A"], dtype, max_tokens=4096, graphs=False)
+    assert g.graphs.enabled and e.graphs is None
+    lens = [3, 70, 130, 9, 40]
+    prompts = [random_tokens(90 + i, cfg["vocab_size"], n) for i, n in enumerate(lens)]
+    sg = [g.open() for _ in lens]
+    se = [e.open() for _ in lens]
+    a = g.step([(s, p, [len(p) - 1]) for s, p in zip(sg, prompts)])
+    b = e.step([(s, p, [len(p) - 1]) for s, p in zip(se, prompts)])
+    assert torch.equal(a, b)
+    toks = [int(t) for t in a.argmax(1)]
+    live = list(range(5))
+    tol = 2e-6 if dtype == "float32" else 2e-2
+    kept = []
+    for k in range(400):
+        a = g.step([(sg[i], [toks[i]], [0]) for i in live])
+        b = e.step([(se[i], [toks[i]], [0]) for i in live])
+        kept.append(a)
+        assert rel_err(a.double().cpu().numpy(), b.double().cpu().numpy()) <= tol, f"decode step {k}, live {live}"
+        for row, i in enumerate(live):
+            toks[i] = int(b[row].argmax())
+        if k == 5:                       # eager work between replays: another sequence is prefilled and dropped
+            x = g.open(); g.step([(x, prompts[2], [])]); g.close(x)
+            y = e.open(); e.step([(y, prompts[2], [])]); e.close(y)
+            torch.cuda.synchronize()
+        if k in (9, 30):                 # a sequence ends: 5 -> 4 -> 3 live in the bucket of 8 / 4 (the longest stays)
+            i = live.pop(1 if k == 9 else 0)
+            g.close(sg[i]); e.close(se[i])
+    assert g.graphs.replays > 380 and len(g.graphs.captured) >= 3
+    assert not torch.equal(kept[0], kept[1]), "each step's logits are a tensor of their own"
+    assert max(g.length(sg[i]) for i in live) > 512, "the page table grew past the first width bucket"
+
+
+def test_a_part_that_is_not_graph_safe_turns_replay_off(folders):
+    from burn_lm_amd.parts.attention import Attention
+    eng = load(folders["A"], "float32")
+    assert eng.graphs.enabled
+    old = Attention.graph_safe
+    Attention.graph_safe = False
+    try:
+        assert not load(folders["A"], "float32").graphs.enabled
+    finally:
+        Attention.graph_safe = old
