@@ -75,8 +75,9 @@ class KVGroup:
         self.need, self.places = need, places
         self.page_size = page_size
         self.pool = PagePool(n_pages)
-        # [place in group, key|value, page, kv head, token in page, head_dim]
-        self.storage = torch.empty(len(places), 2, n_pages, need.n_kv_heads, page_size, need.head_dim,
+        # [place in group, key|value, page, kv head, token in page * head_dim]; a key page is
+        # [token][head_dim], a value page is stored transposed, [head_dim][token]
+        self.storage = torch.empty(len(places), 2, n_pages, need.n_kv_heads, page_size * need.head_dim,
                                    dtype=dtype, device=device)
         self.tables: Dict[int, List[int]] = {}  # slot -> page of each page index (-1 once released)
 
@@ -102,8 +103,9 @@ class KVView:
 
     def __init__(self, group: KVGroup, group_index: int, plane: int, store: bool):
         self.group_index, self.store = group_index, store
-        self.k = group.storage[plane, 0]
-        self.v = group.storage[plane, 1]
+        n_pages, nkv, hd = group.storage.shape[2], group.need.n_kv_heads, group.need.head_dim
+        self.k = group.storage[plane, 0].view(n_pages, nkv, group.page_size, hd)
+        self.v = group.storage[plane, 1].view(n_pages, nkv, hd, group.page_size)
         self.page_size = group.page_size
         self.need = group.need
 

@@ -2,7 +2,8 @@
 // Works for prefill (many query tokens per sequence) and decode (one), any even head size up
 // to 256, any head and group counts, float or bf16 storage.  Scores, the running maximum and
 // sum and the output accumulator are float.  Keys and values of the step's own tokens are
-// already in the cache when this runs.
+// already in the cache when this runs.  Key pages are [kv head][token][head_dim], value pages
+// [kv head][head_dim][token].
 //
 // Visibility: the query at position p of its sequence sees keys j of the same sequence with
 // j <= p and, if window > 0, p - j < window.
@@ -97,11 +98,11 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
       const float pj = __shfl(p, jj, BLM_WAVE);
       const int ja = j0 + jj;
       const int page = bt[ja / page_size];
-      const TA* vrow = vcache + (((size_t)page * nkv + kvh) * page_size + (ja % page_size)) * hd;
+      const TA* vcol = vcache + ((size_t)page * nkv + kvh) * page_size * hd + (ja % page_size);
 #pragma unroll
       for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) {
         const int d = lane + i * BLM_WAVE;
-        if (d < hd) acc[i] = fmaf(pj, to_float(vrow[d]), acc[i]);
+        if (d < hd) acc[i] = fmaf(pj, to_float(vcol[(size_t)d * page_size]), acc[i]);
       }
     }
     m = m_new;

@@ -1,0 +1,372 @@
+// Attention over the paged cache on the matrix cores (bf16 in, float softmax and accumulation).
+//
+// One wavefront works on 16 "query columns" against one page of 64 keys at a time:
+//   S^T = K Q^T        A = K rows (16 keys x head_dim), B = Q^T; the result leaves lane (kg, c) with
+//                       the scores of query column c = lane % 16 for keys kg*4 .. kg*4+3 of each
+//                       16-key tile, so the whole softmax of a query lives in the four lanes that
+//                       share c, and needs two cross-lane steps.
+//   O^T += V^T P^T      A = V^T rows (16 dims x 32 keys), B = P^T.  The probabilities a lane has
+//                       just computed are exactly the B fragment it must supply (the order of the
+//                       32 keys inside an MFMA is free as long as A and B agree), so P never moves.
+//                       V is cached transposed per page ([head_dim][64 tokens]) so that the A
+//                       fragment of V^T is two 8-byte loads.
+// No shared memory is needed for the products and nothing is transposed at run time.
+//
+// Prefill: the 16 query columns are 16 consecutive tokens of one head of one sequence.
+// Decode:  they are the query heads that share a key-value head, for one token; the key range is
+//          cut into splits that are merged afterwards (float partial results).
+// Visibility: query at position p sees keys j <= p of its sequence and, with a window w, p - j < w.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+#define AM_WAVES 4
+#define AM_PAGE 64
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+// keep the first n (0..4) bf16 of an 8-byte group, zero the rest
+__device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
+  if (n >= 4) return v;
+  if (n <= 0) return make_uint2(0u, 0u);
+  const unsigned long long m = (1ull << (16 * n)) - 1ull;
+  const unsigned long long x = ((unsigned long long)v.y << 32) | v.x;
+  const unsigned long long y = x & m;
+  return make_uint2((uint32_t)y, (uint32_t)(y >> 32));
+}
+
+// One page of keys for one wavefront.  qf: B fragments of Q^T.  Lane (kg = lane / 16, c = lane % 16)
+// owns query column c.  qpos / lo: highest / lowest key this lane's query may see.  max_key: highest
+// key index any query of the tile may see (values past it may be garbage and are zeroed).
+template <int HD>
+__device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf16* __restrict__ vp,
+                                          const uint4* qf, int key0, int qpos, int lo, int max_key, float scale,
+                                          float& m, float& l, f32x4_t* o) {
+  constexpr int KS = (HD + 31) / 32;
+  constexpr int DT = (HD + 15) / 16;
+  const int lane = threadIdx.x & (BLM_WAVE - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+
+  // issue the loads of the page: keys for S^T, values for O^T
+  uint4 kf[4][KS];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + kg * 8;
+      kf[t][ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(kp + (size_t)(t * 16 + c) * HD + d) : zero;
+    }
+  uint2 vf[DT][4];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      vf[dt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * AM_PAGE + t * 16 + kg * 4);
+
+  // scores
+  float s[4][4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[t][ks]),
+                                                    __builtin_bit_cast(bf16x8_t, qf[ks]), acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int kj = key0 + t * 16 + kg * 4 + r;
+      s[t][r] = (kj <= qpos && kj >= lo) ? acc[r] * scale : -INFINITY;
+    }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[t][r]);
+  mx = fmaxf(mx, __shfl_xor(mx, 16, BLM_WAVE));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, BLM_WAVE));
+  const float m_new = fmaxf(m, mx);
+  const float corr = (m == m_new) ? 1.f : expf(m - m_new);   // m = -inf, m_new finite -> 0
+  float psum = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float p = (s[t][r] == -INFINITY) ? 0.f : expf(s[t][r] - m_new);
+      s[t][r] = p;
+      psum += p;
+    }
+  l = l * corr + psum;
+  m = m_new;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
+
+  // O^T += V^T P^T, 32 keys (two 16-key tiles) per MFMA
+  const bool tail = key0 + AM_PAGE - 1 > max_key;   // uniform: the page holds places past the data
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    uint4 pf;
+    pf.x = pack_bf16x2(s[2 * h][0], s[2 * h][1]);
+    pf.y = pack_bf16x2(s[2 * h][2], s[2 * h][3]);
+    pf.z = pack_bf16x2(s[2 * h + 1][0], s[2 * h + 1][1]);
+    pf.w = pack_bf16x2(s[2 * h + 1][2], s[2 * h + 1][3]);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 v0 = vf[dt][2 * h], v1 = vf[dt][2 * h + 1];
+      if (tail) {   // 0 * garbage must stay 0
+        v0 = keep_first(v0, max_key - (key0 + (2 * h) * 16 + kg * 4) + 1);
+        v1 = keep_first(v1, max_key - (key0 + (2 * h + 1) * 16 + kg * 4) + 1);
+      }
+      const uint4 va = make_uint4(v0.x, v0.y, v1.x, v1.y);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, va),
+                                                      __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
+    }
+  }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_q(const bf16* qrow, uint4* qf) {
+  constexpr int KS = (HD + 31) / 32;
+  const int kg = (threadIdx.x & (BLM_WAVE - 1)) >> 4;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + kg * 8;
+    qf[ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(qrow + d) : make_uint4(0u, 0u, 0u, 0u);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// prefill: grid (ceil(G * q_tiles / 4), kv heads, sequences); each wavefront is independent
+// ---------------------------------------------------------------------------------------
+template <int HD>
+__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
+    attn_prefill_mfma_kernel(const bf16* __restrict__ q, int q_row_stride, bf16* __restrict__ out,
+                             const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
+                             const int* __restrict__ block_table, int table_width,
+                             const bf16* __restrict__ kcache, const bf16* __restrict__ vcache, int nh, int nkv,
+                             float scale, int window) {
+  constexpr int KS = (HD + 31) / 32;
+  constexpr int DT = (HD + 15) / 16;
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const int G = nh / nkv;
+  const int kvh = blockIdx.y, b = blockIdx.z;
+  const int row_begin = cu_seqlens[b];
+  const int n_b = cu_seqlens[b + 1] - row_begin;
+  const int u = blockIdx.x * AM_WAVES + wave;
+  const int g = u % G, qt = u / G;
+  if (qt * 16 >= n_b) return;   // no block-wide synchronisation is used in this kernel
+  const int head = kvh * G + g;
+  const int nq = min(16, n_b - qt * 16);
+  const int row = row_begin + qt * 16 + min(c, nq - 1);   // columns past the tile's end repeat its last query
+  const int qpos = positions[row];
+  const int qpos_first = positions[row_begin + qt * 16];
+  const int qpos_last = positions[row_begin + qt * 16 + nq - 1];
+  const int lo = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  const int lo_tile = (window > 0 && qpos_first - window + 1 > 0) ? qpos_first - window + 1 : 0;
+
+  uint4 qf[KS];
+  load_q<HD>(q + (size_t)row * q_row_stride + (size_t)head * HD, qf);
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int* bt = block_table + (size_t)b * table_width;
+  for (int pi = lo_tile / AM_PAGE; pi <= qpos_last / AM_PAGE; ++pi) {
+    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
+    attn_page<HD>(kcache + base, vcache + base, qf, pi * AM_PAGE, qpos, lo, qpos_last, scale, m, l, o);
+  }
+  l += __shfl_xor(l, 16, BLM_WAVE);
+  l += __shfl_xor(l, 32, BLM_WAVE);
+  if (c < nq) {
+    const float inv = 1.0f / l;
+    bf16* orow = out + (size_t)row * nh * HD + (size_t)head * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int d = dt * 16 + kg * 4;
+      if (HD % 16 == 0 || d < HD) {
+        uint2 w;
+        w.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+        w.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + d) = w;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// decode: grid (splits, kv heads * head tiles, tokens); partial results per split
+//   part_o [T, nh, splits, HD] float, part_ml [T, nh, splits, 2] float
+// ---------------------------------------------------------------------------------------
+template <int HD>
+__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
+    attn_decode_mfma_kernel(const bf16* __restrict__ q, int q_row_stride, const int* __restrict__ positions,
+                            const int* __restrict__ token_seq, const int* __restrict__ block_table,
+                            int table_width, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
+                            int nh, int nkv, float scale, int window, int n_splits, float* __restrict__ part_o,
+                            float* __restrict__ part_ml) {
+  constexpr int KS = (HD + 31) / 32;
+  constexpr int DT = (HD + 15) / 16;
+  __shared__ float sm_m[AM_WAVES][16], sm_l[AM_WAVES][16];
+  __shared__ float sm_o[AM_WAVES][16][HD];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const int split = blockIdx.x;
+  const int G = nh / nkv;
+  const int gtiles = (G + 15) / 16;
+  const int kvh = blockIdx.y / gtiles, g0 = (blockIdx.y % gtiles) * 16;
+  const int t = blockIdx.z;
+  const int b = token_seq[t];
+  const int head = kvh * G + min(g0 + c, G - 1);   // columns past the group's end repeat its last head
+
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  if (b >= 0) {
+    const int pos = positions[t];
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int first_page = lo / AM_PAGE, last_page = pos / AM_PAGE;
+    const int per_split = (last_page - first_page + 1 + n_splits - 1) / n_splits;
+    const int p_begin = first_page + split * per_split;
+    const int p_end = min(last_page + 1, p_begin + per_split);
+    const int* bt = block_table + (size_t)b * table_width;
+    uint4 qf[KS];
+    load_q<HD>(q + (size_t)t * q_row_stride + (size_t)head * HD, qf);
+    for (int pi = p_begin + wave; pi < p_end; pi += AM_WAVES) {
+      const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
+      attn_page<HD>(kcache + base, vcache + base, qf, pi * AM_PAGE, pos, lo, pos, scale, m, l, o);
+    }
+  }
+  l += __shfl_xor(l, 16, BLM_WAVE);
+  l += __shfl_xor(l, 32, BLM_WAVE);
+  if (kg == 0) { sm_m[wave][c] = m; sm_l[wave][c] = l; }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int d = dt * 16 + kg * 4 + r;
+      if (HD % 16 == 0 || d < HD) sm_o[wave][c][d] = o[dt][r];
+    }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 16 * HD; idx += blockDim.x) {
+    const int cc = idx / HD, d = idx - cc * HD;
+    if (g0 + cc >= G) continue;
+    float M = sm_m[0][cc];
+#pragma unroll
+    for (int k = 1; k < AM_WAVES; ++k) M = fmaxf(M, sm_m[k][cc]);
+    float L = 0.f, O = 0.f;
+#pragma unroll
+    for (int k = 0; k < AM_WAVES; ++k) {
+      const float f = (sm_m[k][cc] == M) ? 1.f : expf(sm_m[k][cc] - M);
+      L += sm_l[k][cc] * f;
+      O += sm_o[k][cc][d] * f;
+    }
+    const size_t at = ((size_t)t * nh + kvh * G + g0 + cc) * n_splits + split;
+    part_o[at * HD + d] = O;
+    if (d == 0) { part_ml[at * 2] = M; part_ml[at * 2 + 1] = L; }
+  }
+}
+
+template <int HD>
+__global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                           const int* __restrict__ token_seq, bf16* __restrict__ out, int nh,
+                                           int n_splits) {
+  const int head = blockIdx.x, t = blockIdx.y;
+  const int d = threadIdx.x;
+  if (d >= HD) return;
+  bf16* o = out + ((size_t)t * nh + head) * HD;
+  if (token_seq[t] < 0) { o[d] = from_float<bf16>(0.f); return; }   // padding token
+  const size_t base = ((size_t)t * nh + head) * n_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  float L = 0.f, O = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float ms = part_ml[(base + s) * 2];
+    const float f = (ms == M) ? 1.f : expf(ms - M);
+    L += part_ml[(base + s) * 2 + 1] * f;
+    O += part_o[(base + s) * HD + d] * f;
+  }
+  o[d] = from_float<bf16>(O / L);
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+static bool hd_ok(int hd, int max_hd) { return hd >= 16 && hd <= max_hd && (hd & (hd - 1)) == 0; }
+
+extern "C" int blm_attn_prefill_mfma_supported(int act_dtype, int hd, int page_size) {
+  return (act_dtype == BLM_BF16 && page_size == AM_PAGE && hd_ok(hd, 256)) ? 1 : 0;
+}
+extern "C" int blm_attn_decode_supported(int act_dtype, int hd, int page_size) {
+  return (act_dtype == BLM_BF16 && page_size == AM_PAGE && hd_ok(hd, 128)) ? 1 : 0;
+}
+
+extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out, int act_dtype,
+                                     const int* positions, const int* cu_seqlens, const int* block_table,
+                                     int table_width, const void* kcache, const void* vcache, int page_size,
+                                     int n_seqs, int max_new, int nh, int nkv, int hd, float scale, int window,
+                                     hipStream_t stream) {
+  BLM_REQUIRE(n_seqs > 0 && n_seqs <= 65535 && max_new > 0 && nh > 0 && nkv > 0 && nkv <= 65535 && nh % nkv == 0,
+              "attn_prefill_mfma: bad sizes seqs=%d max_new=%d heads=%d kv_heads=%d", n_seqs, max_new, nh, nkv);
+  BLM_REQUIRE(blm_attn_prefill_mfma_supported(act_dtype, hd, page_size),
+              "attn_prefill_mfma: needs bfloat16, pages of 64 and a head_dim of 16, 32, 64, 128 or 256 "
+              "(got dtype %d, page %d, head_dim %d)", act_dtype, page_size, hd);
+  BLM_REQUIRE(table_width > 0 && window >= 0, "attn_prefill_mfma: bad geometry");
+  BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0,
+              "attn_prefill_mfma: q rows must be 16-byte aligned");
+  const int G = nh / nkv;
+  const long long units = (long long)G * ((max_new + 15) / 16);
+  dim3 grid((unsigned)((units + AM_WAVES - 1) / AM_WAVES), nkv, n_seqs), block(AM_WAVES * BLM_WAVE);
+#define BLM_AP(HD)                                                                                               \
+  case HD:                                                                                                       \
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<HD>), grid, block, 0, stream, (const bf16*)q, q_row_stride,      \
+                       (bf16*)out, positions, cu_seqlens, block_table, table_width, (const bf16*)kcache,          \
+                       (const bf16*)vcache, nh, nkv, scale, window);                                              \
+    break
+  switch (hd) { BLM_AP(16); BLM_AP(32); BLM_AP(64); BLM_AP(128); BLM_AP(256); }
+#undef BLM_AP
+  BLM_LAUNCH_CHECK("attn_prefill_mfma");
+  return 0;
+}
+
+// workspace: part_o needs T*nh*n_splits*hd floats, part_ml T*nh*n_splits*2 floats
+extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int act_dtype, const int* positions,
+                               const int* token_seq, const int* block_table, int table_width, const void* kcache,
+                               const void* vcache, int page_size, int T, int nh, int nkv, int hd, float scale,
+                               int window, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && T <= 65535 && nh > 0 && nkv > 0 && nh % nkv == 0,
+              "attn_decode: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
+  BLM_REQUIRE(blm_attn_decode_supported(act_dtype, hd, page_size),
+              "attn_decode: needs bfloat16, pages of 64 and a head_dim of 16, 32, 64 or 128 "
+              "(got dtype %d, page %d, head_dim %d)", act_dtype, page_size, hd);
+  BLM_REQUIRE(table_width > 0 && window >= 0 && n_splits >= 1 && n_splits <= 65535,
+              "attn_decode: bad geometry width=%d window=%d splits=%d", table_width, window, n_splits);
+  BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attn_decode: q rows must be 16-byte aligned");
+  const int G = nh / nkv;
+  const int gtiles = (G + 15) / 16;
+  BLM_REQUIRE((long long)nkv * gtiles <= 65535, "attn_decode: too many heads");
+  dim3 grid(n_splits, nkv * gtiles, T), block(AM_WAVES * BLM_WAVE);
+  dim3 cgrid(nh, T), cblock(hd < 64 ? 64 : hd);
+#define BLM_AD(HD)                                                                                                 \
+  case HD:                                                                                                         \
+    hipLaunchKernelGGL((attn_decode_mfma_kernel<HD>), grid, block, 0, stream, (const bf16*)q, q_row_stride,         \
+                       positions, token_seq, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache,    \
+                       nh, nkv, scale, window, n_splits, part_o, part_ml);                                          \
+    BLM_LAUNCH_CHECK("attn_decode_mfma");                                                                          \
+    hipLaunchKernelGGL((attn_decode_combine_kernel<HD>), cgrid, cblock, 0, stream, part_o, part_ml, token_seq,      \
+                       (bf16*)out, nh, n_splits);                                                                  \
+    break
+  switch (hd) { BLM_AD(16); BLM_AD(32); BLM_AD(64); BLM_AD(128); }
+#undef BLM_AD
+  BLM_LAUNCH_CHECK("attn_decode_combine");
+  return 0;
+}

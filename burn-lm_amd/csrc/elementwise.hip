@@ -84,7 +84,9 @@ extern "C" int blm_add_rmsnorm(float* h, const void* delta, const void* gamma, i
 // ---------------------------------------------------------------------------------------
 // rotary encoding of q (in place) and k, and the write of k, v into the paged cache
 //   qkv row layout: [q: nh*hd | k: nkv*hd | v: nkv*hd]
-//   cache plane layout: [page][kv head][slot in page][hd]
+//   key plane layout:   [page][kv head][slot in page][hd]
+//   value plane layout: [page][kv head][hd][slot in page]   (transposed, so that the matrix-core
+//                        attention kernels find the keys of a page contiguous for every lane)
 //   pairing 0: lanes (2i, 2i+1) form a pair; pairing 1: lanes (i, i + hd/2)
 // ---------------------------------------------------------------------------------------
 template <typename TA>
@@ -129,7 +131,7 @@ __global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict
     const TA* v = row + (size_t)(nh + nkv) * hd;
     for (int w = threadIdx.x; w < nkv * hd; w += blockDim.x) {
       const int head = w / hd, d = w - head * hd;
-      vcache[(((size_t)page * nkv + head) * page_size + slot) * hd + d] = v[w];
+      vcache[(((size_t)page * nkv + head) * hd + d) * page_size + slot] = v[w];
     }
   }
 }

@@ -34,7 +34,11 @@ _SIGNATURES = {
     "blm_attn_decode": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                         _c_void_p, _c_void_p, _c_void_p],
-    "blm_attn_decode_supported": [_c_int, _c_int],
+    "blm_attn_decode_supported": [_c_int, _c_int, _c_int],
+    "blm_attn_prefill_mfma_supported": [_c_int, _c_int, _c_int],
+    "blm_attn_prefill_mfma": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                              _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                              _c_int, _c_void_p],
     "blm_gemm_tiled": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_void_p],
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
@@ -116,6 +120,13 @@ def _ptr(t):
     return 0 if t is None else t.data_ptr()
 
 
+def _check_planes(who, kcache, vcache, nkv, page_size, hd):
+    """Key plane [pages, kv_heads, page, head_dim]; value plane [pages, kv_heads, head_dim, page]."""
+    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or tuple(vcache.shape) != (kcache.shape[0], nkv, hd, page_size):
+        raise KernelError(f"{who}: cache planes {tuple(kcache.shape)} / {tuple(vcache.shape)} do not fit keys "
+                          f"[pages, {nkv}, {page_size}, {hd}] and values [pages, {nkv}, {hd}, {page_size}]")
+
+
 # ------------------------------------------------------------------------------------------
 def embed_gather(table, ids, out_h):
     """out_h[t, :] = table[ids[t], :] as float32.  ids must already be checked against the vocabulary."""
@@ -156,7 +167,8 @@ def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True):
 def rope_kv_write(qkv, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,
                   nh, nkv, hd, pairing, write_kv=True):
     """Rotate q (in place) and k of each token by its position's angles and store k, v in the
-    paged cache.  cos_sin: float32 [positions, hd/2, 2].  Cache planes: [pages, nkv, page, hd]."""
+    paged cache.  cos_sin: float32 [positions, hd/2, 2].  Key plane [pages, nkv, page, hd]; value
+    plane [pages, nkv, hd, page]."""
     _gpu(qkv, positions, token_seq, block_table, cos_sin, kcache, vcache)
     T = qkv.shape[0]
     _contig("qkv", qkv); _contig("cos_sin", cos_sin); _contig("kcache", kcache); _contig("vcache", vcache)
@@ -167,9 +179,7 @@ def rope_kv_write(qkv, positions, token_seq, block_table, cos_sin, kcache, vcach
         raise KernelError("rope_kv_write: cos_sin must be float32 [positions, head_dim/2, 2]")
     if kcache.dtype != qkv.dtype or vcache.dtype != qkv.dtype:
         raise KernelError("rope_kv_write: cache and activations must share a dtype")
-    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or kcache.shape != vcache.shape:
-        raise KernelError(f"rope_kv_write: cache plane shape {tuple(kcache.shape)} does not fit "
-                          f"[pages, {nkv}, {page_size}, {hd}]")
+    _check_planes("rope_kv_write", kcache, vcache, nkv, page_size, hd)
     _call("blm_rope_kv_write", qkv.data_ptr(), _code(qkv), positions.data_ptr(), token_seq.data_ptr(),
           block_table.data_ptr(), block_table.shape[1], cos_sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
           page_size, T, nh, nkv, hd, pairing, 1 if write_kv else 0, _stream())
@@ -197,8 +207,7 @@ def attn_paged(q, q_row_stride, out, positions, token_seq, block_table, kcache, 
         raise KernelError("attn_paged: out must be [T, heads*head_dim] and share q's dtype with the cache")
     if q.stride(-1) != 1 or q_row_stride < nh * hd:
         raise KernelError("attn_paged: q rows must be contiguous and at least heads*head_dim long")
-    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or kcache.shape != vcache.shape:
-        raise KernelError("attn_paged: cache plane shape does not fit [pages, kv_heads, page, head_dim]")
+    _check_planes("attn_paged", kcache, vcache, nkv, page_size, hd)
     _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
     _call("blm_attn_paged", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
@@ -206,9 +215,36 @@ def attn_paged(q, q_row_stride, out, positions, token_seq, block_table, kcache, 
     return out
 
 
-def attn_decode_supported(dtype, hd):
-    """Whether the split-key decode kernel takes this head size (else the generic kernel does)."""
-    return dtype in DTYPE_CODE and bool(library().blm_attn_decode_supported(DTYPE_CODE[dtype], int(hd)))
+def attn_decode_supported(dtype, hd, page_size=64):
+    """Whether the matrix-core decode kernel takes this case (else the generic kernel does)."""
+    return dtype in DTYPE_CODE and bool(library().blm_attn_decode_supported(DTYPE_CODE[dtype], int(hd), int(page_size)))
+
+
+def attn_prefill_mfma_supported(dtype, hd, page_size=64):
+    return dtype in DTYPE_CODE and bool(
+        library().blm_attn_prefill_mfma_supported(DTYPE_CODE[dtype], int(hd), int(page_size)))
+
+
+def attn_prefill_mfma(q, q_row_stride, out, positions, cu_seqlens, block_table, kcache, vcache, page_size,
+                      n_seqs, max_new, nh, nkv, hd, scale, window=0):
+    """Causal attention of packed sequences over their cached keys on the matrix cores (bfloat16).
+    Rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out belong to sequence b; max_new is the most
+    rows any sequence has."""
+    _gpu(q, out, positions, cu_seqlens, block_table, kcache, vcache)
+    T = out.shape[0]
+    _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
+    if out.shape[1] != nh * hd or out.dtype != q.dtype or kcache.dtype != q.dtype:
+        raise KernelError("attn_prefill_mfma: out must be [T, heads*head_dim] and share q's dtype with the cache")
+    if q.stride(-1) != 1 or q_row_stride < nh * hd:
+        raise KernelError("attn_prefill_mfma: q rows must be contiguous and at least heads*head_dim long")
+    _check_planes("attn_prefill_mfma", kcache, vcache, nkv, page_size, hd)
+    _i32("positions", positions, T); _i32("cu_seqlens", cu_seqlens, n_seqs + 1); _i32("block_table", block_table)
+    if block_table.shape[0] < n_seqs:
+        raise KernelError("attn_prefill_mfma: the page table has fewer rows than there are sequences")
+    _call("blm_attn_prefill_mfma", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
+          cu_seqlens.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
+          page_size, int(n_seqs), int(max_new), nh, nkv, hd, float(scale), int(window), _stream())
+    return out
 
 
 def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache, vcache, page_size,
@@ -221,8 +257,7 @@ def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache,
         raise KernelError("attn_decode: out must be [T, heads*head_dim] and share q's dtype with the cache")
     if q.stride(-1) != 1 or q_row_stride < nh * hd:
         raise KernelError("attn_decode: q rows must be contiguous and at least heads*head_dim long")
-    if tuple(kcache.shape[1:]) != (nkv, page_size, hd) or kcache.shape != vcache.shape:
-        raise KernelError("attn_decode: cache plane shape does not fit [pages, kv_heads, page, head_dim]")
+    _check_planes("attn_decode", kcache, vcache, nkv, page_size, hd)
     _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
     n_splits = max(1, int(n_splits))
     part_o = torch.empty(T * nh * n_splits * hd, dtype=torch.float32, device=out.device)

@@ -51,15 +51,20 @@ class Attention(Mixer):
         qkv = rt.linear(x, self.w_qkv)
         self.position.encode_and_store(qkv, step, view, nh, nkv, hd, store=view.store)
         out = torch.empty(x.shape[0], nh * hd, dtype=rt.dtype, device=x.device)
-        if step.max_new == 1 and rt.ops.attn_decode_supported(rt.dtype, hd) and qkv.shape[1] % 8 == 0:
+        table = view.block_table(step)
+        aligned = qkv.shape[1] % 8 == 0
+        if step.max_new == 1 and aligned and rt.ops.attn_decode_supported(rt.dtype, hd, view.page_size):
             # decode: cut each sequence's keys so that the whole chip has work
             span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
             pages = (span + view.page_size - 1) // view.page_size
-            blocks = x.shape[0] * nkv * ((nh // nkv + 7) // 8)
+            blocks = x.shape[0] * nkv * ((nh // nkv + 15) // 16)
             n_splits = max(1, min(pages, (1024 + blocks - 1) // blocks))
-            rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, view.block_table(step),
-                               view.k, view.v, view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
+            rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
+                               view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
+        elif aligned and rt.ops.attn_prefill_mfma_supported(rt.dtype, hd, view.page_size):
+            rt.ops.attn_prefill_mfma(qkv, qkv.shape[1], out, step.positions, step.cu_seqlens, table, view.k, view.v,
+                                     view.page_size, step.n_seqs, step.max_new, nh, nkv, hd, self.scale, self.window)
         else:
-            rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, view.block_table(step),
-                              view.k, view.v, view.page_size, nh, nkv, hd, self.scale, self.window)
+            rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
+                              view.page_size, nh, nkv, hd, self.scale, self.window)
         return rt.linear(out, self.w_o)

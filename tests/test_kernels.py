@@ -105,7 +105,7 @@ def test_rope_kv_write(ops, dtype, pairing, nh, nkv, hd):
     ang = torch.arange(64).double()[:, None] * freqs[None, :]
     cs = torch.stack([ang.cos(), ang.sin()], -1).float()
     k = torch.full((n_pages, nkv, page, hd), 99.0).to(DT[dtype])
-    v = torch.full((n_pages, nkv, page, hd), 99.0).to(DT[dtype])
+    v = torch.full((n_pages, nkv, hd, page), 99.0).to(DT[dtype])      # values are kept transposed per page
     qd, kd, vd = dev(qkv.clone()), dev(k), dev(v)
     ops.rope_kv_write(qd, dev(positions), dev(token_seq), dev(table), dev(cs), kd, vd, page, nh, nkv, hd,
                       PAIRING[pairing])
@@ -122,9 +122,10 @@ def test_rope_kv_write(ops, dtype, pairing, nh, nkv, hd):
         pg = int(table[int(token_seq[t]), p // page])
         written[pg, p % page] = True
         close(kc[pg, :, p % page], k_ref[t], EPS[dtype])
-        assert torch.equal(vc[pg, :, p % page], v_ref[t].to(DT[dtype]).double())
+        assert torch.equal(vc[pg, :, :, p % page], v_ref[t].to(DT[dtype]).double())
     untouched = ~written[:, None, :, None].expand(n_pages, nkv, page, hd)
-    assert bool((kc[untouched] == 99).all()) and bool((vc[untouched] == 99).all()), "nothing else is written"
+    assert bool((kc[untouched] == 99).all()), "nothing else is written"
+    assert bool((vc.transpose(2, 3)[untouched] == 99).all()), "nothing else is written"
     # a place that reads another's cache rotates q only
     qd2, kd2 = dev(qkv.clone()), dev(k)
     ops.rope_kv_write(qd2, dev(positions), dev(token_seq), dev(table), dev(cs), kd2, dev(v), page, nh, nkv, hd,
@@ -165,7 +166,7 @@ def test_attn_paged(ops, dtype, nh, nkv, hd, window):
     table = torch.full((3, width), -1, dtype=torch.int32)
     keys, values = [], []
     kc = torch.full((n_pages, nkv, page, hd), float("nan"))
-    vc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    vc = torch.full((n_pages, nkv, hd, page), float("nan"))
     for b, L in enumerate(lens):
         kb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
         vb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
@@ -177,7 +178,7 @@ def test_attn_paged(ops, dtype, nh, nkv, hd, window):
             table[b, i] = pg
             n = min(page, L - i * page)
             kc[pg, :, :n] = kb[i * page: i * page + n].transpose(0, 1).float()
-            vc[pg, :, :n] = vb[i * page: i * page + n].transpose(0, 1).float()
+            vc[pg, :, :, :n] = vb[i * page: i * page + n].permute(1, 2, 0).float()
     positions, token_seq = [], []
     for b, (L, n) in enumerate(zip(lens, new)):
         positions += list(range(L - n, L)); token_seq += [b] * n
@@ -199,48 +200,53 @@ def test_attn_paged(ops, dtype, nh, nkv, hd, window):
     assert bool((got[T - 1] == 0).all()), "a padding token gives zeros"
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("nh,nkv,hd,window,splits", [(4, 2, 16, 0, 3), (6, 1, 32, 0, 1), (5, 5, 64, 0, 4), (8, 2, 128, 0, 16),
-                                                      (12, 1, 64, 0, 2), (3, 1, 256, 0, 5), (4, 2, 32, 37, 2)])
-def test_attn_decode(ops, dtype, nh, nkv, hd, window, splits):
-    """The split-key decode kernel: sequences of very different lengths in one call (one of a single
-    key, one that ends exactly at a page edge), scrambled pages with NaN in every unused place, a far
-    key that stands out, more splits than some sequences have pages, a padding token."""
-    assert ops.attn_decode_supported(DT[dtype], hd) and not ops.attn_decode_supported(DT[dtype], 24)
-    g = torch.Generator().manual_seed(14)
-    page, n_pages = 16, 60
-    lens = [403, 1, 64, 17, 130]
+def _paged_case(g, lens, nkv, hd, page=64, n_pages=40, far_key=None):
+    """Random keys and values of several sequences laid out in scrambled pages, NaN everywhere else."""
     perm = torch.randperm(n_pages, generator=g).tolist()
-    width = 26
+    width = max((L + page - 1) // page for L in lens) + 2
     table = torch.full((len(lens), width), -1, dtype=torch.int32)
     keys, values = [], []
     kc = torch.full((n_pages, nkv, page, hd), float("nan"))
-    vc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    vc = torch.full((n_pages, nkv, hd, page), float("nan"))
     for b, L in enumerate(lens):
-        kb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
-        vb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
-        if L > 100:
-            kb[2] *= 5.0
+        kb = torch.randn(L, nkv, hd, generator=g).bfloat16()
+        vb = torch.randn(L, nkv, hd, generator=g).bfloat16()
+        if far_key is not None and L > far_key + 60:
+            kb[far_key] *= 5.0
         keys.append(kb); values.append(vb)
         for i in range((L + page - 1) // page):
             pg = perm.pop()
             table[b, i] = pg
             n = min(page, L - i * page)
             kc[pg, :, :n] = kb[i * page: i * page + n].transpose(0, 1).float()
-            vc[pg, :, :n] = vb[i * page: i * page + n].transpose(0, 1).float()
+            vc[pg, :, :, :n] = vb[i * page: i * page + n].permute(1, 2, 0).float()
+    return table, keys, values, kc.bfloat16(), vc.bfloat16()
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window,splits", [(4, 2, 16, 0, 3), (6, 1, 32, 0, 1), (5, 5, 64, 0, 4), (8, 2, 128, 0, 16),
+                                                      (32, 1, 64, 0, 2), (20, 1, 32, 0, 5), (4, 2, 32, 100, 2)])
+def test_attn_decode(ops, nh, nkv, hd, window, splits):
+    """The matrix-core decode kernel: sequences of very different lengths in one call (one of a single
+    key, one that ends exactly at a page edge), scrambled pages with NaN in every unused place, a far
+    key that stands out, more splits than some sequences have pages, more than 16 heads to a group,
+    a padding token."""
+    assert ops.attn_decode_supported(torch.bfloat16, hd) and not ops.attn_decode_supported(torch.bfloat16, 24)
+    assert not ops.attn_decode_supported(torch.float32, hd) and not ops.attn_decode_supported(torch.bfloat16, hd, 16)
+    g = torch.Generator().manual_seed(14)
+    lens = [403, 1, 64, 17, 130, 65]
+    table, keys, values, kc, vc = _paged_case(g, lens, nkv, hd, far_key=2)
     positions = [L - 1 for L in lens] + [0]
     token_seq = list(range(len(lens))) + [-1]
-    # order of the tokens need not be the order of the sequences
-    order = [3, 0, 5, 4, 1, 2]
+    order = [3, 0, 6, 4, 1, 2, 5]           # the order of the tokens need not be the order of the sequences
     positions = [positions[i] for i in order]; token_seq = [token_seq[i] for i in order]
     T = len(positions)
     stride = (nh + 2 * nkv) * hd
-    qkv = torch.randn(T, stride, generator=g).to(DT[dtype])
-    out = torch.full((T, nh * hd), 7.0, dtype=DT[dtype], device="cuda")
+    qkv = torch.randn(T, stride, generator=g).bfloat16()
+    out = torch.full((T, nh * hd), 7.0, dtype=torch.bfloat16, device="cuda")
     scale = 1.0 / math.sqrt(hd)
     ops.attn_decode(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
-                    dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc.to(DT[dtype])),
-                    dev(vc.to(DT[dtype])), page, nh, nkv, hd, scale, window, splits)
+                    dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc), dev(vc), 64, nh, nkv, hd,
+                    scale, window, splits)
     got = out.cpu().double().reshape(T, nh, hd)
     assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
     for t in range(T):
@@ -249,7 +255,37 @@ def test_attn_decode(ops, dtype, nh, nkv, hd, window, splits):
             assert bool((got[t] == 0).all())
             continue
         want = _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[b], values[b], positions[t], scale, window, nh // nkv)
-        close(got[t], want, EPS[dtype] * 2)
+        close(got[t], want, 1.5e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (6, 1, 32, 0), (5, 5, 64, 0), (8, 2, 128, 0), (2, 1, 256, 0),
+                                               (4, 2, 64, 90)])
+def test_attn_prefill_mfma(ops, nh, nkv, hd, window):
+    """The matrix-core prefill kernel on packed sequences: a whole prompt from position 0 (not a
+    multiple of 16 long), a chunk that continues a long past, one token on top of a past that ends at
+    a page edge, a single first token; a far key stands out; unused places hold NaN."""
+    assert ops.attn_prefill_mfma_supported(torch.bfloat16, hd) and not ops.attn_prefill_mfma_supported(torch.float32, hd)
+    g = torch.Generator().manual_seed(15)
+    lens = [150, 333, 65, 1, 40]             # length of each sequence after the step
+    new = [150, 70, 1, 1, 33]                # rows this step brings
+    table, keys, values, kc, vc = _paged_case(g, lens, nkv, hd, far_key=3)
+    positions, cu = [], [0]
+    for L, n in zip(lens, new):
+        positions += list(range(L - n, L)); cu.append(cu[-1] + n)
+    T = len(positions)
+    stride = (nh + 2 * nkv) * hd
+    qkv = torch.randn(T, stride, generator=g).bfloat16()
+    out = torch.full((T, nh * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+    scale = 1.0 / math.sqrt(hd)
+    ops.attn_prefill_mfma(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
+                          dev(torch.tensor(cu, dtype=torch.int32)), dev(table), dev(kc), dev(vc), 64, len(lens), max(new),
+                          nh, nkv, hd, scale, window)
+    got = out.cpu().double().reshape(T, nh, hd)
+    assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
+    for b in range(len(lens)):
+        for t in range(cu[b], cu[b + 1]):
+            want = _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[b], values[b], positions[t], scale, window, nh // nkv)
+            close(got[t], want, 1.5e-2)
 
 
 def test_attn_paged_refuses_what_it_cannot_do(ops):
@@ -258,6 +294,9 @@ def test_attn_paged_refuses_what_it_cannot_do(ops):
     i = torch.zeros(1, dtype=torch.int32, device="cuda")
     c = torch.zeros(1, 1, 16, 258, device="cuda")
     with pytest.raises(KernelError, match="head_dim 258"):
+        ops.attn_paged(z, 3 * 258, torch.zeros(1, 258, device="cuda"), i, i, i.view(1, 1), c, c.transpose(2, 3).contiguous(),
+                       16, 1, 1, 258, 1.0)
+    with pytest.raises(KernelError, match="cache planes"):
         ops.attn_paged(z, 3 * 258, torch.zeros(1, 258, device="cuda"), i, i, i.view(1, 1), c, c, 16, 1, 1, 258, 1.0)
     with pytest.raises(KernelError, match="GPU only"):
         ops.swiglu(torch.zeros(1, 4), torch.zeros(1, 2))
