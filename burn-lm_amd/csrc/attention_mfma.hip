@@ -276,6 +276,8 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   }
 }
 
+// Merge of the splits.  The loads of eight splits are issued together: a loop that waits for each
+// split in turn spends a memory round trip per split.
 template <int HD>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                            const int* __restrict__ token_seq, bf16* __restrict__ out, int nh,
@@ -286,14 +288,33 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, con
   bf16* o = out + ((size_t)t * nh + head) * HD;
   if (token_seq[t] < 0) { o[d] = from_float<bf16>(0.f); return; }   // padding token
   const size_t base = ((size_t)t * nh + head) * n_splits;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
   float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  for (int s0 = 0; s0 < n_splits; s0 += 8) {
+    float2 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = ml[min(s0 + i, n_splits - 1)];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) M = fmaxf(M, v[i].x);
+  }
   float L = 0.f, O = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ms = part_ml[(base + s) * 2];
-    const float f = (ms == M) ? 1.f : expf(ms - M);
-    L += part_ml[(base + s) * 2 + 1] * f;
-    O += part_o[(base + s) * HD + d] * f;
+  for (int s0 = 0; s0 < n_splits; s0 += 8) {
+    float2 v[8];
+    float po[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int s = min(s0 + i, n_splits - 1);
+      v[i] = ml[s];
+      po[i] = part_o[(base + s) * HD + d];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (s0 + i < n_splits) {
+        const float f = (v[i].x == M) ? 1.f : expf(v[i].x - M);
+        L += v[i].y * f;
+        O += po[i] * f;
+      }
+    }
   }
   o[d] = from_float<bf16>(O / L);
 }

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 _lib = None
 _lock = threading.Lock()
 
@@ -43,9 +43,10 @@ _SIGNATURES = {
                        _c_int, _c_int, _c_void_p],
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                         _c_int, _c_int, _c_void_p],
-    "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                      _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
-    "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
 }
 
@@ -301,13 +302,21 @@ def gemv_mfma_supported(M, N, K):
     return bool(library().blm_gemv_mfma_supported(int(M), int(N), int(K)))
 
 
-def gemv_mfma(a, w, out):
-    """bfloat16 product for M <= 16 rows on the matrix cores; streams w once.  out: bfloat16 or float32."""
-    M, N, K = _check_mm(a, w, out)
+def gemv_mfma(a, w, out, swiglu=False):
+    """bfloat16 product for M <= 16 rows on the matrix cores; streams w once.  out: bfloat16 or
+    float32.  swiglu=True: a is [M, 2K] = [gate | up] and the product runs on silu(gate) * up."""
+    _gpu(a, w, out)
+    M = a.shape[0]
+    N, K = w.shape
+    if a.shape[1] != (2 * K if swiglu else K) or out.shape != (M, N):
+        raise KernelError(f"gemv_mfma: shapes a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)} do not fit")
+    if a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemv_mfma: a and out need unit stride along their rows")
+    _contig("w", w)
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("gemv_mfma: operands must be bfloat16")
     _call("blm_gemv_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
-          out.stride(0), _stream())
+          out.stride(0), 1 if swiglu else 0, _stream())
     return out
 
 
@@ -320,7 +329,10 @@ def argmax(logits, out=None):
     if out is None:
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
     _i32("out", out, R)
-    _call("blm_argmax", logits.data_ptr(), out.data_ptr(), R, V, logits.stride(0), _stream())
+    slice_val = torch.empty(R * 32, dtype=torch.float32, device=logits.device)
+    slice_idx = torch.empty(R * 32, dtype=torch.int32, device=logits.device)
+    _call("blm_argmax", logits.data_ptr(), out.data_ptr(), R, V, logits.stride(0), slice_val.data_ptr(),
+          slice_idx.data_ptr(), _stream())
     return out
 
 

@@ -8,37 +8,65 @@
 
 #define SMP_THREADS 1024
 
-__global__ void __launch_bounds__(SMP_THREADS)
-    argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V, int ld) {
-  __shared__ float sv[SMP_THREADS / BLM_WAVE];
-  __shared__ int si[SMP_THREADS / BLM_WAVE];
-  const float* x = logits + (size_t)blockIdx.x * ld;
+// Two stages so that a row of a large vocabulary is searched by many blocks: stage one leaves the
+// best (value, index) of each slice of the row, stage two picks among the slices.  Ties go to the
+// lower index in both.
+#define ARGMAX_SLICES 32
+
+__device__ __forceinline__ void argmax_merge(float& best, int& bi, float ov, int oi) {
+  if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+}
+
+__global__ void __launch_bounds__(256)
+    argmax_slice_kernel(const float* __restrict__ logits, float* __restrict__ slice_val, int* __restrict__ slice_idx,
+                        int V, int ld) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const int row = blockIdx.y, slice = blockIdx.x;
+  const int per = (V + ARGMAX_SLICES - 1) / ARGMAX_SLICES;
+  const int beg = slice * per, end = min(V, beg + per);
+  const float* x = logits + (size_t)row * ld;
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const float v = x[i];
-    if (v > best || (v == best && i < bi)) { best = v; bi = i; }
-  }
+  for (int i = beg + threadIdx.x; i < end; i += blockDim.x) argmax_merge(best, bi, x[i], i);
 #pragma unroll
   for (int o = BLM_WAVE / 2; o > 0; o >>= 1) {
     const float ov = __shfl_xor(best, o, BLM_WAVE);
     const int oi = __shfl_xor(bi, o, BLM_WAVE);
-    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    argmax_merge(best, bi, ov, oi);
   }
   const int lane = threadIdx.x & (BLM_WAVE - 1), w = threadIdx.x / BLM_WAVE;
   if (lane == 0) { sv[w] = best; si[w] = bi; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int k = 1; k < SMP_THREADS / BLM_WAVE; ++k)
-      if (sv[k] > best || (sv[k] == best && si[k] < bi)) { best = sv[k]; bi = si[k]; }
-    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    for (int k = 1; k < 4; ++k) argmax_merge(best, bi, sv[k], si[k]);
+    slice_val[row * ARGMAX_SLICES + slice] = best;
+    slice_idx[row * ARGMAX_SLICES + slice] = bi;
   }
 }
 
-extern "C" int blm_argmax(const float* logits, int* out, int R, int V, int ld, hipStream_t stream) {
-  BLM_REQUIRE(R > 0 && V > 0 && ld >= V, "argmax: bad sizes R=%d V=%d ld=%d", R, V, ld);
-  hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(SMP_THREADS), 0, stream, logits, out, V, ld);
-  BLM_LAUNCH_CHECK("argmax");
+__global__ void argmax_final_kernel(const float* __restrict__ slice_val, const int* __restrict__ slice_idx,
+                                    int* __restrict__ out) {
+  const int row = blockIdx.x, lane = threadIdx.x;   // one wavefront per row
+  float best = lane < ARGMAX_SLICES ? slice_val[row * ARGMAX_SLICES + lane] : -INFINITY;
+  int bi = lane < ARGMAX_SLICES ? slice_idx[row * ARGMAX_SLICES + lane] : 0x7fffffff;
+#pragma unroll
+  for (int o = BLM_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, BLM_WAVE);
+    const int oi = __shfl_xor(bi, o, BLM_WAVE);
+    argmax_merge(best, bi, ov, oi);
+  }
+  if (lane == 0) out[row] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// scratch: R * 32 floats and R * 32 ints
+extern "C" int blm_argmax(const float* logits, int* out, int R, int V, int ld, float* slice_val, int* slice_idx,
+                          hipStream_t stream) {
+  BLM_REQUIRE(R > 0 && R <= 65535 && V > 0 && ld >= V, "argmax: bad sizes R=%d V=%d ld=%d", R, V, ld);
+  hipLaunchKernelGGL(argmax_slice_kernel, dim3(ARGMAX_SLICES, R), dim3(256), 0, stream, logits, slice_val, slice_idx, V, ld);
+  BLM_LAUNCH_CHECK("argmax_slice");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(BLM_WAVE), 0, stream, slice_val, slice_idx, out);
+  BLM_LAUNCH_CHECK("argmax_final");
   return 0;
 }
 

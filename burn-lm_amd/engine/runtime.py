@@ -58,3 +58,17 @@ class Runtime:
             return torch.matmul(x, w.t(), out=out)
         # float32 logits from bfloat16 operands with many rows: own kernel (float accumulation)
         return ops.gemm_tiled(x, w, out)
+
+    def swiglu_linear(self, gate_up, w):
+        """(silu(gate) * up) [M,K] @ w[N,K]^T for gate_up = [gate | up] of width 2K.  With few rows in
+        bfloat16 the gating is fused into the product's operand load; otherwise it runs as a kernel
+        of its own before the product."""
+        M = gate_up.shape[0]
+        N, K = w.shape
+        if (gate_up.dtype == w.dtype == torch.bfloat16 and M <= MFMA_SKINNY_MAX_ROWS and K % 8 == 0
+                and gate_up.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0 and ops.gemv_mfma_supported(M, N, K)):
+            out = torch.empty(M, N, dtype=self.dtype, device=gate_up.device)
+            return ops.gemv_mfma(gate_up, w, out, swiglu=True)
+        act = torch.empty(M, K, dtype=gate_up.dtype, device=gate_up.device)
+        ops.swiglu(gate_up, act)
+        return self.linear(act, w)

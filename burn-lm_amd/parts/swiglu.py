@@ -30,7 +30,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, step):
         rt = self.rt
-        gu = rt.linear(x, self.w_gate_up)
-        act = torch.empty(x.shape[0], self.inner, dtype=rt.dtype, device=x.device)
-        rt.ops.swiglu(gu, act)
-        return rt.linear(act, self.w_down)
+        return rt.swiglu_linear(rt.linear(x, self.w_gate_up), self.w_down)

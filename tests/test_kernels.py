@@ -349,7 +349,8 @@ def test_gemv_skinny(ops, dtype, out_dtype, M):
 
 @pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
 @pytest.mark.parametrize("M,N,K", [(1, 1001, 264), (8, 48, 64), (7, 130, 144), (16, 16, 512), (11, 333, 520),
-                                   (8, 257, 2048), (3, 40, 8192), (16, 100, 8200), (5, 31, 14336)])
+                                   (8, 257, 2048), (3, 40, 8192), (16, 100, 8200), (5, 31, 14336), (9, 77, 4104),
+                                   (2, 9000, 264), (8, 8200, 1024), (6, 100, 4096), (4, 52, 600)])
 def test_gemv_mfma(ops, out_dtype, M, N, K):
     """Matrix-core skinny product: every way K is cut among wavefronts, tails in N, K and M."""
     g = torch.Generator().manual_seed(16)
@@ -364,6 +365,17 @@ def test_gemv_mfma(ops, out_dtype, M, N, K):
     got = out.double().cpu()
     err = ((got - want).abs() / (want.abs() + want.abs().mean())).max()
     assert float(err) <= (2e-5 if out_dtype == "float32" else 8e-3), f"error {float(err):.3g}"
+    # the SwiGLU gating fused into the operand load equals the gating kernel followed by the product
+    gu = (torch.randn(M, 2 * K, generator=g) * 2).bfloat16()
+    act = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+    ops.swiglu(dev(gu), act)
+    plain = torch.empty(M, N, dtype=DT[out_dtype], device="cuda")
+    ops.gemv_mfma(act, dev(W), plain)
+    fused = torch.empty(M, N, dtype=DT[out_dtype], device="cuda")
+    ops.gemv_mfma(dev(gu), dev(W), fused, swiglu=True)
+    assert torch.equal(fused, plain)
+    x = gu.double()
+    close(fused, (torch.nn.functional.silu(x[:, :K]) * x[:, K:]).bfloat16().double() @ W.double().T, EPS[out_dtype] * 2)
     # rows of a wider buffer, and an output with a row stride
     wide = torch.randn(M, K + 24, generator=g).bfloat16()
     big = torch.zeros(M, N + 5, dtype=DT[out_dtype], device="cuda")
