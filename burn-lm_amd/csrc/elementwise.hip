@@ -32,23 +32,25 @@ extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* i
 
 // ---------------------------------------------------------------------------------------
 // residual add + RMS norm
-//   v = h[r] (+ delta[r]);  if write_h: h[r] = v;  out[i] = v / sqrt(mean(v^2) + eps) * gamma
-//   r = rows ? rows[i] : i
+//   v = h[r] (+ sum over planes p of delta[p][r]);  if write_h: h[r] = v;
+//   out[i] = v / sqrt(mean(v^2) + eps) * gamma;     r = rows ? rows[i] : i
+//   delta: n_planes planes of [T, D], in the activation dtype or float (partial products of a
+//   matrix product whose K was cut over blocks; summed here in plane order).
 // ---------------------------------------------------------------------------------------
-template <typename TA, typename TG>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta,
-                                   const TG* __restrict__ gamma, TA* __restrict__ out,
+template <typename TA, typename TG, typename TD>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_planes,
+                                   size_t plane_stride, const TG* __restrict__ gamma, TA* __restrict__ out,
                                    const int* __restrict__ rows, int D, float eps, int write_h) {
   __shared__ float red[17];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* hr = h + (size_t)r * D;
-  const TA* dr = delta ? delta + (size_t)r * D : nullptr;
+  const TD* dr = delta ? delta + (size_t)r * D : nullptr;
   float ss = 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float v = hr[d];
     if (dr) {
-      v += to_float(dr[d]);
+      for (int p = 0; p < n_planes; ++p) v += to_float(dr[p * plane_stride + d]);
       if (write_h) hr[d] = v;
     }
     ss += v * v;
@@ -58,27 +60,135 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__
   TA* o = out + (size_t)i * D;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float v = hr[d];
-    if (dr && !write_h) v += to_float(dr[d]);
+    if (dr && !write_h)
+      for (int p = 0; p < n_planes; ++p) v += to_float(dr[p * plane_stride + d]);
     o[d] = from_float<TA>(v * inv * to_float(gamma[d]));
   }
 }
 
-extern "C" int blm_add_rmsnorm(float* h, const void* delta, const void* gamma, int gamma_dtype,
-                               void* out, int act_dtype, const int* rows, int n_out, int D,
-                               float eps, int write_h, hipStream_t stream) {
-  BLM_REQUIRE(n_out > 0 && D > 0, "add_rmsnorm: bad sizes n=%d D=%d", n_out, D);
+// Fast form for rows that fit the block's registers (D a multiple of 4, at most 4 * 512 * ITERS):
+// every load of a row is issued at once with 16-byte accesses, and the normalised row is written
+// from registers instead of being read again.
+template <typename T>
+__device__ __forceinline__ void load4(const T* p, float* v);
+template <>
+__device__ __forceinline__ void load4<float>(const float* p, float* v) {
+  const float4 r = *reinterpret_cast<const float4*>(p);
+  v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+}
+template <>
+__device__ __forceinline__ void load4<bf16>(const bf16* p, float* v) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+  v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, const float* v);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <>
+__device__ __forceinline__ void store4<bf16>(bf16* p, const float* v) {
+  uint2 r;
+  r.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+  r.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = r;
+}
+
+template <typename TA, typename TG, typename TD, int ITERS>
+__global__ void __launch_bounds__(512)
+    add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_planes, size_t plane_stride,
+                           const TG* __restrict__ gamma, TA* __restrict__ out, const int* __restrict__ rows, int D,
+                           float eps, int write_h) {
+  __shared__ float red[17];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* hr = h + (size_t)r * D;
+  const TD* dr = delta ? delta + (size_t)r * D : nullptr;
+  float v[ITERS][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int d = (it * blockDim.x + threadIdx.x) * 4;
+    if (d < D) {
+      load4<float>(hr + d, v[it]);
+      if (dr) {
+        for (int p = 0; p < n_planes; ++p) {
+          float t[4];
+          load4<TD>(dr + p * plane_stride + d, t);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[it][e] += t[e];
+        }
+        if (write_h) store4<float>(hr + d, v[it]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += v[it][e] * v[it][e];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+  TA* o = out + (size_t)i * D;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int d = (it * blockDim.x + threadIdx.x) * 4;
+    if (d < D) {
+      float g[4], y[4];
+      load4<TG>(gamma + d, g);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = v[it][e] * inv * g[e];
+      store4<TA>(o + d, y);
+    }
+  }
+}
+
+template <typename TA, typename TG>
+static int launch_norm(float* h, const void* delta, int delta_dtype, int n_planes, size_t plane_stride,
+                       const void* gamma, void* out, const int* rows, int n_out, int D, float eps, int write_h,
+                       hipStream_t stream) {
   dim3 grid(n_out), block(D >= 2048 ? 512 : 256);
-#define BLM_NORM_CASE(TA, TG)                                                                  \
-  hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG>), grid, block, 0, stream, h, (const TA*)delta, \
-                     (const TG*)gamma, (TA*)out, rows, D, eps, write_h)
-  if (act_dtype == BLM_F32 && gamma_dtype == BLM_F32) BLM_NORM_CASE(float, float);
-  else if (act_dtype == BLM_BF16 && gamma_dtype == BLM_BF16) BLM_NORM_CASE(bf16, bf16);
-  else if (act_dtype == BLM_BF16 && gamma_dtype == BLM_F32) BLM_NORM_CASE(bf16, float);
-  else if (act_dtype == BLM_F32 && gamma_dtype == BLM_BF16) BLM_NORM_CASE(float, bf16);
-  else return blm_fail("add_rmsnorm: unsupported dtypes act=%d gamma=%d", act_dtype, gamma_dtype);
-#undef BLM_NORM_CASE
+  const bool aligned = D % 4 == 0 && plane_stride % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                       ((uintptr_t)gamma % 16) == 0 && ((uintptr_t)delta % 16) == 0;
+  if (aligned && D <= 4 * (int)block.x * 4) {
+    const int iters = (D + 4 * (int)block.x - 1) / (4 * (int)block.x);
+#define BLM_NV(TD, IT)                                                                                             \
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TG, TD, IT>), grid, block, 0, stream, h, (const TD*)delta, n_planes, \
+                     plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h)
+    if (delta_dtype == BLM_F32) {
+      if (iters == 1) BLM_NV(float, 1); else if (iters == 2) BLM_NV(float, 2); else BLM_NV(float, 4);
+    } else {
+      if (iters == 1) BLM_NV(bf16, 1); else if (iters == 2) BLM_NV(bf16, 2); else BLM_NV(bf16, 4);
+    }
+#undef BLM_NV
+    BLM_LAUNCH_CHECK("add_rmsnorm_vec");
+    return 0;
+  }
+  if (delta_dtype == BLM_F32)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG, float>), grid, block, 0, stream, h, (const float*)delta, n_planes,
+                       plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h);
+  else
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG, bf16>), grid, block, 0, stream, h, (const bf16*)delta, n_planes,
+                       plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h);
   BLM_LAUNCH_CHECK("add_rmsnorm");
   return 0;
+}
+
+extern "C" int blm_add_rmsnorm(float* h, const void* delta, int delta_dtype, int n_planes, long long plane_stride,
+                               const void* gamma, int gamma_dtype, void* out, int act_dtype, const int* rows,
+                               int n_out, int D, float eps, int write_h, hipStream_t stream) {
+  BLM_REQUIRE(n_out > 0 && D > 0, "add_rmsnorm: bad sizes n=%d D=%d", n_out, D);
+  BLM_REQUIRE(delta == nullptr || (n_planes >= 1 && n_planes <= 64 && plane_stride >= 0),
+              "add_rmsnorm: bad planes %d", n_planes);
+  BLM_REQUIRE(delta == nullptr || delta_dtype == BLM_F32 || delta_dtype == BLM_BF16, "add_rmsnorm: delta dtype %d", delta_dtype);
+  if (act_dtype == BLM_F32 && gamma_dtype == BLM_F32)
+    return launch_norm<float, float>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
+  if (act_dtype == BLM_BF16 && gamma_dtype == BLM_BF16)
+    return launch_norm<bf16, bf16>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
+  if (act_dtype == BLM_BF16 && gamma_dtype == BLM_F32)
+    return launch_norm<bf16, float>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
+  if (act_dtype == BLM_F32 && gamma_dtype == BLM_BF16)
+    return launch_norm<float, bf16>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
+  return blm_fail("add_rmsnorm: unsupported dtypes act=%d gamma=%d", act_dtype, gamma_dtype);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 2
+ABI_VERSION = 4
 _lib = None
 _lock = threading.Lock()
 
@@ -23,8 +23,8 @@ class KernelError(RuntimeError):
 
 _SIGNATURES = {
     "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
-    "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int,
-                        _c_int, _c_float, _c_int, _c_void_p],
+    "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p, _c_int,
+                        _c_void_p, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "blm_rope_kv_write": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                           _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -44,7 +44,7 @@ _SIGNATURES = {
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                         _c_int, _c_int, _c_void_p],
     "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                      _c_void_p],
+                      _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
@@ -143,7 +143,8 @@ def embed_gather(table, ids, out_h):
 
 def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True):
     """v = h[r] (+ delta[r]); h[r] = v if write_h; out[i] = v / sqrt(mean(v^2) + eps) * gamma,
-    with r = rows[i] if rows is given, else i.  h is the float32 residual stream."""
+    with r = rows[i] if rows is given, else i.  h is the float32 residual stream.  delta: [T, D] in
+    out's dtype, or float32 [planes, T, D] whose planes are summed (partial matrix products)."""
     _gpu(h, delta, gamma, out, rows)
     D = h.shape[1]
     n_out = out.shape[0]
@@ -152,16 +153,22 @@ def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True):
     _contig("h", h); _contig("out", out); _contig("gamma", gamma)
     if gamma.numel() != D or out.shape[1] != D:
         raise KernelError(f"add_rmsnorm: width mismatch h={D} gamma={gamma.numel()} out={out.shape[1]}")
+    planes, stride, dcode = 1, 0, 0
     if delta is not None:
         _contig("delta", delta)
-        if delta.shape != h.shape or delta.dtype != out.dtype:
-            raise KernelError("add_rmsnorm: delta must match h in shape and out in dtype")
+        if delta.dim() == 3:
+            if delta.shape[1:] != h.shape or delta.dtype != torch.float32:
+                raise KernelError("add_rmsnorm: partial deltas must be float32 [planes, T, D]")
+            planes, stride = delta.shape[0], h.shape[0] * D
+        elif delta.shape != h.shape or delta.dtype not in (out.dtype, torch.float32):
+            raise KernelError("add_rmsnorm: delta must match h in shape and be of out's dtype or float32")
+        dcode = _code(delta)
     if rows is not None:
         _i32("rows", rows, n_out)
     elif n_out != h.shape[0]:
         raise KernelError("add_rmsnorm: out needs one row per row of h when rows is not given")
-    _call("blm_add_rmsnorm", h.data_ptr(), _ptr(delta), gamma.data_ptr(), _code(gamma), out.data_ptr(), _code(out),
-          _ptr(rows), n_out, D, float(eps), 1 if write_h else 0, _stream())
+    _call("blm_add_rmsnorm", h.data_ptr(), _ptr(delta), dcode, planes, stride, gamma.data_ptr(), _code(gamma),
+          out.data_ptr(), _code(out), _ptr(rows), n_out, D, float(eps), 1 if write_h else 0, _stream())
     return out
 
 
@@ -302,21 +309,46 @@ def gemv_mfma_supported(M, N, K):
     return bool(library().blm_gemv_mfma_supported(int(M), int(N), int(K)))
 
 
-def gemv_mfma(a, w, out, swiglu=False):
-    """bfloat16 product for M <= 16 rows on the matrix cores; streams w once.  out: bfloat16 or
-    float32.  swiglu=True: a is [M, 2K] = [gate | up] and the product runs on silu(gate) * up."""
-    _gpu(a, w, out)
-    M = a.shape[0]
+def pack_weight(w):
+    """Copy of a bfloat16 weight matrix [N, K] in the order the matrix-core skinny product streams
+    it: packed[tile, step, lane, e] = w[tile*16 + lane%16, step*32 + (lane//16)*8 + e], with N
+    padded to a multiple of 16 and K to a multiple of 32 by zeros.  Returns a flat tensor."""
+    if w.dtype != torch.bfloat16 or w.dim() != 2:
+        raise KernelError("pack_weight: needs a bfloat16 matrix")
     N, K = w.shape
-    if a.shape[1] != (2 * K if swiglu else K) or out.shape != (M, N):
-        raise KernelError(f"gemv_mfma: shapes a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)} do not fit")
-    if a.stride(1) != 1 or out.stride(1) != 1:
+    Np, Kp = (N + 15) // 16 * 16, (K + 31) // 32 * 32
+    if (Np, Kp) != (N, K):
+        padded = torch.zeros(Np, Kp, dtype=w.dtype, device=w.device)
+        padded[:N, :K] = w
+        w = padded
+    # [tile, row, step, kg, e] -> [tile, step, kg, row, e]
+    return w.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+
+
+def gemv_mfma(a, packed, out, K, swiglu=False):
+    """bfloat16 product for M <= 16 rows on the matrix cores; streams the packed weights once.
+    packed: pack_weight(w) of w [N, K], N = out's width.  out: bfloat16 or float32 [M, N], or
+    float32 [groups, M, N]: K is then cut into that many groups whose partial products fill the
+    planes of out (the reader sums them).  swiglu=True: a is [M, 2K] = [gate | up] and the product
+    runs on silu(gate) * up."""
+    _gpu(a, packed, out)
+    groups = 1
+    if out.dim() == 3:
+        groups = out.shape[0]
+        if out.dtype != torch.float32 or not out.is_contiguous():
+            raise KernelError("gemv_mfma: partial outputs must be contiguous float32 [groups, M, N]")
+    M, N = out.shape[-2:]
+    if a.shape != (M, 2 * K if swiglu else K):
+        raise KernelError(f"gemv_mfma: shapes a={tuple(a.shape)} out={tuple(out.shape)} K={K} do not fit")
+    if packed.numel() != ((N + 15) // 16) * ((K + 31) // 32) * 512 or not packed.is_contiguous():
+        raise KernelError(f"gemv_mfma: the packed weights have {packed.numel()} elements, not those of a "
+                          f"[{N}, {K}] matrix")
+    if a.stride(1) != 1 or out.stride(-1) != 1:
         raise KernelError("gemv_mfma: a and out need unit stride along their rows")
-    _contig("w", w)
-    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+    if a.dtype != torch.bfloat16 or packed.dtype != torch.bfloat16:
         raise KernelError("gemv_mfma: operands must be bfloat16")
-    _call("blm_gemv_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
-          out.stride(0), 1 if swiglu else 0, _stream())
+    _call("blm_gemv_mfma", a.data_ptr(), packed.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
+          out.stride(-2), 1 if swiglu else 0, groups, _stream())
     return out
 
 

@@ -12,6 +12,8 @@ node is recorded (buffers are cleared, where needed, by kernels).
 """
 from __future__ import annotations
 
+import gc
+import weakref
 from typing import Dict, List, Tuple
 
 import torch
@@ -64,8 +66,16 @@ class _Captured:
         self.dev.copy_(self.host)
         self.graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize()
-        with torch.cuda.graph(self.graph, pool=pool):
-            self.logits = engine.model.forward(self.step, cache)
+        # No garbage collection while the capture is open: a collected object that owns GPU memory or
+        # another graph would free it in the middle of the capture, which HIP answers with an abort.
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph, pool=pool):
+                self.logits = engine.model.forward(self.step, cache)
+        finally:
+            if was_enabled:
+                gc.enable()
         torch.cuda.synchronize()
 
     def fill(self, entries, lengths, cache):
@@ -99,7 +109,9 @@ class _Captured:
 
 class DecodeGraphs:
     def __init__(self, engine):
-        self.engine = engine
+        # a weak reference: the engine owns this object, and a cycle would leave the graphs to the
+        # cyclic collector, which may run at any time (see the note on capture above)
+        self._engine = weakref.ref(engine)
         self.captured: Dict[Tuple[int, int], _Captured] = {}
         self.seen = set()
         self.pool = None
@@ -113,7 +125,7 @@ class DecodeGraphs:
         B = batch_bucket(len(entries))
         if B is None:
             return None
-        cache = self.engine.cache
+        cache = self._engine().cache
         pages = (max(lengths) + 1 + cache.page_size - 1) // cache.page_size
         return B, width_bucket(pages, cache.table_width)
 
@@ -124,7 +136,7 @@ class DecodeGraphs:
         if c is None:
             return None
         self.replays += 1
-        return c.run(entries, lengths, self.engine.cache)
+        return c.run(entries, lengths, self._engine().cache)
 
     def after_eager(self, key):
         """The shape has just run eagerly (so every kernel and library handle it needs exists):
@@ -133,4 +145,4 @@ class DecodeGraphs:
             return
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
-        self.captured[key] = _Captured(self.engine, key[0], key[1], self.pool)
+        self.captured[key] = _Captured(self._engine(), key[0], key[1], self.pool)

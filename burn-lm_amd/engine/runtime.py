@@ -20,6 +20,14 @@ SKINNY_MAX_ROWS = 8
 MFMA_SKINNY_MAX_ROWS = 16
 
 
+class LinearWeight:
+    """A bound weight matrix [N, K] and, for bfloat16, its copy packed for the skinny product."""
+
+    def __init__(self, w, packed=None):
+        self.w, self.packed = w, packed
+        self.shape, self.dtype = w.shape, w.dtype
+
+
 class Runtime:
     def __init__(self, dtype=torch.bfloat16, device="cuda:0", page_size=64):
         if dtype not in (torch.bfloat16, torch.float32):
@@ -37,12 +45,39 @@ class Runtime:
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
 
-    def linear(self, x, w, out_dtype=None, out=None):
-        """x [M,K] @ w[N,K]^T -> [M,N] in out_dtype (default: the activation dtype)."""
+    def weight(self, w):
+        """Prepares a bound matrix for linear(): bfloat16 matrices get the packed copy that the
+        skinny product streams (it doubles their memory; the plain copy serves prefill)."""
+        w = w.contiguous()
+        N, K = w.shape
+        if w.dtype == torch.bfloat16 and ops.gemv_mfma_supported(1, N, K):
+            return LinearWeight(w, ops.pack_weight(w))
+        return LinearWeight(w)
+
+    @staticmethod
+    def k_groups(N, K):
+        """Into how many groups a skinny product's K is cut so that a narrow output still gives
+        every compute unit a block: groups * (N / 16) tiles should reach 256 and a group should
+        span at most 2048 of K (its activations then fit the product's shared memory), but keeps at
+        least 1024."""
+        tiles = (N + 15) // 16
+        g = 1
+        while g < 8 and K // (g * 2) >= 1024 and (tiles * g < 256 or K // g > 2048):
+            g *= 2
+        return g
+
+    def linear(self, x, w, out_dtype=None, out=None, partials=False):
+        """x [M,K] @ w[N,K]^T -> [M,N] in out_dtype (default: the activation dtype).  w: a
+        LinearWeight from weight(), or a plain tensor.  partials=True allows the result to come as
+        float32 [groups, M, N] partial products (the caller hands it to a norm's add, which sums
+        them); it is used for narrow outputs in decode."""
+        packed = None
+        if isinstance(w, LinearWeight):
+            w, packed = w.w, w.packed
         M, K = x.shape
         N = w.shape[0]
         out_dtype = out_dtype or self.dtype
-        if out is None:
+        if out is None and not (partials and packed is not None):
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         if w.dtype == torch.float32 or x.dtype == torch.float32:
             if M <= SKINNY_MAX_ROWS and x.dtype == w.dtype == out_dtype == torch.float32 and K % 8 == 0 \
@@ -50,8 +85,15 @@ class Runtime:
                 return ops.gemv_skinny(x, w, out)
             return ops.gemm_tiled(x, w, out)
         aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-        if M <= MFMA_SKINNY_MAX_ROWS and aligned and ops.gemv_mfma_supported(M, N, K):
-            return ops.gemv_mfma(x, w, out)
+        if packed is not None and M <= MFMA_SKINNY_MAX_ROWS and aligned:
+            groups = self.k_groups(N, K) if partials else 1
+            if groups > 1:
+                return ops.gemv_mfma(x, packed, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), K)
+            if out is None:
+                out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+            return ops.gemv_mfma(x, packed, out, K)
+        if out is None:
+            out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         if M <= SKINNY_MAX_ROWS and aligned:
             return ops.gemv_skinny(x, w, out)
         if out_dtype == torch.bfloat16:
@@ -59,16 +101,21 @@ class Runtime:
         # float32 logits from bfloat16 operands with many rows: own kernel (float accumulation)
         return ops.gemm_tiled(x, w, out)
 
-    def swiglu_linear(self, gate_up, w):
+    def swiglu_linear(self, gate_up, w, partials=False):
         """(silu(gate) * up) [M,K] @ w[N,K]^T for gate_up = [gate | up] of width 2K.  With few rows in
         bfloat16 the gating is fused into the product's operand load; otherwise it runs as a kernel
         of its own before the product."""
         M = gate_up.shape[0]
         N, K = w.shape
-        if (gate_up.dtype == w.dtype == torch.bfloat16 and M <= MFMA_SKINNY_MAX_ROWS and K % 8 == 0
-                and gate_up.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0 and ops.gemv_mfma_supported(M, N, K)):
-            out = torch.empty(M, N, dtype=self.dtype, device=gate_up.device)
-            return ops.gemv_mfma(gate_up, w, out, swiglu=True)
+        packed = w.packed if isinstance(w, LinearWeight) else None
+        if (packed is not None and gate_up.dtype == torch.bfloat16 and M <= MFMA_SKINNY_MAX_ROWS
+                and gate_up.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0):
+            groups = self.k_groups(N, K) if partials else 1
+            if groups > 1:
+                out = torch.empty(groups, M, N, dtype=torch.float32, device=gate_up.device)
+            else:
+                out = torch.empty(M, N, dtype=self.dtype, device=gate_up.device)
+            return ops.gemv_mfma(gate_up, packed, out, K, swiglu=True)
         act = torch.empty(M, K, dtype=gate_up.dtype, device=gate_up.device)
         ops.swiglu(gate_up, act)
         return self.linear(act, w)

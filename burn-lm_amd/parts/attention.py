@@ -11,7 +11,12 @@ from __future__ import annotations
 
 import torch
 
+import os
+
 from .base import KVNeed, Mixer, TensorSpec
+
+# blocks the decode attention aims for when it cuts the key ranges into splits
+DECODE_TARGET_BLOCKS = int(os.environ.get("BLM_DECODE_BLOCKS", "512"))
 
 
 class Attention(Mixer):
@@ -42,8 +47,8 @@ class Attention(Mixer):
         ws = [tensors[self.names[r]] for r in ("q", "k", "v")]
         if len({w.dtype for w in ws}) != 1:
             ws = [w.float() for w in ws]
-        self.w_qkv = torch.cat(ws, dim=0).contiguous()
-        self.w_o = tensors[self.names["o"]].contiguous()
+        self.w_qkv = rt.weight(torch.cat(ws, dim=0))
+        self.w_o = rt.weight(tensors[self.names["o"]])
 
     def forward(self, x, step, view):
         rt = self.rt
@@ -58,7 +63,7 @@ class Attention(Mixer):
             span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
             pages = (span + view.page_size - 1) // view.page_size
             blocks = x.shape[0] * nkv * ((nh // nkv + 15) // 16)
-            n_splits = max(1, min(pages, (1024 + blocks - 1) // blocks))
+            n_splits = max(1, min(pages, (DECODE_TARGET_BLOCKS + blocks - 1) // blocks))
             rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                                view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
         elif aligned and rt.ops.attn_prefill_mfma_supported(rt.dtype, hd, view.page_size):
@@ -67,4 +72,4 @@ class Attention(Mixer):
         else:
             rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                               view.page_size, nh, nkv, hd, self.scale, self.window)
-        return rt.linear(out, self.w_o)
+        return rt.linear(out, self.w_o, partials=True)   # the block's next norm sums partial products

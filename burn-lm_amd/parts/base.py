@@ -10,7 +10,9 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
 
 * ``Part.tensor_specs() -> {checkpoint name: TensorSpec}`` and ``Part.bind(tensors, rt)``.
 * ``Norm.add_norm(h, delta, rows=None, write_h=True) -> x``: ``h += delta`` (if given), then
-  the normalised rows (all rows, or the rows listed in ``rows``).
+  the normalised rows (all rows, or the rows listed in ``rows``).  ``delta`` is ``[tokens, width]``
+  in the activation dtype, or float32 ``[planes, tokens, width]`` whose planes are summed (a
+  mixer or feed-forward may hand on the partial products of its last matrix product).
 * ``Mixer.cache_need() -> KVNeed | StateNeed | None`` and
   ``Mixer.forward(x, step, view) -> delta``; ``view`` is what the cache holds for this place
   in the layer order (``KVView``, ``StateView`` or ``None``).

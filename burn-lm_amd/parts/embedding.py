@@ -38,7 +38,7 @@ class LMHead(Part):
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.weight = tensors[self.names["weight"]].contiguous()
+        self.weight = rt.weight(tensors[self.names["weight"]])
 
     def forward(self, x):
         return self.rt.linear(x, self.weight, out_dtype=torch.float32)

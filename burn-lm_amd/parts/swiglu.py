@@ -24,10 +24,10 @@ class SwiGLU(FeedForward):
         g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
-        self.w_down = tensors[self.names["down"]].contiguous()
+        self.w_gate_up = rt.weight(torch.cat([g, u], dim=0))
+        self.w_down = rt.weight(tensors[self.names["down"]])
         self.inner = self.params["inner"]
 
     def forward(self, x, step):
         rt = self.rt
-        return rt.swiglu_linear(rt.linear(x, self.w_gate_up), self.w_down)
+        return rt.swiglu_linear(rt.linear(x, self.w_gate_up), self.w_down, partials=True)

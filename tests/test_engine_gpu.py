@@ -244,3 +244,29 @@ def test_a_part_that_is_not_graph_safe_turns_replay_off(folders):
         assert not load(folders["A"], "float32").graphs.enabled
     finally:
         Attention.graph_safe = old
+
+
+def test_wide_layers_take_the_grouped_products(tmp_path):
+    """A configuration wide enough (width 2048, feed-forward 4096) that the decode products of the
+    output and down projections are cut over K into partial planes: prompts, then decoded tokens,
+    against the plain implementation."""
+    from burn_lm_amd.engine.runtime import Runtime
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=4096, num_hidden_layers=1,
+               num_attention_heads=16, num_key_value_heads=4, head_dim=128, vocab_size=300, max_position_embeddings=256,
+               rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False)
+    assert Runtime.k_groups(2048, 2048) == 2 and Runtime.k_groups(2048, 4096) == 2 and Runtime.k_groups(6144, 2048) == 1
+    assert Runtime.k_groups(2048, 8192) == 4 and Runtime.k_groups(16384, 2048) == 1
+    folder = make_folder(tmp_path / "wide", cfg, seed=5, std=0.03)
+    plain = P.load_model_folder(folder)
+    reqs = [random_tokens(200 + i, 300, n) for i, n in enumerate([20, 9, 41])]
+    want = [P.transformer_forward([r], plain)[0] for r in reqs]
+    eng = load(folder, "bfloat16", max_tokens=512)
+    slots = [eng.open() for _ in reqs]
+    cut = [len(r) - 6 for r in reqs]
+    got = eng.step([(s, r[:c], [c - 1]) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
+    for i in range(3):
+        assert rel_err(got[i], want[i][cut[i] - 1]) <= TOL["bfloat16"]
+    for k in range(6):
+        got = eng.step([(s, [r[c + k]], [0]) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
+        for i in range(3):
+            assert rel_err(got[i], want[i][cut[i] + k]) <= TOL["bfloat16"], f"request {i}, decode step {k}"
