@@ -41,9 +41,12 @@ __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
 // One page of keys for one wavefront.  qf: B fragments of Q^T.  Lane (kg = lane / 16, c = lane % 16)
 // owns query column c.  qpos / lo: highest / lowest key this lane's query may see.  max_key: highest
 // key index any query of the tile may see (values past it may be garbage and are zeroed).
-template <int HD>
+// FULL: every key of the page is visible to every query of the tile, so no mask is computed.
+// The softmax runs in base 2: scale2 = scale * log2(e), m is the running maximum of s * scale2,
+// probabilities are exp2(s * scale2 - m); sums and outputs are the same as in base e.
+template <int HD, bool FULL>
 __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf16* __restrict__ vp,
-                                          const uint4* qf, int key0, int qpos, int lo, int max_key, float scale,
+                                          const uint4* qf, int key0, int qpos, int lo, int max_key, float scale2,
                                           float& m, float& l, f32x4_t* o) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
@@ -78,25 +81,30 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
                                                     __builtin_bit_cast(bf16x8_t, qf[ks]), acc, 0, 0, 0);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int kj = key0 + t * 16 + kg * 4 + r;
-      s[t][r] = (kj <= qpos && kj >= lo) ? acc[r] * scale : -INFINITY;
+      if (FULL) {
+        s[t][r] = acc[r] * scale2;
+      } else {
+        const int kj = key0 + t * 16 + kg * 4 + r;
+        s[t][r] = (kj <= qpos && kj >= lo) ? acc[r] * scale2 : -INFINITY;
+      }
     }
   }
-  float mx = -INFINITY;
+  float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[t][r]);
+  for (int t = 1; t < 4; ++t) mx = fmaxf(mx, fmaxf(fmaxf(s[t][0], s[t][1]), fmaxf(s[t][2], s[t][3])));
   mx = fmaxf(mx, __shfl_xor(mx, 16, BLM_WAVE));
   mx = fmaxf(mx, __shfl_xor(mx, 32, BLM_WAVE));
   const float m_new = fmaxf(m, mx);
-  const float corr = (m == m_new) ? 1.f : expf(m - m_new);   // m = -inf, m_new finite -> 0
+  // m = -inf, m_new finite -> 0;  both -inf (nothing visible yet) -> 1, and every p below is 0
+  const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
   float psum = 0.f;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float p = (s[t][r] == -INFINITY) ? 0.f : expf(s[t][r] - m_new);
+      float p;
+      if (FULL) p = __builtin_amdgcn_exp2f(s[t][r] - m_new);
+      else p = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s[t][r] - m_new);
       s[t][r] = p;
       psum += p;
     }
@@ -108,7 +116,7 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
     for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
 
   // O^T += V^T P^T, 32 keys (two 16-key tiles) per MFMA
-  const bool tail = key0 + AM_PAGE - 1 > max_key;   // uniform: the page holds places past the data
+  const bool tail = !FULL && key0 + AM_PAGE - 1 > max_key;   // uniform: the page holds places past the data
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     uint4 pf;
@@ -159,7 +167,9 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   const int kvh = blockIdx.y, b = blockIdx.z;
   const int row_begin = cu_seqlens[b];
   const int n_b = cu_seqlens[b + 1] - row_begin;
-  const int u = blockIdx.x * AM_WAVES + wave;
+  // The longest tiles (the last queries of a causal prompt see the most keys) are launched first,
+  // so that the tail of the launch is made of short ones.
+  const int u = (gridDim.x - 1 - blockIdx.x) * AM_WAVES + wave;
   const int g = u % G, qt = u / G;
   if (qt * 16 >= n_b) return;   // no block-wide synchronisation is used in this kernel
   const int head = kvh * G + g;
@@ -179,9 +189,17 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   const int* bt = block_table + (size_t)b * table_width;
+  const float scale2 = scale * 1.4426950408889634f;
+  // pages wholly inside every query's range need no mask: all keys <= the first query's position
+  // and, with a window, >= the last query's lower bound
+  const int lo_last = (window > 0 && qpos_last - window + 1 > 0) ? qpos_last - window + 1 : 0;
   for (int pi = lo_tile / AM_PAGE; pi <= qpos_last / AM_PAGE; ++pi) {
     const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
-    attn_page<HD>(kcache + base, vcache + base, qf, pi * AM_PAGE, qpos, lo, qpos_last, scale, m, l, o);
+    const int key0 = pi * AM_PAGE;
+    if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)
+      attn_page<HD, true>(kcache + base, vcache + base, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+    else
+      attn_page<HD, false>(kcache + base, vcache + base, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
   }
   l += __shfl_xor(l, 16, BLM_WAVE);
   l += __shfl_xor(l, 32, BLM_WAVE);
@@ -241,9 +259,14 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     const int* bt = block_table + (size_t)b * table_width;
     uint4 qf[KS];
     load_q<HD>(q + (size_t)t * q_row_stride + (size_t)head * HD, qf);
+    const float scale2 = scale * 1.4426950408889634f;
     for (int pi = p_begin + wave; pi < p_end; pi += AM_WAVES) {
       const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
-      attn_page<HD>(kcache + base, vcache + base, qf, pi * AM_PAGE, pos, lo, pos, scale, m, l, o);
+      const int key0 = pi * AM_PAGE;
+      if (key0 + AM_PAGE - 1 <= pos && key0 >= lo)
+        attn_page<HD, true>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+      else
+        attn_page<HD, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
     }
   }
   l += __shfl_xor(l, 16, BLM_WAVE);
@@ -266,7 +289,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     float L = 0.f, O = 0.f;
 #pragma unroll
     for (int k = 0; k < AM_WAVES; ++k) {
-      const float f = (sm_m[k][cc] == M) ? 1.f : expf(sm_m[k][cc] - M);
+      const float f = (sm_m[k][cc] == M) ? 1.f : __builtin_amdgcn_exp2f(sm_m[k][cc] - M);   // maxima are in base 2
       L += sm_l[k][cc] * f;
       O += sm_o[k][cc][d] * f;
     }
@@ -310,7 +333,7 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, con
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       if (s0 + i < n_splits) {
-        const float f = (v[i].x == M) ? 1.f : expf(v[i].x - M);
+        const float f = (v[i].x == M) ? 1.f : __builtin_amdgcn_exp2f(v[i].x - M);   // maxima are in base 2
         L += v[i].y * f;
         O += po[i] * f;
       }

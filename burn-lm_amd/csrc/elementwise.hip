@@ -284,8 +284,38 @@ __global__ void swiglu_kernel(const TA* __restrict__ gu, TA* __restrict__ out, i
   }
 }
 
+// 8 elements per thread with 16-byte accesses (bf16, I a multiple of 8)
+__global__ void swiglu_vec_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int I, long long total8) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total8) return;
+  const int per_row = I / 8;
+  const long long t = idx / per_row;
+  const int c = (int)(idx - t * per_row) * 8;
+  const bf16* g = gu + t * 2 * I + c;
+  const uint4 gv = *reinterpret_cast<const uint4*>(g);
+  const uint4 uv = *reinterpret_cast<const uint4*>(g + I);
+  const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+    const float f0 = g0 / (1.0f + expf(-g0)) * u0, f1 = g1 / (1.0f + expf(-g1)) * u1;
+    o[i] = (uint32_t)f32_to_bf16_bits(f0) | ((uint32_t)f32_to_bf16_bits(f1) << 16);
+  }
+  *reinterpret_cast<uint4*>(out + t * I + c) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 extern "C" int blm_swiglu(const void* gu, void* out, int act_dtype, int T, int I, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && I > 0 && T <= 65535 * 64, "swiglu: bad sizes T=%d I=%d", T, I);
+  if (act_dtype == BLM_BF16 && I % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+    const long long total8 = (long long)T * (I / 8);
+    const long long blocks = (total8 + 255) / 256;
+    BLM_REQUIRE(blocks < 2147483647LL, "swiglu: too many elements");
+    hipLaunchKernelGGL(swiglu_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16*)gu, (bf16*)out, I, total8);
+    BLM_LAUNCH_CHECK("swiglu_vec");
+    return 0;
+  }
   int gx = (I + 255) / 256;
   if (gx > 64) gx = 64;
   for (int t0 = 0; t0 < T; t0 += 65535) {
