@@ -44,7 +44,8 @@ __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
 // FULL: every key of the page is visible to every query of the tile, so no mask is computed.
 // The softmax runs in base 2: scale2 = scale * log2(e), m is the running maximum of s * scale2,
 // probabilities are exp2(s * scale2 - m); sums and outputs are the same as in base e.
-template <int HD, bool FULL>
+// KSTR / VSTR: row strides (elements) of the key page [64][KSTR] and the value page [HD][VSTR].
+template <int HD, bool FULL, int KSTR, int VSTR>
 __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf16* __restrict__ vp,
                                           const uint4* qf, int key0, int qpos, int lo, int max_key, float scale2,
                                           float& m, float& l, f32x4_t* o) {
@@ -61,14 +62,14 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + kg * 8;
-      kf[t][ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(kp + (size_t)(t * 16 + c) * HD + d) : zero;
+      kf[t][ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(kp + (size_t)(t * 16 + c) * KSTR + d) : zero;
     }
   uint2 vf[DT][4];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int t = 0; t < 4; ++t)
-      vf[dt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * AM_PAGE + t * 16 + kg * 4);
+      vf[dt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * VSTR + t * 16 + kg * 4);
 
   // scores
   float s[4][4];
@@ -150,7 +151,13 @@ __device__ __forceinline__ void load_q(const bf16* qrow, uint4* qf) {
 }
 
 // ---------------------------------------------------------------------------------------
-// prefill: grid (ceil(G * q_tiles / 4), kv heads, sequences); each wavefront is independent
+// prefill: grid (ceil(G * q_tiles / 4), kv heads, sequences)
+//
+// The four wavefronts of a block are four (head, 16-query tile) units that share a key-value head
+// and, for groups of four or more heads, the same queries.  Every page they need is brought into
+// shared memory once per block with coalesced 16-byte loads (the next page travels in registers
+// while the current one is used) and each wavefront takes its MFMA fragments from there; rows are
+// padded by 16 bytes so that the fragment reads do not collide.
 // ---------------------------------------------------------------------------------------
 template <int HD>
 __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
@@ -161,6 +168,11 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
                              float scale, int window) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
+  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 8;
+  constexpr int CHUNKS = AM_PAGE * HD / 8;              // 16-byte pieces of a page (keys and values alike)
+  constexpr int PER_THREAD = (CHUNKS + AM_WAVES * BLM_WAVE - 1) / (AM_WAVES * BLM_WAVE);
+  __shared__ __align__(16) bf16 k_lds[AM_PAGE * KSTR];
+  __shared__ __align__(16) bf16 v_lds[HD * VSTR];
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int c = lane & 15, kg = lane >> 4;
   const int G = nh / nkv;
@@ -169,17 +181,27 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   const int n_b = cu_seqlens[b + 1] - row_begin;
   // The longest tiles (the last queries of a causal prompt see the most keys) are launched first,
   // so that the tail of the launch is made of short ones.
-  const int u = (gridDim.x - 1 - blockIdx.x) * AM_WAVES + wave;
+  const int u0 = (gridDim.x - 1 - blockIdx.x) * AM_WAVES;
+  if ((u0 / G) * 16 >= n_b) return;   // the whole block lies past the sequence's end (uniform)
+  const int u = u0 + wave;
   const int g = u % G, qt = u / G;
-  if (qt * 16 >= n_b) return;   // no block-wide synchronisation is used in this kernel
+  const bool active = qt * 16 < n_b;
   const int head = kvh * G + g;
-  const int nq = min(16, n_b - qt * 16);
-  const int row = row_begin + qt * 16 + min(c, nq - 1);   // columns past the tile's end repeat its last query
+  const int nq = active ? min(16, n_b - qt * 16) : 1;
+  const int row = row_begin + (active ? qt * 16 + min(c, nq - 1) : 0);   // columns past the tile's end repeat its last query
   const int qpos = positions[row];
-  const int qpos_first = positions[row_begin + qt * 16];
-  const int qpos_last = positions[row_begin + qt * 16 + nq - 1];
+  const int qpos_first = positions[row_begin + (active ? qt * 16 : 0)];
+  const int qpos_last = positions[row_begin + (active ? qt * 16 + nq - 1 : 0)];
   const int lo = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
   const int lo_tile = (window > 0 && qpos_first - window + 1 > 0) ? qpos_first - window + 1 : 0;
+  const int lo_last = (window > 0 && qpos_last - window + 1 > 0) ? qpos_last - window + 1 : 0;
+  const int my_first = active ? lo_tile / AM_PAGE : 0x7fffffff, my_last = active ? qpos_last / AM_PAGE : -1;
+  // page range of the block: from its first unit's first page to its last active unit's last page
+  const int qt_lo = u0 / G, qt_hi = min((u0 + AM_WAVES - 1) / G, (n_b - 1) / 16);
+  const int blk_qfirst = positions[row_begin + qt_lo * 16];
+  const int blk_qlast = positions[row_begin + min(qt_hi * 16 + 15, n_b - 1)];
+  const int blk_first = ((window > 0 && blk_qfirst - window + 1 > 0) ? blk_qfirst - window + 1 : 0) / AM_PAGE;
+  const int blk_last = blk_qlast / AM_PAGE;
 
   uint4 qf[KS];
   load_q<HD>(q + (size_t)row * q_row_stride + (size_t)head * HD, qf);
@@ -187,20 +209,46 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   f32x4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-  const int* bt = block_table + (size_t)b * table_width;
   const float scale2 = scale * 1.4426950408889634f;
-  // pages wholly inside every query's range need no mask: all keys <= the first query's position
-  // and, with a window, >= the last query's lower bound
-  const int lo_last = (window > 0 && qpos_last - window + 1 > 0) ? qpos_last - window + 1 : 0;
-  for (int pi = lo_tile / AM_PAGE; pi <= qpos_last / AM_PAGE; ++pi) {
+  const int* bt = block_table + (size_t)b * table_width;
+
+  uint4 kreg[PER_THREAD], vreg[PER_THREAD];
+  auto fetch = [&](int pi) {
     const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
-    const int key0 = pi * AM_PAGE;
-    if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)
-      attn_page<HD, true>(kcache + base, vcache + base, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
-    else
-      attn_page<HD, false>(kcache + base, vcache + base, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;
+      if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {
+        kreg[i] = *reinterpret_cast<const uint4*>(kcache + base + (size_t)j * 8);
+        vreg[i] = *reinterpret_cast<const uint4*>(vcache + base + (size_t)j * 8);
+      }
+    }
+  };
+  fetch(blk_first);
+  for (int pi = blk_first; pi <= blk_last; ++pi) {
+    __syncthreads();   // the page before has been used by every wavefront
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;
+      if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {
+        const int kr = j / (HD / 8), kc = j - kr * (HD / 8);          // key row, 16-byte column
+        *reinterpret_cast<uint4*>(k_lds + kr * KSTR + kc * 8) = kreg[i];
+        const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8);  // value row (a dim), 16-byte column
+        *reinterpret_cast<uint4*>(v_lds + vr * VSTR + vc * 8) = vreg[i];
+      }
+    }
+    __syncthreads();
+    if (pi < blk_last) fetch(pi + 1);   // travels while this page is used
+    if (pi >= my_first && pi <= my_last) {
+      const int key0 = pi * AM_PAGE;
+      // pages wholly inside every query's range need no mask
+      if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)
+        attn_page<HD, true, KSTR, VSTR>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+      else
+        attn_page<HD, false, KSTR, VSTR>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+    }
   }
+  if (!active) return;
   l += __shfl_xor(l, 16, BLM_WAVE);
   l += __shfl_xor(l, 32, BLM_WAVE);
   if (c < nq) {
@@ -264,9 +312,9 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
       const int key0 = pi * AM_PAGE;
       if (key0 + AM_PAGE - 1 <= pos && key0 >= lo)
-        attn_page<HD, true>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+        attn_page<HD, true, HD, AM_PAGE>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
       else
-        attn_page<HD, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+        attn_page<HD, false, HD, AM_PAGE>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
     }
   }
   l += __shfl_xor(l, 16, BLM_WAVE);
