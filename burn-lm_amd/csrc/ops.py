@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 _lib = None
 _lock = threading.Lock()
 
@@ -309,13 +309,20 @@ def gemv_mfma_supported(M, N, K):
     return bool(library().blm_gemv_mfma_supported(int(M), int(N), int(K)))
 
 
-def pack_weight(w):
+def pack_weight(w, gated=False):
     """Copy of a bfloat16 weight matrix [N, K] in the order the matrix-core skinny product streams
     it: packed[tile, step, lane, e] = w[tile*16 + lane%16, step*32 + (lane//16)*8 + e], with N
-    padded to a multiple of 16 and K to a multiple of 32 by zeros.  Returns a flat tensor."""
+    padded to a multiple of 16 and K to a multiple of 32 by zeros.  Returns a flat tensor.
+    gated=True: w is [gate rows; up rows]; its rows are first re-ordered into blocks of 8 gate rows
+    followed by the 8 matching up rows, so that each tile holds 8 gated pairs (gemv_mfma gated=True)."""
     if w.dtype != torch.bfloat16 or w.dim() != 2:
         raise KernelError("pack_weight: needs a bfloat16 matrix")
     N, K = w.shape
+    if gated:
+        if N % 16:
+            raise KernelError("pack_weight: a gated matrix needs a multiple of 8 features")
+        half = N // 2
+        w = torch.stack([w[:half].view(half // 8, 8, K), w[half:].view(half // 8, 8, K)], dim=1).reshape(N, K)
     Np, Kp = (N + 15) // 16 * 16, (K + 31) // 32 * 32
     if (Np, Kp) != (N, K):
         padded = torch.zeros(Np, Kp, dtype=w.dtype, device=w.device)
@@ -325,20 +332,21 @@ def pack_weight(w):
     return w.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
 
 
-def gemv_mfma(a, packed, out, K, swiglu=False):
+def gemv_mfma(a, packed, out, K, gated=False):
     """bfloat16 product for M <= 16 rows on the matrix cores; streams the packed weights once.
-    packed: pack_weight(w) of w [N, K], N = out's width.  out: bfloat16 or float32 [M, N], or
-    float32 [groups, M, N]: K is then cut into that many groups whose partial products fill the
-    planes of out (the reader sums them).  swiglu=True: a is [M, 2K] = [gate | up] and the product
-    runs on silu(gate) * up."""
+    packed: pack_weight(w) of w [N, K].  out: bfloat16 or float32 [M, N], or float32
+    [groups, M, N]: K is then cut into that many groups whose partial products fill the planes of
+    out (the reader sums them).  gated=True: packed = pack_weight(w, gated=True) of a [2I, K] matrix
+    and out is [M, I] = silu(a gate^T) * (a up^T)."""
     _gpu(a, packed, out)
     groups = 1
     if out.dim() == 3:
         groups = out.shape[0]
         if out.dtype != torch.float32 or not out.is_contiguous():
             raise KernelError("gemv_mfma: partial outputs must be contiguous float32 [groups, M, N]")
-    M, N = out.shape[-2:]
-    if a.shape != (M, 2 * K if swiglu else K):
+    M = out.shape[-2]
+    N = out.shape[-1] * (2 if gated else 1)
+    if a.shape != (M, K):
         raise KernelError(f"gemv_mfma: shapes a={tuple(a.shape)} out={tuple(out.shape)} K={K} do not fit")
     if packed.numel() != ((N + 15) // 16) * ((K + 31) // 32) * 512 or not packed.is_contiguous():
         raise KernelError(f"gemv_mfma: the packed weights have {packed.numel()} elements, not those of a "
@@ -348,7 +356,7 @@ def gemv_mfma(a, packed, out, K, swiglu=False):
     if a.dtype != torch.bfloat16 or packed.dtype != torch.bfloat16:
         raise KernelError("gemv_mfma: operands must be bfloat16")
     _call("blm_gemv_mfma", a.data_ptr(), packed.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
-          out.stride(-2), 1 if swiglu else 0, groups, _stream())
+          out.stride(-2), 1 if gated else 0, groups, _stream())
     return out
 
 

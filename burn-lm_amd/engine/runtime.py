@@ -23,8 +23,8 @@ MFMA_SKINNY_MAX_ROWS = 16
 class LinearWeight:
     """A bound weight matrix [N, K] and, for bfloat16, its copy packed for the skinny product."""
 
-    def __init__(self, w, packed=None):
-        self.w, self.packed = w, packed
+    def __init__(self, w, packed=None, gated=False):
+        self.w, self.packed, self.gated = w, packed, gated
         self.shape, self.dtype = w.shape, w.dtype
 
 
@@ -45,13 +45,15 @@ class Runtime:
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
 
-    def weight(self, w):
+    def weight(self, w, gated=False):
         """Prepares a bound matrix for linear(): bfloat16 matrices get the packed copy that the
-        skinny product streams (it doubles their memory; the plain copy serves prefill)."""
+        skinny product streams (it doubles their memory; the plain copy serves prefill).
+        gated=True: w is [gate rows; up rows] of a gated feed-forward and will be used through
+        gated_linear(); its packed copy pairs each gate row with its up row."""
         w = w.contiguous()
         N, K = w.shape
-        if w.dtype == torch.bfloat16 and ops.gemv_mfma_supported(1, N, K):
-            return LinearWeight(w, ops.pack_weight(w))
+        if w.dtype == torch.bfloat16 and ops.gemv_mfma_supported(1, N, K) and (not gated or N % 16 == 0):
+            return LinearWeight(w, ops.pack_weight(w, gated=gated), gated)
         return LinearWeight(w)
 
     @staticmethod
@@ -73,7 +75,7 @@ class Runtime:
         them); it is used for narrow outputs in decode."""
         packed = None
         if isinstance(w, LinearWeight):
-            w, packed = w.w, w.packed
+            w, packed = w.w, (None if w.gated else w.packed)   # a gated copy has its rows re-ordered
         M, K = x.shape
         N = w.shape[0]
         out_dtype = out_dtype or self.dtype
@@ -101,21 +103,17 @@ class Runtime:
         # float32 logits from bfloat16 operands with many rows: own kernel (float accumulation)
         return ops.gemm_tiled(x, w, out)
 
-    def swiglu_linear(self, gate_up, w, partials=False):
-        """(silu(gate) * up) [M,K] @ w[N,K]^T for gate_up = [gate | up] of width 2K.  With few rows in
-        bfloat16 the gating is fused into the product's operand load; otherwise it runs as a kernel
-        of its own before the product."""
-        M = gate_up.shape[0]
-        N, K = w.shape
-        packed = w.packed if isinstance(w, LinearWeight) else None
-        if (packed is not None and gate_up.dtype == torch.bfloat16 and M <= MFMA_SKINNY_MAX_ROWS
-                and gate_up.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0):
-            groups = self.k_groups(N, K) if partials else 1
-            if groups > 1:
-                out = torch.empty(groups, M, N, dtype=torch.float32, device=gate_up.device)
-            else:
-                out = torch.empty(M, N, dtype=self.dtype, device=gate_up.device)
-            return ops.gemv_mfma(gate_up, packed, out, K, swiglu=True)
-        act = torch.empty(M, K, dtype=gate_up.dtype, device=gate_up.device)
-        ops.swiglu(gate_up, act)
-        return self.linear(act, w)
+    def gated_linear(self, x, w):
+        """silu(x gate^T) * (x up^T) for w = [gate rows; up rows] ([2I, K]) -> [M, I].  With few rows
+        in bfloat16 the gating is fused into the product (weight(w, gated=True) pairs the rows for
+        it); otherwise the product is followed by the gating kernel."""
+        M, K = x.shape
+        inner = w.shape[0] // 2
+        if (isinstance(w, LinearWeight) and w.packed is not None and w.gated and x.dtype == torch.bfloat16
+                and M <= MFMA_SKINNY_MAX_ROWS and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+            out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
+            return ops.gemv_mfma(x, w.packed, out, K, gated=True)
+        gu = self.linear(x, w.w if isinstance(w, LinearWeight) else w)
+        act = torch.empty(M, inner, dtype=gu.dtype, device=x.device)
+        ops.swiglu(gu, act)
+        return act

@@ -1,7 +1,8 @@
 """Dense SwiGLU feed-forward: ``(silu(x W1) * (x W3)) W2`` without bias
 (crates/burn-lm-llama/src/nn/fftn.rs:44-46; W1 = gate, W3 = up, W2 = down,
 nn/llama/import.rs:22-31).  Gate and up run as one product on the stacked weight; silu and the
-product are float32 in the kernel."""
+product are float32, in the product's own epilogue when few rows run (decode) and in a kernel of
+their own otherwise."""
 from __future__ import annotations
 
 import torch
@@ -24,10 +25,10 @@ class SwiGLU(FeedForward):
         g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = rt.weight(torch.cat([g, u], dim=0))
+        self.w_gate_up = rt.weight(torch.cat([g, u], dim=0), gated=True)
         self.w_down = rt.weight(tensors[self.names["down"]])
         self.inner = self.params["inner"]
 
     def forward(self, x, step):
         rt = self.rt
-        return rt.swiglu_linear(rt.linear(x, self.w_gate_up), self.w_down, partials=True)
+        return rt.linear(rt.gated_linear(x, self.w_gate_up), self.w_down, partials=True)

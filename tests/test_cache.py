@@ -58,10 +58,11 @@ def test_pages_follow_each_sequences_own_length():
 
 def test_layers_of_one_need_share_a_group_and_planes_are_their_own():
     c = make()
-    assert len(c.groups) == 1 and c.groups[0].storage.shape == (3, 2, 16, 2, 16, 8)
+    assert len(c.groups) == 1 and c.groups[0].storage.shape == (3, 2, 16, 2, 16 * 8)
     v0, v2 = c.views[0], c.views[2]
     assert isinstance(v0, KVView) and v0.k.data_ptr() != v2.k.data_ptr() and v0.k.data_ptr() != v0.v.data_ptr()
-    assert v0.store and v0.k.shape == (16, 2, 16, 8)
+    # key pages are [token][head_dim], value pages are kept transposed
+    assert v0.store and v0.k.shape == (16, 2, 16, 8) and v0.v.shape == (16, 2, 8, 16)
 
 
 def test_groups_with_different_needs_have_storage_and_pools_of_their_own():

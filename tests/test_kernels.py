@@ -377,16 +377,6 @@ def test_gemv_mfma(ops, out_dtype, M, N, K):
     got = out.double().cpu()
     err = ((got - want).abs() / (want.abs() + want.abs().mean())).max()
     assert float(err) <= (2e-5 if out_dtype == "float32" else 8e-3), f"error {float(err):.3g}"
-    # the SwiGLU gating fused into the operand load equals the gating kernel followed by the product
-    gu = (torch.randn(M, 2 * K, generator=g) * 2).bfloat16()
-    act = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
-    ops.swiglu(dev(gu), act)
-    plain = torch.empty(M, N, dtype=DT[out_dtype], device="cuda")
-    ops.gemv_mfma(act, Wp, plain, K)
-    fused = torch.empty(M, N, dtype=DT[out_dtype], device="cuda")
-    ops.gemv_mfma(dev(gu), Wp, fused, K, swiglu=True)
-    # the fused gating uses the fast exponential: a gated value may round to the neighbouring bfloat16
-    assert float((fused.double() - plain.double()).abs().max() / plain.double().abs().max()) <= 4e-3
     # rows of a wider buffer, and an output with a row stride
     wide = torch.randn(M, K + 24, generator=g).bfloat16()
     big = torch.zeros(M, N + 5, dtype=DT[out_dtype], device="cuda")
@@ -425,12 +415,23 @@ def test_gemv_mfma_partial_products_are_summed_by_the_norm(ops, M, N, K, groups)
     out2 = torch.empty(2, N, dtype=torch.bfloat16, device="cuda")
     ops.add_rmsnorm(hd2, planes, dev(gamma), 1e-5, out2, rows=dev(rows), write_h=False)
     assert torch.equal(out2.cpu(), out.cpu()[rows.long()]) and torch.equal(hd2.cpu(), h)
-    # the fused gating with groups
-    gu = torch.randn(M, 2 * K, generator=g).bfloat16()
-    act = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
-    ops.swiglu(dev(gu), act)
-    ops.gemv_mfma(dev(gu), Wp, planes, K, swiglu=True)
-    close(planes.double().sum(0), act.double().cpu() @ W.double().T, 4e-3)
+
+
+@pytest.mark.parametrize("M,I,K", [(8, 176, 64), (3, 384, 144), (16, 8, 520), (5, 1000, 2048), (1, 64, 4104)])
+def test_gemv_mfma_gated(ops, M, I, K):
+    """The SwiGLU gating in the epilogue of the product that computes gate and up: the packed copy pairs
+    every 8 gate rows with their 8 up rows, the result is silu(x gate^T) * (x up^T)."""
+    g = torch.Generator().manual_seed(18)
+    A = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(2 * I, K, generator=g) * (2.0 / K ** 0.5)).bfloat16()
+    Wp = ops.pack_weight(dev(W), gated=True)
+    out = torch.full((M, I), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.gemv_mfma(dev(A), Wp, out, K, gated=True)
+    gate, up = A.double() @ W[:I].double().T, A.double() @ W[I:].double().T
+    want = torch.nn.functional.silu(gate) * up
+    close(out, want, EPS["bfloat16"] * 1.5)
+    # gate and up swapped, or pairs shifted, would show
+    assert float((torch.nn.functional.silu(up) * gate - want).abs().max() / want.abs().max()) > 0.1
 
 
 def test_gemv_mfma_refuses_what_it_cannot_do(ops):
