@@ -96,6 +96,12 @@ class Runtime:
             return ops.gemv_mfma(x, packed, out, K)
         if out is None:
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+        if packed is not None and aligned and out_dtype == torch.float32 and M <= 4 * MFMA_SKINNY_MAX_ROWS:
+            # float32 results (logits) for a few dozen rows: the skinny product 16 rows at a time; the
+            # weights stream once per 16 rows, which still beats the plain tiled kernel by far
+            for r in range(0, M, MFMA_SKINNY_MAX_ROWS):
+                ops.gemv_mfma(x[r:r + MFMA_SKINNY_MAX_ROWS], packed, out[r:r + MFMA_SKINNY_MAX_ROWS], K)
+            return out
         if M <= SKINNY_MAX_ROWS and aligned:
             return ops.gemv_skinny(x, w, out)
         if out_dtype == torch.bfloat16:
