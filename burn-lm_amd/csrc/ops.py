@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 _lib = None
 _lock = threading.Lock()
 
@@ -46,6 +46,10 @@ _SIGNATURES = {
     "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
+    "blm_gemv_qkv_rope_supported": [_c_int, _c_int, _c_int],
+    "blm_gemv_qkv_rope": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                          _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                          _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
 }
@@ -358,6 +362,38 @@ def gemv_mfma(a, packed, out, K, gated=False):
     _call("blm_gemv_mfma", a.data_ptr(), packed.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
           out.stride(-2), 1 if gated else 0, groups, _stream())
     return out
+
+
+def gemv_qkv_rope_supported(M, K, hd):
+    return bool(library().blm_gemv_qkv_rope_supported(int(M), int(K), int(hd)))
+
+
+def gemv_qkv_rope(x, packed, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,
+                  nh, nkv, hd, pairing, write_kv=True):
+    """Decode: x [M<=16, K] @ W_qkv^T on the matrix cores, rotary encoding of q and k on the float
+    results, q into qkv_out[:, :nh*hd], k and v into their cache pages, all in one kernel.
+    packed: pack_weight of W_qkv [(nh + 2 nkv) * hd, K]."""
+    _gpu(x, packed, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache)
+    M, K = x.shape
+    N = (nh + 2 * nkv) * hd
+    if x.dtype != torch.bfloat16 or packed.dtype != torch.bfloat16 or qkv_out.dtype != torch.bfloat16:
+        raise KernelError("gemv_qkv_rope: operands must be bfloat16")
+    if packed.numel() != (N // 16) * ((K + 31) // 32) * 512 or not packed.is_contiguous():
+        raise KernelError(f"gemv_qkv_rope: the packed weights are not those of a [{N}, {K}] matrix")
+    if qkv_out.shape[0] != M or qkv_out.stride(1) != 1 or qkv_out.shape[1] < nh * hd or x.stride(1) != 1:
+        raise KernelError("gemv_qkv_rope: qkv_out must be [M, >= heads*head_dim] with unit stride along rows")
+    _i32("positions", positions, M); _i32("token_seq", token_seq, M); _i32("block_table", block_table)
+    if cos_sin.dtype != torch.float32 or cos_sin.shape[1:] != (hd // 2, 2) or not cos_sin.is_contiguous():
+        raise KernelError("gemv_qkv_rope: cos_sin must be contiguous float32 [positions, head_dim/2, 2]")
+    if kcache.dtype != torch.bfloat16:
+        raise KernelError("gemv_qkv_rope: the cache must be bfloat16")
+    _contig("kcache", kcache); _contig("vcache", vcache)
+    _check_planes("gemv_qkv_rope", kcache, vcache, nkv, page_size, hd)
+    _call("blm_gemv_qkv_rope", x.data_ptr(), packed.data_ptr(), qkv_out.data_ptr(), positions.data_ptr(),
+          token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], cos_sin.data_ptr(), kcache.data_ptr(),
+          vcache.data_ptr(), page_size, M, K, x.stride(0), qkv_out.stride(0), nh, nkv, hd, pairing,
+          1 if write_kv else 0, _stream())
+    return qkv_out
 
 
 def argmax(logits, out=None):

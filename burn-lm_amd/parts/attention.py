@@ -53,8 +53,7 @@ class Attention(Mixer):
     def forward(self, x, step, view):
         rt = self.rt
         nh, nkv, hd = self.heads, self.kv_heads, self.head_dim
-        qkv = rt.linear(x, self.w_qkv)
-        self.position.encode_and_store(qkv, step, view, nh, nkv, hd, store=view.store)
+        qkv = self.position.project_encode_store(x, self.w_qkv, step, view, nh, nkv, hd)
         out = torch.empty(x.shape[0], nh * hd, dtype=rt.dtype, device=x.device)
         table = view.block_table(step)
         aligned = qkv.shape[1] % 8 == 0

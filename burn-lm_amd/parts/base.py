@@ -18,7 +18,9 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
   in the layer order (``KVView``, ``StateView`` or ``None``).
 * ``FeedForward.forward(x, step) -> delta``.
 * ``PositionEncoding.prepare(n_positions, rt)`` and, for encodings that act on queries and keys,
-  ``encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store)``.
+  ``encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store)``; the attention mixer calls
+  ``project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)``, whose default is the
+  projection followed by ``encode_and_store`` and which an encoding may fuse.
 * ``Block.forward(h, delta, step, view) -> delta``: runs its parts; the returned delta has not
   been added to ``h`` yet (the next norm adds it, in float32).
 """
@@ -98,6 +100,14 @@ class FeedForward(Part):
 class PositionEncoding(Part):
     def prepare(self, n_positions: int, rt) -> None:
         pass
+
+    def project_encode_store(self, x, w_qkv, step, view, heads, kv_heads, head_dim):
+        """x @ w_qkv^T, then encode q and k by position and store k, v (unless view.store is
+        False).  Returns the [tokens, (heads + 2 kv_heads) * head_dim] buffer whose first
+        heads * head_dim columns are the encoded queries.  A subclass may fuse the steps."""
+        qkv = self.rt.linear(x, w_qkv)
+        self.encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store=view.store)
+        return qkv
 
 
 class Block:

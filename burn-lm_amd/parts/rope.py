@@ -62,3 +62,20 @@ class RotaryEncoding(PositionEncoding):
         self.rt.ops.rope_kv_write(qkv, step.positions, step.token_seq, view.block_table(step), self.table,
                                   view.k, view.v, view.page_size, heads, kv_heads, head_dim, self.pairing,
                                   write_kv=store)
+
+    def project_encode_store(self, x, w_qkv, step, view, heads, kv_heads, head_dim):
+        """Decode (few rows, bfloat16, packed weights): projection, rotation and cache write in one
+        kernel, the rotation applied to the float accumulators.  Otherwise the three steps apart."""
+        rt = self.rt
+        packed = getattr(w_qkv, "packed", None)
+        M, K = x.shape
+        if (packed is not None and not getattr(w_qkv, "gated", False) and x.dtype == torch.bfloat16
+                and rt.ops.gemv_qkv_rope_supported(M, K, head_dim) and x.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0 and view.k.dtype == torch.bfloat16):
+            if step.max_position >= self.n_positions:
+                raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
+            qkv = torch.empty(M, (heads + 2 * kv_heads) * head_dim, dtype=torch.bfloat16, device=x.device)
+            return rt.ops.gemv_qkv_rope(x, packed, qkv, step.positions, step.token_seq, view.block_table(step),
+                                        self.table, view.k, view.v, view.page_size, heads, kv_heads, head_dim,
+                                        self.pairing, write_kv=view.store)
+        return super().project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)

@@ -500,3 +500,57 @@ def test_sample_top_p_keeps_the_nucleus_only(ops):
     big[3, 40000] = 30.0
     out = ops.sample(dev(big), dev(torch.full((5,), 0.5)), 0.8, 0.9).cpu()
     assert int(out[3]) == 40000 and all(0 <= int(t) < 50257 for t in out)
+
+
+@pytest.mark.parametrize("pairing", ["interleaved", "half"])
+@pytest.mark.parametrize("M,K,nh,nkv,hd", [(8, 2048, 4, 2, 64), (5, 264, 3, 1, 32), (16, 3072, 2, 2, 128), (1, 64, 6, 3, 64)])
+def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
+    """The fused decode projection: equals the product, the rotation of its float result and the
+    cache write done one after the other (in float64), for both pairings, with a padding row and
+    scrambled pages; nothing else in the cache is touched."""
+    from burn_lm_amd.parts.rope import PAIRING, rope_frequencies
+    g = torch.Generator().manual_seed(19)
+    page, n_pages = 64, 16
+    N = (nh + 2 * nkv) * hd
+    x = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(N, K, generator=g) / K ** 0.5).bfloat16()
+    positions = torch.tensor([(37 * i + 5) % 250 for i in range(M)], dtype=torch.int32)
+    token_seq = torch.arange(M, dtype=torch.int32)
+    if M > 2:
+        token_seq[2] = -1                      # a padding row: no cache write
+        token_seq[3:] -= 1
+    n_seq = int(token_seq.max()) + 1
+    perm = torch.randperm(n_pages * 4, generator=g)[: n_seq * 4].reshape(n_seq, 4).to(torch.int32)
+    freqs = torch.from_numpy(rope_frequencies(hd, 500000.0, (8, 1, 4, 32)))
+    ang = torch.arange(256).double()[:, None] * freqs[None, :]
+    cs = torch.stack([ang.cos(), ang.sin()], -1).float()
+    k = torch.full((n_pages * 4, nkv, page, hd), 99.0).bfloat16()
+    v = torch.full((n_pages * 4, nkv, hd, page), 99.0).bfloat16()
+    kd, vd = dev(k), dev(v)
+    out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.gemv_qkv_rope(dev(x), ops.pack_weight(dev(W)), out, dev(positions), dev(token_seq), dev(perm), dev(cs), kd, vd,
+                      page, nh, nkv, hd, PAIRING[pairing])
+    qkv = x.double() @ W.double().T
+    q_ref = _rope_ref(qkv[:, : nh * hd].reshape(M, nh, hd), positions, freqs, pairing)
+    k_ref = _rope_ref(qkv[:, nh * hd: (nh + nkv) * hd].reshape(M, nkv, hd), positions, freqs, pairing)
+    v_ref = qkv[:, (nh + nkv) * hd:].reshape(M, nkv, hd)
+    close(out[:, : nh * hd].reshape(M, nh, hd), q_ref, EPS["bfloat16"] * 1.5)
+    assert bool((out[:, nh * hd:] == 7).all()), "only the queries are written to the buffer"
+    kc, vc = kd.cpu().double(), vd.cpu().double()
+    written = torch.zeros(n_pages * 4, page, dtype=torch.bool)
+    for t in range(M):
+        b = int(token_seq[t])
+        if b < 0:
+            continue
+        p = int(positions[t]); pg = int(perm[b, p // page])
+        written[pg, p % page] = True
+        close(kc[pg, :, p % page], k_ref[t], EPS["bfloat16"] * 1.5)
+        close(vc[pg, :, :, p % page], v_ref[t], EPS["bfloat16"] * 1.5)
+    untouched = ~written[:, None, :, None].expand(n_pages * 4, nkv, page, hd)
+    assert bool((kc[untouched] == 99).all()) and bool((vc.transpose(2, 3)[untouched] == 99).all())
+    # a place that reads another's cache: queries only
+    kd2 = dev(k)
+    out2 = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.gemv_qkv_rope(dev(x), ops.pack_weight(dev(W)), out2, dev(positions), dev(token_seq), dev(perm), dev(cs), kd2, dev(v),
+                      page, nh, nkv, hd, PAIRING[pairing], write_kv=False)
+    assert torch.equal(out2.cpu(), out.cpu()) and bool((kd2.cpu() == 99).all())
