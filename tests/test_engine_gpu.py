@@ -270,3 +270,60 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
         got = eng.step([(s, [r[c + k]], [0]) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
         for i in range(3):
             assert rel_err(got[i], want[i][cut[i] + k]) <= TOL["bfloat16"], f"request {i}, decode step {k}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_with_library_products_inside(folders, dtype):
+    """More than 16 sequences per decode step: the layer products are the library's, recorded into
+    the graph.  Every replay is checked against the eager engine, with eager prefills and
+    synchronisations between replays."""
+    cfg, seed = TINIES["B"]
+    g = load(folders["B"], dtype, max_tokens=8192, max_seqs=32)
+    e = load(folders["B"], dtype, max_tokens=8192, max_seqs=32, graphs=False)
+    n = 20
+    prompts = [random_tokens(300 + i, cfg["vocab_size"], 3 + (7 * i) % 40) for i in range(n)]
+    sg = [g.open() for _ in range(n)]
+    se = [e.open() for _ in range(n)]
+    a = g.step([(s, p, [len(p) - 1]) for s, p in zip(sg, prompts)])
+    b = e.step([(s, p, [len(p) - 1]) for s, p in zip(se, prompts)])
+    toks = [int(t) for t in b.argmax(1)]
+    tol = 2e-6 if dtype == "float32" else 2e-2
+    live = list(range(n))
+    for k in range(40):
+        a = g.step([(sg[i], [toks[i]], [0]) for i in live])
+        b = e.step([(se[i], [toks[i]], [0]) for i in live])
+        assert rel_err(a.double().cpu().numpy(), b.double().cpu().numpy()) <= tol, f"decode step {k}"
+        for row, i in enumerate(live):
+            toks[i] = int(b[row].argmax())
+        if k % 9 == 4:          # eager work between replays, and the batch shrinks within its bucket
+            x = g.open(); g.step([(x, prompts[0], [])]); g.close(x)
+            y = e.open(); e.step([(y, prompts[0], [])]); e.close(y)
+            i = live.pop(3)
+            g.close(sg[i]); e.close(se[i])
+            torch.cuda.synchronize()
+    assert g.graphs.replays >= 35 and any(k[0] == 24 for k in g.graphs.captured)
+
+
+def test_head_size_that_is_no_power_of_two_and_odd_counts(tmp_path):
+    """head_dim 48 (a step of 16 that the matrix-core attention does not take: the generic kernel
+    runs), 5 heads without grouping, an odd vocabulary: whole, tail and batch against plain."""
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=120, intermediate_size=200, num_hidden_layers=2,
+               num_attention_heads=5, num_key_value_heads=5, head_dim=48, vocab_size=257, max_position_embeddings=256,
+               rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)
+    folder = make_folder(tmp_path / "m48", cfg, seed=9)
+    plain = P.load_model_folder(folder)
+    reqs = [random_tokens(400 + i, 257, n) for i, n in enumerate([70, 5, 130])]
+    want = [P.transformer_forward([r], plain)[0] for r in reqs]
+    for dtype in ("float32", "bfloat16"):
+        eng = load(folder, dtype, max_tokens=1024)
+        slots = [eng.open() for _ in reqs]
+        cut = [len(r) - 4 for r in reqs]
+        got = eng.step([(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
+        o = 0
+        for r, c, w in zip(reqs, cut, want):
+            assert rel_err(got[o:o + c], w[:c]) <= TOL[dtype], dtype
+            o += c
+        for k in range(4):
+            got = eng.step([(s, [r[c + k]], [0]) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
+            for i in range(3):
+                assert rel_err(got[i], want[i][cut[i] + k]) <= TOL[dtype], f"{dtype} request {i} decode {k}"

@@ -169,3 +169,96 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype, tol):
                 eng.close(slots[1])
         eng.close(slots[0]); eng.close(slots[2])
     assert eng.cache.pages_in_use() == 0
+
+
+def test_a_windowed_attention_layer_beside_a_full_one(tmp_path):
+    """Two attention layers of one model with different needs: the first keeps a window of 40 keys
+    (its group gives pages back as they fall out of the window), the second all keys.  Prompts longer
+    than the window, then decoding across the window's edge and page edges, against the plain
+    attention with the window's mask; the page pools of the two groups are checked as well."""
+    import math as _m
+    from burn_lm_amd import registry
+    from burn_lm_amd.engine.loading import load_engine
+    from burn_lm_amd.models.plan import LayerPlan, ModelPlan, Place
+    from burn_lm_amd.parts.base import PartSpec
+    from burn_lm_amd.weights import safetensors_io as st
+    W = 40
+    c = dict(architectures=["ToyWindowLM"], width=64, inner=96, heads=4, kv_heads=2, head_dim=16, vocab=101, eps=1e-5,
+             theta=10000.0, max_positions=512)
+
+    def plan(cfg, names=None):
+        D = cfg["width"]
+        norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=cfg["eps"]), dict(weight=n))
+        layer = lambda i, window: LayerPlan(
+            "pre_norm",
+            PartSpec("attention", dict(width=D, heads=cfg["heads"], kv_heads=cfg["kv_heads"], head_dim=cfg["head_dim"],
+                                       scale=1 / _m.sqrt(cfg["head_dim"]), window=window),
+                     dict(q=f"l{i}.q", k=f"l{i}.k", v=f"l{i}.v", o=f"l{i}.o")),
+            PartSpec("swiglu", dict(width=D, inner=cfg["inner"]), dict(gate=f"l{i}.gate", up=f"l{i}.up", down=f"l{i}.down")),
+            norm(f"l{i}.n1"), norm(f"l{i}.n2"), position="rope")
+        return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
+                         embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         layers=[layer(0, W), layer(1, 0)], order=[Place(0), Place(1)], final_norm=norm("norm"),
+                         head=PartSpec("linear", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         positions={"rope": PartSpec("rope", dict(head_dim=cfg["head_dim"], theta=cfg["theta"],
+                                                                  pairing="interleaved", scaling=None))})
+
+    registry.register_architecture(registry.Architecture("ToyWindowLM", read_config=lambda d: d, plan=plan))
+    g = torch.Generator().manual_seed(21)
+    m = lambda *s: (torch.randn(*s, generator=g) * 0.2).bfloat16()
+    n = lambda: (1 + 0.1 * torch.randn(c["width"], generator=g)).bfloat16()
+    D, I, hd = c["width"], c["inner"], c["head_dim"]
+    t = {"emb": m(c["vocab"], D), "norm": n()}
+    for i in (0, 1):
+        t.update({f"l{i}.q": m(c["heads"] * hd, D), f"l{i}.k": m(c["kv_heads"] * hd, D), f"l{i}.v": m(c["kv_heads"] * hd, D),
+                  f"l{i}.o": m(D, c["heads"] * hd), f"l{i}.gate": m(I, D), f"l{i}.up": m(I, D), f"l{i}.down": m(D, I),
+                  f"l{i}.n1": n(), f"l{i}.n2": n()})
+    json.dump(c, open(tmp_path / "config.json", "w"))
+    st.write_file(str(tmp_path / "model.safetensors"), t.items())
+    w = {k: v.double().numpy() for k, v in t.items()}
+    freqs = P.rope_base_frequencies(hd, c["theta"])
+
+    def plain(tokens):
+        T = len(tokens)
+        h = w["emb"][np.asarray(tokens)][None]
+        pos = np.arange(T)
+        for i, window in ((0, W), (1, 0)):
+            x = P.rms_norm(h, w[f"l{i}.n1"], c["eps"])
+            q = (x @ w[f"l{i}.q"].T).reshape(1, T, c["heads"], hd).swapaxes(1, 2)
+            k = (x @ w[f"l{i}.k"].T).reshape(1, T, c["kv_heads"], hd).swapaxes(1, 2)
+            v = (x @ w[f"l{i}.v"].T).reshape(1, T, c["kv_heads"], hd).swapaxes(1, 2)
+            hidden = P.hidden_mask(T, T) if T > 1 else np.zeros((1, 1), dtype=bool)
+            if window:
+                hidden = hidden | (pos[:, None] - pos[None, :] >= window)   # key j is seen iff p - j < window
+            o = P.scaled_attention(P.rope_interleaved(q, pos, freqs), P.rope_interleaved(k, pos, freqs), v, hidden)
+            h = h + o.swapaxes(1, 2).reshape(1, T, -1) @ w[f"l{i}.o"].T
+            h = h + P.swiglu_feed_forward(P.rms_norm(h, w[f"l{i}.n2"], c["eps"]), w[f"l{i}.gate"], w[f"l{i}.up"], w[f"l{i}.down"])
+        return (P.rms_norm(h, w["norm"], c["eps"]) @ w["emb"].T)[0]
+
+    rng = np.random.default_rng(5)
+    reqs = [[int(x) for x in rng.integers(0, 101, L)] for L in (150, 30, 75)]
+    want = [plain(r) for r in reqs]
+    err = lambda got, ww: float(np.abs(got.double().cpu().numpy() - ww).max() / np.abs(ww).max())
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 3e-2)):
+        eng = load_engine(str(tmp_path), dtype=dtype, max_tokens=1024, max_seqs=4)
+        assert len(eng.cache.groups) == 2 and {g_.need.window for g_ in eng.cache.groups} == {0, W}
+        slots = [eng.open() for _ in reqs]
+        cut = [len(r) - 20 for r in reqs]
+        got = eng.step([(s, r[:k], list(range(k))) for s, r, k in zip(slots, reqs, cut)])
+        o = 0
+        for r, k, ww in zip(reqs, cut, want):
+            assert err(got[o:o + k], ww[:k]) <= tol, f"{dtype} prompt"
+            o += k
+        for j in range(20):
+            got = eng.step([(s, [r[k + j]], [0]) for s, r, k in zip(slots, reqs, cut)])
+            for i in range(3):
+                assert err(got[i], want[i][cut[i] + j]) <= tol, f"{dtype} request {i} decode {j}"
+        win = next(g_ for g_ in eng.cache.groups if g_.need.window == W)
+        full = next(g_ for g_ in eng.cache.groups if g_.need.window == 0)
+        # request 0 holds 150 tokens: 3 pages in the full group; in the windowed group only the pages
+        # that still hold keys 111.. (pages 1 and 2), page 0 went back to the pool
+        assert [p >= 0 for p in win.tables[slots[0]]] == [False, True, True]
+        assert all(p >= 0 for p in full.tables[slots[0]]) and len(full.tables[slots[0]]) == 3
+        for s in slots:
+            eng.close(s)
+        assert eng.cache.pages_in_use() == 0
