@@ -327,3 +327,101 @@ def test_head_size_that_is_no_power_of_two_and_odd_counts(tmp_path):
             got = eng.step([(s, [r[c + k]], [0]) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
             for i in range(3):
                 assert rel_err(got[i], want[i][cut[i] + k]) <= TOL[dtype], f"{dtype} request {i} decode {k}"
+
+
+def _write_folder(path, cfg, tensors):
+    from burn_lm_amd.weights import safetensors_io as st
+    os.makedirs(path, exist_ok=True)
+    json.dump(cfg, open(os.path.join(path, "config.json"), "w"))
+    st.write_file(os.path.join(path, "model.safetensors"), tensors.items())
+    return str(path)
+
+
+def test_the_references_whole_model_vector_in_32_bit(tmp_path):
+    """crates/burn-lm-llama/src/nn/transformer.rs:299-349: vocabulary 8, 2 layers, width 8, inner 16,
+    2 heads on 1 KV head (head_dim 4), every tensor arange(n)*5/n in the reference's [d_in, d_out]
+    order, token ids [[0, 1], [2, 3]].  The engine reads the same numbers as a Meta-named 32-bit
+    checkpoint ([d_out, d_in], so each matrix transposed) and must give the reference's logits."""
+    r = lambda *s: torch.arange(int(np.prod(s)), dtype=torch.float64).mul(5.0 / int(np.prod(s))).reshape(*s)
+    lin = lambda d_in, d_out: r(d_in, d_out).T.contiguous().float()
+    t = {"tok_embeddings.weight": r(8, 8).float(), "norm.weight": r(8).float(), "output.weight": lin(8, 8)}
+    for i in range(2):
+        p = f"layers.{i}."
+        t.update({p + "attention.wq.weight": lin(8, 8), p + "attention.wk.weight": lin(8, 4),
+                  p + "attention.wv.weight": lin(8, 4), p + "attention.wo.weight": lin(8, 8),
+                  p + "feed_forward.w1.weight": lin(8, 16), p + "feed_forward.w3.weight": lin(8, 16),
+                  p + "feed_forward.w2.weight": lin(16, 8), p + "attention_norm.weight": r(8).float(),
+                  p + "ffn_norm.weight": r(8).float()})
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=8, intermediate_size=16, num_hidden_layers=2,
+               num_attention_heads=2, num_key_value_heads=1, vocab_size=8, rms_norm_eps=1e-5, rope_theta=10000.0,
+               tie_word_embeddings=False, max_position_embeddings=64)
+    want = np.array([[[56.37573, 57.77283, 59.169933, 60.567043, 61.964146, 63.361248, 64.758354, 66.15546],
+                      [56.374626, 57.77171, 59.168793, 60.56588, 61.962963, 63.360046, 64.75713, 66.15422]],
+                     [[56.374252, 57.771328, 59.168407, 60.565487, 61.962566, 63.359642, 64.75672, 66.1538],
+                      [56.37408, 57.771156, 59.168232, 60.565304, 61.96238, 63.359455, 64.75653, 66.15361]]])
+    eng = load(_write_folder(tmp_path / "ref", cfg, t), "float32")
+    a, b = eng.open(), eng.open()
+    got = eng.step([(a, [0, 1], [0, 1]), (b, [2, 3], [0, 1])]).double().cpu().numpy().reshape(2, 2, 8)
+    np.testing.assert_allclose(got, want, rtol=2e-6)
+    # the same, token by token from the cache
+    eng.close(a); eng.close(b)
+    a = eng.open()
+    one = [eng.step([(a, [tok], [0])]).double().cpu().numpy()[0] for tok in (0, 1)]
+    np.testing.assert_allclose(np.stack(one), want[0], rtol=2e-6)
+
+
+def test_meta_names_equal_hugging_face_names_and_a_tied_head_equals_a_copied_one(folders, tmp_path):
+    """The same model under the two checkpoint layouts (import.rs:20-88): Meta names with the q/k rows
+    in adjacent-pair order (import.rs:94-127) against Hugging Face names with half-split rows; and
+    tie_word_embeddings against an lm_head that is a copy of the table."""
+    from burn_lm_amd.models.llama import HF_NAMES, META_NAMES
+    from burn_lm_amd.weights import safetensors_io as st
+    cfg = dict(TINY_A)
+    f = st.open_folder(folders["A"])
+    hf = {name: file.tensor(name).clone() for name, file in f.items()}
+    meta = {}
+    for name, w in hf.items():
+        new = name.replace(HF_NAMES["embedding"], META_NAMES["embedding"]).replace(HF_NAMES["final_norm"], META_NAMES["final_norm"])
+        new = new.replace("model.layers.", "layers.")
+        for key in ("q", "k", "v", "o", "gate", "up", "down", "mixer_norm", "ffn_norm"):
+            new = new.replace(HF_NAMES[key], META_NAMES[key])
+        if name.endswith(HF_NAMES["q"]) or name.endswith(HF_NAMES["k"]):
+            heads = cfg["num_attention_heads"] if name.endswith(HF_NAMES["q"]) else cfg["num_key_value_heads"]
+            w = torch.from_numpy(P.permute_hf_rows(w.float().numpy(), heads).copy()).to(w.dtype)
+        meta[new] = w
+    assert "tok_embeddings.weight" in meta and "layers.1.attention.wq.weight" in meta
+    untied = dict(hf); untied["lm_head.weight"] = hf[HF_NAMES["embedding"]].clone()
+    toks = [random_tokens(500 + i, cfg["vocab_size"], n) for i, n in enumerate([40, 9])]
+    outs = {}
+    for key, c, t in (("hf", cfg, hf), ("meta", cfg, meta), ("untied", dict(cfg, tie_word_embeddings=False), untied)):
+        eng = load(_write_folder(tmp_path / key, c, t), "float32")
+        slots = [eng.open() for _ in toks]
+        outs[key] = eng.step([(s, tk, list(range(len(tk)))) for s, tk in zip(slots, toks)]).double().cpu().numpy()
+    assert rel_err(outs["meta"], outs["hf"]) <= 2e-6
+    assert np.array_equal(outs["untied"], outs["hf"])
+
+
+def test_sampled_tokens_follow_the_plain_probabilities(folders):
+    """Prompts of 1, 7, 20 and 33 tokens, 12 tokens each at temperature 0.8 and top-p 0.9 in 32-bit:
+    every token the engine draws lies in the plain implementation's nucleus, and its interval of
+    the plain cumulative distribution (kept tokens in index order) holds the draw's uniform number."""
+    from burn_lm_amd.sampling.sampler import uniform
+    from burn_lm_amd.server import InferenceServer
+    cfg, seed = TINIES["B"]
+    plain = P.load_model_folder(folders["B"])
+    prompts = [random_tokens(80 + i, cfg["vocab_size"], n) for i, n in enumerate([1, 7, 20, 33])]
+    server = InferenceServer(folders["B"], dtype="float32", batch_size=4)
+    server.config.update(max_seq_len=128, sample_len=12, temperature=0.8, top_p=0.9, seed=11)
+    results, _ = server.generate(prompts, stop_ids=[])
+    for i, res in enumerate(results):
+        seq = list(prompts[i])
+        assert len(res.tokens) == 12
+        for n, tok in enumerate(res.tokens):
+            probs = P.temperature_softmax(P.transformer_forward([seq], plain)[0][-1], 0.8)
+            kept = sorted(P.top_p_keep(probs, 0.9))
+            assert tok in kept, f"request {i} token {n}"
+            cdf = np.cumsum(probs[kept]) / probs[kept].sum()
+            k = kept.index(tok)
+            u = uniform(11, i, n)
+            assert (cdf[k - 1] if k else 0.0) - 1e-4 <= u <= cdf[k] + 1e-4, f"request {i} token {n}"
+            seq.append(tok)
