@@ -1,5 +1,6 @@
-// Skinny matrix product for decode on the matrix cores: C[M<=16, N] = A[M, K] * W[N, K]^T, bf16
-// operands, float accumulation, bf16 or float output.
+// Skinny matrix product for decode on the matrix cores: C[M<=64, N] = A[M, K] * W[N, K]^T, bf16
+// operands, float accumulation, bf16 or float output.  Up to 16 rows run gemv_mfma_kernel, 17 to 64
+// rows gemv_mfma_rows_kernel (two to four row tiles against every weight fragment).
 //
 // The weight matrix is streamed exactly once, from a copy packed in the order the MFMA wants it:
 // for the 16x16x32 instruction the weights are the B operand, lane l of a wavefront holding
@@ -120,6 +121,101 @@ __global__ void __launch_bounds__(MAXT)
   }
 }
 
+// 17..64 rows: MT row tiles of 16.  A wavefront keeps the activations of all MT tiles for its 8
+// k-steps in registers (MT * 8 fragments) and runs MT MFMAs per weight fragment, so the weights
+// still stream once.  Blocks have up to 8 wavefronts, so one K-group spans at most 2048.  The
+// weights of the block's next column tile are requested before the current tile is multiplied and
+// reduced (and the first tile's before the activations), so the memory pipeline never idles while
+// the block synchronises.
+#define ROWS_KSTEPS 8
+template <int MT, typename TC>
+__global__ void __launch_bounds__(512)
+    gemv_mfma_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wp, TC* __restrict__ C, int M, int N,
+                          int K, int lda, int ldc, int n_tiles, int k_steps, int c_mode, int steps_per_group) {
+  constexpr int KSTEPS = ROWS_KSTEPS;
+  extern __shared__ float red[];  // [waves][MT][256]
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int n_waves = blockDim.x / BLM_WAVE;
+  const int row = lane & 15, kg = lane >> 4;
+  const int group_begin = blockIdx.y * steps_per_group;
+  const int group_end = min(k_steps, group_begin + steps_per_group);
+  const int step0 = group_begin + wave * KSTEPS;
+  const int kbase = step0 * 32 + kg * 8;
+  C += (size_t)blockIdx.y * M * ldc;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+
+  // weight fragment s of a tile, with the k-step clamped into the matrix (the activations are zero there)
+  const bf16* wbase = Wp + (size_t)lane * 8;
+  int woff[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) woff[s] = (step0 + s < k_steps ? step0 + s : k_steps - 1) * 512;
+
+  uint4 w[KSTEPS], wn[KSTEPS];
+  {
+    const bf16* wt = wbase + (size_t)blockIdx.x * k_steps * 512;   // gridDim.x <= n_tiles
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) w[s] = ld16(wt + woff[s]);
+  }
+  uint4 a[MT][KSTEPS];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + row;
+    const bf16* ap = A + (size_t)(m < M ? m : M - 1) * lda;   // rows >= M read a real row and are zeroed
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int k = kbase + s * 32;
+      const uint4 v = ld16(ap + (k < K ? k : K - 8));
+      a[mt][s] = (m < M && k < K && step0 + s < group_end) ? v : zero;
+    }
+  }
+
+  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    {
+      const int next = tile + (int)gridDim.x < n_tiles ? tile + (int)gridDim.x : tile;   // the last round re-reads its own
+      const bf16* wt = wbase + (size_t)next * k_steps * 512;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) wn[s] = ld16(wt + woff[s]);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // the next tile's loads are issued before this tile's first MFMA
+    f32x4_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[mt][s]),
+                                                          __builtin_bit_cast(bf16x8_t, w[s]), acc[mt], 0, 0, 0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[(wave * MT + mt) * 256 + r * 64 + lane] = acc[mt][r];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
+      const int mt = idx >> 8, i = idx & 255;
+      const int r = i >> 6, l2 = i & 63, col = l2 & 15;
+      const int m = mt * 16 + (l2 >> 4) * 4 + r;
+      if (c_mode == 0) {
+        float s = 0.f;
+        for (int w2 = 0; w2 < n_waves; ++w2) s += red[(w2 * MT + mt) * 256 + i];
+        const int nn = tile * 16 + col;
+        if (m < M && nn < N) C[(size_t)m * ldc + nn] = from_float<TC>(s);
+      } else if (col < 8) {
+        float g = 0.f, u = 0.f;
+        for (int w2 = 0; w2 < n_waves; ++w2) {
+          g += red[(w2 * MT + mt) * 256 + i];
+          u += red[(w2 * MT + mt) * 256 + i + 8];
+        }
+        const int nn = tile * 8 + col;
+        if (m < M && nn < N / 2) C[(size_t)m * ldc + nn] = from_float<TC>(g / (1.0f + expf(-g)) * u);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) w[s] = wn[s];
+  }
+}
+
 // How K is cut: k-steps of 32 per wavefront and wavefronts per block; 0 if K is out of range.
 //   K <= 512: 4 steps, <= 4 wavefronts;  K <= 4096: 16 steps, <= 8 wavefronts (512 threads);
 //   K <= 8192: 32 steps, <= 8 wavefronts (512 threads);  K <= 16384: 32 steps, <= 16 wavefronts
@@ -131,9 +227,15 @@ static int plan_k(int K, int* ksteps) {
   return 0;
 }
 
+// The largest K that one K-group may span for M rows (more rows leave fewer registers per k-step).
+extern "C" int blm_gemv_mfma_group_limit(int M) {
+  if (M < 1 || M > 64) return 0;
+  return M <= 16 ? 16384 : 2048;
+}
+
+// Whether the product runs with all of K in one group.
 extern "C" int blm_gemv_mfma_supported(int M, int N, int K) {
-  int ks;
-  return (M >= 1 && M <= 16 && N >= 1 && K >= 8 && K % 8 == 0 && plan_k(K, &ks) > 0) ? 1 : 0;
+  return (N >= 1 && K >= 8 && K % 8 == 0 && K <= blm_gemv_mfma_group_limit(M)) ? 1 : 0;
 }
 
 template <typename TC>
@@ -142,6 +244,24 @@ static int launch_mfma(const void* A, const void* Wp, void* C, int M, int N, int
   const int n_tiles = (N + 15) / 16;
   const int k_steps = (K + 31) / 32;
   const int steps_per_group = (k_steps + k_groups - 1) / k_groups;
+  if (M > 16) {
+    const int mt = (M + 15) / 16;
+    const int waves = (steps_per_group + ROWS_KSTEPS - 1) / ROWS_KSTEPS;   // at most 8 by the group limit
+    int blocks = n_tiles;
+    const int cap = 256 / k_groups;
+    if (blocks > cap) blocks = cap > 0 ? cap : 1;
+    dim3 grid(blocks, k_groups), block(waves * BLM_WAVE);
+    const size_t smem = (size_t)waves * mt * 256 * sizeof(float);
+#define BLM_GR(MT)                                                                                              \
+  hipLaunchKernelGGL((gemv_mfma_rows_kernel<MT, TC>), grid, block, smem, stream, (const bf16*)A,                \
+                     (const bf16*)Wp, (TC*)C, M, N, K, lda, ldc, n_tiles, k_steps, c_mode, steps_per_group)
+    if (mt == 2) BLM_GR(2);
+    else if (mt == 3) BLM_GR(3);
+    else BLM_GR(4);
+#undef BLM_GR
+    BLM_LAUNCH_CHECK("gemv_mfma_rows");
+    return 0;
+  }
   int ksteps = 0;
   const int waves = plan_k(steps_per_group * 32, &ksteps);
   // enough blocks to fill the chip, few enough that a block reuses its activations
@@ -173,12 +293,18 @@ static int launch_mfma(const void* A, const void* Wp, void* C, int M, int N, int
 // residual add in front of the next norm does it), so narrow outputs still occupy the whole chip.
 extern "C" int blm_gemv_mfma(const void* A, const void* Wp, void* C, int c_dtype, int M, int N, int K, int lda,
                              int ldc, int c_mode, int k_groups, hipStream_t stream) {
-  BLM_REQUIRE(M >= 1 && M <= 16, "gemv_mfma: M=%d out of range 1..16", M);
-  BLM_REQUIRE(blm_gemv_mfma_supported(M, N, K), "gemv_mfma: sizes N=%d K=%d not supported (K a multiple of 8, at most 16384)", N, K);
+  BLM_REQUIRE(M >= 1 && M <= 64, "gemv_mfma: M=%d out of range 1..64", M);
+  BLM_REQUIRE(N >= 1 && K >= 8 && K % 8 == 0, "gemv_mfma: sizes N=%d K=%d not supported (K a multiple of 8)", N, K);
   BLM_REQUIRE(c_mode == 0 || (c_mode == 1 && N % 16 == 0 && k_groups == 1),
               "gemv_mfma: c_mode %d needs N a multiple of 16 and one K group", c_mode);
   BLM_REQUIRE(k_groups >= 1 && k_groups <= 64 && (k_groups == 1 || c_dtype == BLM_F32),
               "gemv_mfma: k_groups=%d needs 1..64 and a float output when above 1", k_groups);
+  {
+    const int steps = (K + 31) / 32, per_group = (steps + k_groups - 1) / k_groups;
+    BLM_REQUIRE(per_group * 32 <= blm_gemv_mfma_group_limit(M),
+                "gemv_mfma: %d rows take at most K=%d per group, got K=%d in %d group(s)", M,
+                blm_gemv_mfma_group_limit(M), K, k_groups);
+  }
   BLM_REQUIRE(lda % 8 == 0 && lda >= K && ldc >= (c_mode ? N / 2 : N), "gemv_mfma: bad strides lda=%d ldc=%d", lda, ldc);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0, "gemv_mfma: operands must be 16-byte aligned");
   if (c_dtype == BLM_BF16) return launch_mfma<bf16>(A, Wp, C, M, N, K, lda, ldc, c_mode, k_groups, stream);

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 _lib = None
 _lock = threading.Lock()
 
@@ -46,6 +46,7 @@ _SIGNATURES = {
     "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
+    "blm_gemv_mfma_group_limit": [_c_int],
     "blm_gemv_qkv_rope_supported": [_c_int, _c_int, _c_int],
     "blm_gemv_qkv_rope": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -310,7 +311,13 @@ def gemv_skinny(a, w, out):
 
 
 def gemv_mfma_supported(M, N, K):
+    """Whether gemv_mfma takes M rows with all of K in one group."""
     return bool(library().blm_gemv_mfma_supported(int(M), int(N), int(K)))
+
+
+def gemv_mfma_group_limit(M):
+    """The largest K that one K-group of gemv_mfma may span for M rows (0: M out of range)."""
+    return int(library().blm_gemv_mfma_group_limit(int(M)))
 
 
 def pack_weight(w, gated=False):

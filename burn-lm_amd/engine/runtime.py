@@ -4,8 +4,8 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
 * float32 weights: the hand-written float kernels always (plain fused multiply-adds, no
   reduced-precision matrix mode), whatever the activation dtype.  This is the whole float32 path
   and also what keeps a tensor that a checkpoint stores in 32 bits exact in a bfloat16 run.
-* bfloat16 weights, up to 16 rows (decode): the hand-written skinny kernel on the matrix cores that
-  streams the weight once.
+* bfloat16 weights, up to 64 rows (decode): the hand-written skinny kernel on the matrix cores that
+  streams the weight once (where the width fits its registers: see ops.gemv_mfma_group_limit).
 * bfloat16 weights, many rows (prefill): the library product (hipBLASLt through torch), as the
   reference's engine leaves its matrix products to its tensor library
   (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).
@@ -17,7 +17,7 @@ import torch
 from ..csrc import ops
 
 SKINNY_MAX_ROWS = 8
-MFMA_SKINNY_MAX_ROWS = 16
+MFMA_SKINNY_MAX_ROWS = 64
 
 
 class LinearWeight:
@@ -57,14 +57,18 @@ class Runtime:
         return LinearWeight(w)
 
     @staticmethod
-    def k_groups(N, K):
+    def k_groups(N, K, M=1):
         """Into how many groups a skinny product's K is cut so that a narrow output still gives
         every compute unit a block: groups * (N / 16) tiles should reach 256 and a group should
-        span at most 2048 of K (its activations then fit the product's shared memory), but keeps at
-        least 1024."""
+        span at most 2048 of K, but keeps at least 1024; and a group must fit what the kernel
+        takes for M rows."""
         tiles = (N + 15) // 16
         g = 1
         while g < 8 and K // (g * 2) >= 1024 and (tiles * g < 256 or K // g > 2048):
+            g *= 2
+        limit = ops.gemv_mfma_group_limit(M)
+        steps = (K + 31) // 32
+        while g < 64 and (steps + g - 1) // g * 32 > limit:
             g *= 2
         return g
 
@@ -88,19 +92,21 @@ class Runtime:
             return ops.gemm_tiled(x, w, out)
         aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
         if packed is not None and M <= MFMA_SKINNY_MAX_ROWS and aligned:
-            groups = self.k_groups(N, K) if partials else 1
-            if groups > 1:
-                return ops.gemv_mfma(x, packed, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), K)
-            if out is None:
-                out = torch.empty(M, N, dtype=out_dtype, device=x.device)
-            return ops.gemv_mfma(x, packed, out, K)
+            if partials and out is None:
+                groups = self.k_groups(N, K, M)
+                if groups > 1:
+                    return ops.gemv_mfma(x, packed, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), K)
+            if ops.gemv_mfma_supported(M, N, K):
+                if out is None:
+                    out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+                return ops.gemv_mfma(x, packed, out, K)
         if out is None:
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
-        if packed is not None and aligned and out_dtype == torch.float32 and M <= 4 * MFMA_SKINNY_MAX_ROWS:
-            # float32 results (logits) for a few dozen rows: the skinny product 16 rows at a time; the
-            # weights stream once per 16 rows, which still beats the plain tiled kernel by far
-            for r in range(0, M, MFMA_SKINNY_MAX_ROWS):
-                ops.gemv_mfma(x[r:r + MFMA_SKINNY_MAX_ROWS], packed, out[r:r + MFMA_SKINNY_MAX_ROWS], K)
+        if packed is not None and aligned and out_dtype == torch.float32 and M <= MFMA_SKINNY_MAX_ROWS:
+            # float32 results (logits) for rows whose width the wide form does not take: 16 rows at a
+            # time; the weights stream once per 16 rows, which still beats the plain tiled kernel by far
+            for r in range(0, M, 16):
+                ops.gemv_mfma(x[r:r + 16], packed, out[r:r + 16], K)
             return out
         if M <= SKINNY_MAX_ROWS and aligned:
             return ops.gemv_skinny(x, w, out)
@@ -116,7 +122,8 @@ class Runtime:
         M, K = x.shape
         inner = w.shape[0] // 2
         if (isinstance(w, LinearWeight) and w.packed is not None and w.gated and x.dtype == torch.bfloat16
-                and M <= MFMA_SKINNY_MAX_ROWS and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+                and M <= MFMA_SKINNY_MAX_ROWS and ops.gemv_mfma_supported(M, w.shape[0], K)
+                and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
             return ops.gemv_mfma(x, w.packed, out, K, gated=True)
         gu = self.linear(x, w.w if isinstance(w, LinearWeight) else w)

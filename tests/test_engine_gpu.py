@@ -273,14 +273,14 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_graph_replays_with_library_products_inside(folders, dtype):
-    """More than 16 sequences per decode step: the layer products are the library's, recorded into
-    the graph.  Every replay is checked against the eager engine, with eager prefills and
-    synchronisations between replays."""
+@pytest.mark.parametrize("n,bucket", [(20, 24), (70, 96)])
+def test_graph_replays_of_larger_batches(folders, dtype, n, bucket):
+    """20 sequences per decode step: the skinny product with several row tiles; 70: the layer products
+    are the library's, recorded into the graph.  Every replay is checked against the eager engine,
+    with eager prefills and synchronisations between replays."""
     cfg, seed = TINIES["B"]
-    g = load(folders["B"], dtype, max_tokens=8192, max_seqs=32)
-    e = load(folders["B"], dtype, max_tokens=8192, max_seqs=32, graphs=False)
-    n = 20
+    g = load(folders["B"], dtype, max_tokens=16384, max_seqs=80)
+    e = load(folders["B"], dtype, max_tokens=16384, max_seqs=80, graphs=False)
     prompts = [random_tokens(300 + i, cfg["vocab_size"], 3 + (7 * i) % 40) for i in range(n)]
     sg = [g.open() for _ in range(n)]
     se = [e.open() for _ in range(n)]
@@ -301,7 +301,7 @@ def test_graph_replays_with_library_products_inside(folders, dtype):
             i = live.pop(3)
             g.close(sg[i]); e.close(se[i])
             torch.cuda.synchronize()
-    assert g.graphs.replays >= 35 and any(k[0] == 24 for k in g.graphs.captured)
+    assert g.graphs.replays >= 35 and any(k[0] == bucket for k in g.graphs.captured)
 
 
 def test_head_size_that_is_no_power_of_two_and_odd_counts(tmp_path):
