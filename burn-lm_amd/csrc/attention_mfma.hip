@@ -20,13 +20,12 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
 
 #define AM_WAVES 4
 #define AM_PAGE 64
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
 
 // keep the first n (0..4) bf16 of an 8-byte group, zero the rest
 __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
@@ -45,7 +44,9 @@ __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
 // The softmax runs in base 2: scale2 = scale * log2(e), m is the running maximum of s * scale2,
 // probabilities are exp2(s * scale2 - m); sums and outputs are the same as in base e.
 // KSTR / VSTR: row strides (elements) of the key page [64][KSTR] and the value page [HD][VSTR].
-template <int HD, bool FULL, int KSTR, int VSTR>
+// V_LATE: the values are read after the scores (pages in shared memory: short latency, fewer
+// registers); otherwise together with the keys (pages in global memory: one round trip for both).
+template <int HD, bool FULL, int KSTR, int VSTR, bool V_LATE>
 __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf16* __restrict__ vp,
                                           const uint4* qf, int key0, int qpos, int lo, int max_key, float scale2,
                                           float& m, float& l, f32x4_t* o) {
@@ -65,13 +66,12 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
       kf[t][ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(kp + (size_t)(t * 16 + c) * KSTR + d) : zero;
     }
   uint2 vf[DT][4];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-      vf[dt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * VSTR + t * 16 + kg * 4);
+#define AM_LOAD_VALUES()                                                                                    \
+  _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) _Pragma("unroll") for (int t = 0; t < 4; ++t)           \
+      vf[dt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * VSTR + t * 16 + kg * 4)
+  if (!V_LATE) { AM_LOAD_VALUES(); }
 
-  // scores
+  // scores, unscaled; the scale (> 0) goes into the exponent's multiply-add
   float s[4][4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
@@ -83,19 +83,20 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       if (FULL) {
-        s[t][r] = acc[r] * scale2;
+        s[t][r] = acc[r];
       } else {
         const int kj = key0 + t * 16 + kg * 4 + r;
-        s[t][r] = (kj <= qpos && kj >= lo) ? acc[r] * scale2 : -INFINITY;
+        s[t][r] = (kj <= qpos && kj >= lo) ? acc[r] : -INFINITY;
       }
     }
   }
+  if (V_LATE) { AM_LOAD_VALUES(); }   // the keys' registers are free now; the values arrive during the softmax
   float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
 #pragma unroll
   for (int t = 1; t < 4; ++t) mx = fmaxf(mx, fmaxf(fmaxf(s[t][0], s[t][1]), fmaxf(s[t][2], s[t][3])));
   mx = fmaxf(mx, __shfl_xor(mx, 16, BLM_WAVE));
   mx = fmaxf(mx, __shfl_xor(mx, 32, BLM_WAVE));
-  const float m_new = fmaxf(m, mx);
+  const float m_new = fmaxf(m, mx * scale2);
   // m = -inf, m_new finite -> 0;  both -inf (nothing visible yet) -> 1, and every p below is 0
   const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
   float psum = 0.f;
@@ -104,18 +105,21 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float p;
-      if (FULL) p = __builtin_amdgcn_exp2f(s[t][r] - m_new);
-      else p = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s[t][r] - m_new);
+      if (FULL) p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
+      else p = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
       s[t][r] = p;
       psum += p;
     }
   l = l * corr + psum;
+  if (__any(m != m_new)) {   // once the running maxima have settled, most pages change none of them
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
+  }
   m = m_new;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
 
+#undef AM_LOAD_VALUES
   // O^T += V^T P^T, 32 keys (two 16-key tiles) per MFMA
   const bool tail = !FULL && key0 + AM_PAGE - 1 > max_key;   // uniform: the page holds places past the data
 #pragma unroll
@@ -160,7 +164,7 @@ __device__ __forceinline__ void load_q(const bf16* qrow, uint4* qf) {
 // padded by 16 bytes so that the fragment reads do not collide.
 // ---------------------------------------------------------------------------------------
 template <int HD>
-__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
+__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 4 : (HD <= 128 ? 2 : 1))))
     attn_prefill_mfma_kernel(const bf16* __restrict__ q, int q_row_stride, bf16* __restrict__ out,
                              const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
                              const int* __restrict__ block_table, int table_width,
@@ -176,12 +180,22 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int c = lane & 15, kg = lane >> 4;
   const int G = nh / nkv;
-  const int kvh = blockIdx.y, b = blockIdx.z;
+  const int b = blockIdx.z;
   const int row_begin = cu_seqlens[b];
   const int n_b = cu_seqlens[b + 1] - row_begin;
-  // The longest tiles (the last queries of a causal prompt see the most keys) are launched first,
-  // so that the tail of the launch is made of short ones.
-  const int u0 = (gridDim.x - 1 - blockIdx.x) * AM_WAVES;
+  // Which (key-value head, query tiles) this block takes.  Blocks are handed out in the order of
+  // their linear index, consecutive ones to different dies: the key-value head changes fastest, so
+  // a die (with its own L2) mostly sees the pages of one head.  Along the other axis the work of a
+  // causal prompt falls from the last query tile (most keys) to the first; every second run of 32
+  // is reversed so that compute units that receive one block of each run get equal shares.
+  const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+  const int kvh = lin % nkv;
+  int x = lin / nkv;
+  {
+    const int seg = x >> 5;
+    if ((seg & 1) && seg * 32 + 32 <= (int)gridDim.x) x = seg * 32 + 31 - (x & 31);
+  }
+  const int u0 = ((int)gridDim.x - 1 - x) * AM_WAVES;
   if ((u0 / G) * 16 >= n_b) return;   // the whole block lies past the sequence's end (uniform)
   const int u = u0 + wave;
   const int g = u % G, qt = u / G;
@@ -212,19 +226,19 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   const float scale2 = scale * 1.4426950408889634f;
   const int* bt = block_table + (size_t)b * table_width;
 
-  uint4 kreg[PER_THREAD], vreg[PER_THREAD];
-  auto fetch = [&](int pi) {
-    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; ++i) {
-      const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;
-      if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {
-        kreg[i] = *reinterpret_cast<const uint4*>(kcache + base + (size_t)j * 8);
-        vreg[i] = *reinterpret_cast<const uint4*>(vcache + base + (size_t)j * 8);
-      }
-    }
-  };
-  fetch(blk_first);
+  u32x4_t kreg[PER_THREAD], vreg[PER_THREAD];
+#define AM_FETCH(pi)                                                                          \
+  {                                                                                           \
+    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;                          \
+    _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                  \
+      const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                    \
+      if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {                                \
+        kreg[i] = *reinterpret_cast<const u32x4_t*>(kcache + base + (size_t)j * 8);             \
+        vreg[i] = *reinterpret_cast<const u32x4_t*>(vcache + base + (size_t)j * 8);             \
+      }                                                                                       \
+    }                                                                                         \
+  }
+  AM_FETCH(blk_first);
   for (int pi = blk_first; pi <= blk_last; ++pi) {
     __syncthreads();   // the page before has been used by every wavefront
 #pragma unroll
@@ -232,22 +246,23 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;
       if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {
         const int kr = j / (HD / 8), kc = j - kr * (HD / 8);          // key row, 16-byte column
-        *reinterpret_cast<uint4*>(k_lds + kr * KSTR + kc * 8) = kreg[i];
+        *reinterpret_cast<u32x4_t*>(k_lds + kr * KSTR + kc * 8) = kreg[i];
         const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8);  // value row (a dim), 16-byte column
-        *reinterpret_cast<uint4*>(v_lds + vr * VSTR + vc * 8) = vreg[i];
+        *reinterpret_cast<u32x4_t*>(v_lds + vr * VSTR + vc * 8) = vreg[i];
       }
     }
     __syncthreads();
-    if (pi < blk_last) fetch(pi + 1);   // travels while this page is used
+    if (pi < blk_last) AM_FETCH(pi + 1);   // travels while this page is used
     if (pi >= my_first && pi <= my_last) {
       const int key0 = pi * AM_PAGE;
       // pages wholly inside every query's range need no mask
       if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)
-        attn_page<HD, true, KSTR, VSTR>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+        attn_page<HD, true, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
       else
-        attn_page<HD, false, KSTR, VSTR>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+        attn_page<HD, false, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
     }
   }
+#undef AM_FETCH
   if (!active) return;
   l += __shfl_xor(l, 16, BLM_WAVE);
   l += __shfl_xor(l, 32, BLM_WAVE);
@@ -312,9 +327,9 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
       const int key0 = pi * AM_PAGE;
       if (key0 + AM_PAGE - 1 <= pos && key0 >= lo)
-        attn_page<HD, true, HD, AM_PAGE>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+        attn_page<HD, true, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
       else
-        attn_page<HD, false, HD, AM_PAGE>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+        attn_page<HD, false, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
     }
   }
   l += __shfl_xor(l, 16, BLM_WAVE);
@@ -413,6 +428,7 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
               "attn_prefill_mfma: needs bfloat16, pages of 64 and a head_dim of 16, 32, 64, 128 or 256 "
               "(got dtype %d, page %d, head_dim %d)", act_dtype, page_size, hd);
   BLM_REQUIRE(table_width > 0 && window >= 0, "attn_prefill_mfma: bad geometry");
+  BLM_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive (got %g)", (double)scale);
   BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0,
               "attn_prefill_mfma: q rows must be 16-byte aligned");
   const int G = nh / nkv;
@@ -443,6 +459,7 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
   BLM_REQUIRE(table_width > 0 && window >= 0 && n_splits >= 1 && n_splits <= 65535,
               "attn_decode: bad geometry width=%d window=%d splits=%d", table_width, window, n_splits);
   BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attn_decode: q rows must be 16-byte aligned");
+  BLM_REQUIRE(scale > 0.f, "attn_decode: the score scale must be positive (got %g)", (double)scale);
   const int G = nh / nkv;
   const int gtiles = (G + 15) / 16;
   BLM_REQUIRE((long long)nkv * gtiles <= 65535, "attn_decode: too many heads");

@@ -13,12 +13,17 @@ struct bf16 {
 __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16 x) { return __uint_as_float(((uint32_t)x.v) << 16); }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN (the hardware conversion of gfx950)
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+
+// two floats to a pair of bf16 in one register (lo in the low half), one instruction
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float blm_f32x2;
+  typedef __attribute__((ext_vector_type(2))) __bf16 blm_bf16x2;
+  const blm_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, blm_bf16x2));
 }
 
 template <typename T>
