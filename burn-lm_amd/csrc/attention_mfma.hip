@@ -27,6 +27,15 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
 
+// Stores and loads that bypass the per-die caches: what one block writes this way, a block on
+// another die reads this way, once the store has completed.
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // keep the first n (0..4) bf16 of an 8-byte group, zero the rest
 __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
   if (n >= 4) return v;
@@ -284,15 +293,16 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 
 // ---------------------------------------------------------------------------------------
 // decode: grid (splits, kv heads * head tiles, tokens); partial results per split
-//   part_o [T, nh, splits, HD] float, part_ml [T, nh, splits, 2] float
+//   part_o [T, nh, splits, HD] float, part_ml [T, nh, splits, 2] float,
+// merged by whichever split of a (token, head tile) finishes last
 // ---------------------------------------------------------------------------------------
 template <int HD>
 __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     attn_decode_mfma_kernel(const bf16* __restrict__ q, int q_row_stride, const int* __restrict__ positions,
                             const int* __restrict__ token_seq, const int* __restrict__ block_table,
                             int table_width, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
-                            int nh, int nkv, float scale, int window, int n_splits, float* __restrict__ part_o,
-                            float* __restrict__ part_ml) {
+                            int nh, int nkv, float scale, int window, int n_splits, float* part_o,
+                            float* part_ml, int* arrivals, bf16* out) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
   __shared__ float sm_m[AM_WAVES][16], sm_l[AM_WAVES][16];
@@ -356,53 +366,69 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       L += sm_l[k][cc] * f;
       O += sm_o[k][cc][d] * f;
     }
-    const size_t at = ((size_t)t * nh + kvh * G + g0 + cc) * n_splits + split;
-    part_o[at * HD + d] = O;
-    if (d == 0) { part_ml[at * 2] = M; part_ml[at * 2 + 1] = L; }
+    if (n_splits == 1 || b < 0) {   // nothing to merge (a padding token gives zeros)
+      out[((size_t)t * nh + kvh * G + g0 + cc) * HD + d] = from_float<bf16>(b < 0 ? 0.f : O / L);
+    } else {
+      const size_t at = ((size_t)t * nh + kvh * G + g0 + cc) * n_splits + split;
+      coherent_store(part_o + at * HD + d, O);
+      if (d == 0) { coherent_store(part_ml + at * 2, M); coherent_store(part_ml + at * 2 + 1, L); }
+    }
   }
-}
+  if (n_splits == 1 || b < 0) return;
 
-// Merge of the splits.  The loads of eight splits are issued together: a loop that waits for each
-// split in turn spends a memory round trip per split.
-template <int HD>
-__global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                           const int* __restrict__ token_seq, bf16* __restrict__ out, int nh,
-                                           int n_splits) {
-  const int head = blockIdx.x, t = blockIdx.y;
-  const int d = threadIdx.x;
-  if (d >= HD) return;
-  bf16* o = out + ((size_t)t * nh + head) * HD;
-  if (token_seq[t] < 0) { o[d] = from_float<bf16>(0.f); return; }   // padding token
-  const size_t base = ((size_t)t * nh + head) * n_splits;
-  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
-  float M = -INFINITY;
-  for (int s0 = 0; s0 < n_splits; s0 += 8) {
-    float2 v[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = ml[min(s0 + i, n_splits - 1)];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) M = fmaxf(M, v[i].x);
+  // The block that finishes last among the splits of its (token, head tile) merges them.  Every
+  // block writes its partial result with stores that go through to device-coherent memory, waits
+  // for them to complete, and then counts itself in; the block that finds all the others counted
+  // reads their results with loads that come from device-coherent memory and writes the output.
+  // Nobody waits for anybody, and no cache is flushed or invalidated as a whole (a device-wide
+  // fence does that on every one of the eight dies, and costs far more than the merge).  The
+  // counter goes back to zero for the next launch.
+  __shared__ int last;
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's stores have been acknowledged
+  __syncthreads();
+  int* counter = arrivals + (size_t)t * gridDim.y + blockIdx.y;
+  if (threadIdx.x == 0) {
+    const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = before == n_splits - 1;
+    if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  float L = 0.f, O = 0.f;
-  for (int s0 = 0; s0 < n_splits; s0 += 8) {
-    float2 v[8];
-    float po[8];
+  __syncthreads();
+  if (!last) return;
+  for (int idx = threadIdx.x; idx < 16 * HD; idx += blockDim.x) {
+    const int cc = idx / HD, d = idx - cc * HD;
+    if (g0 + cc >= G) continue;
+    const size_t head_at = (size_t)t * nh + kvh * G + g0 + cc;
+    const size_t base = head_at * n_splits;
+    const float* ml = part_ml + base * 2;
+    // eight splits per memory round trip, merged online
+    float M = -INFINITY, L = 0.f, O = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float vm[8], vl[8], po[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int s = min(s0 + i, n_splits - 1);
-      v[i] = ml[s];
-      po[i] = part_o[(base + s) * HD + d];
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (s0 + i < n_splits) {
-        const float f = (v[i].x == M) ? 1.f : __builtin_amdgcn_exp2f(v[i].x - M);   // maxima are in base 2
-        L += v[i].y * f;
-        O += po[i] * f;
+      for (int i = 0; i < 8; ++i) {
+        const int sp = min(s0 + i, n_splits - 1);
+        vm[i] = coherent_load(ml + 2 * sp);
+        vl[i] = coherent_load(ml + 2 * sp + 1);
+        po[i] = coherent_load(part_o + (base + sp) * HD + d);
       }
+      float Mc = M;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) Mc = fmaxf(Mc, vm[i]);
+      const float keep = (M == Mc) ? 1.f : __builtin_amdgcn_exp2f(M - Mc);   // maxima are in base 2
+      L *= keep;
+      O *= keep;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (s0 + i < n_splits) {
+          const float f = (vm[i] == Mc) ? 1.f : __builtin_amdgcn_exp2f(vm[i] - Mc);
+          L += vl[i] * f;
+          O += po[i] * f;
+        }
+      }
+      M = Mc;
     }
+    out[head_at * HD + d] = from_float<bf16>(O / L);
   }
-  o[d] = from_float<bf16>(O / L);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -446,11 +472,14 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
   return 0;
 }
 
-// workspace: part_o needs T*nh*n_splits*hd floats, part_ml T*nh*n_splits*2 floats
+// workspace: part_o needs T*nh*n_splits*hd floats, part_ml T*nh*n_splits*2 floats; arrivals needs
+// T * kv_heads * ceil(group / 16) ints that are zero before the first call (every call leaves them
+// zero again).  Calls that share the arrivals buffer must not overlap in time.
 extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int act_dtype, const int* positions,
                                const int* token_seq, const int* block_table, int table_width, const void* kcache,
                                const void* vcache, int page_size, int T, int nh, int nkv, int hd, float scale,
-                               int window, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
+                               int window, int n_splits, float* part_o, float* part_ml, int* arrivals,
+                               hipStream_t stream) {
   BLM_REQUIRE(T > 0 && T <= 65535 && nh > 0 && nkv > 0 && nh % nkv == 0,
               "attn_decode: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
   BLM_REQUIRE(blm_attn_decode_supported(act_dtype, hd, page_size),
@@ -464,18 +493,14 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
   const int gtiles = (G + 15) / 16;
   BLM_REQUIRE((long long)nkv * gtiles <= 65535, "attn_decode: too many heads");
   dim3 grid(n_splits, nkv * gtiles, T), block(AM_WAVES * BLM_WAVE);
-  dim3 cgrid(nh, T), cblock(hd < 64 ? 64 : hd);
 #define BLM_AD(HD)                                                                                                 \
   case HD:                                                                                                         \
     hipLaunchKernelGGL((attn_decode_mfma_kernel<HD>), grid, block, 0, stream, (const bf16*)q, q_row_stride,         \
                        positions, token_seq, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache,    \
-                       nh, nkv, scale, window, n_splits, part_o, part_ml);                                          \
-    BLM_LAUNCH_CHECK("attn_decode_mfma");                                                                          \
-    hipLaunchKernelGGL((attn_decode_combine_kernel<HD>), cgrid, cblock, 0, stream, part_o, part_ml, token_seq,      \
-                       (bf16*)out, nh, n_splits);                                                                  \
+                       nh, nkv, scale, window, n_splits, part_o, part_ml, arrivals, (bf16*)out);                    \
     break
   switch (hd) { BLM_AD(16); BLM_AD(32); BLM_AD(64); BLM_AD(128); }
 #undef BLM_AD
-  BLM_LAUNCH_CHECK("attn_decode_combine");
+  BLM_LAUNCH_CHECK("attn_decode_mfma");
   return 0;
 }

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 _lib = None
 _lock = threading.Lock()
 
@@ -33,7 +33,7 @@ _SIGNATURES = {
                        _c_void_p],
     "blm_attn_decode": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
-                        _c_void_p, _c_void_p, _c_void_p],
+                        _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     "blm_attn_decode_supported": [_c_int, _c_int, _c_int],
     "blm_attn_prefill_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_attn_prefill_mfma": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -124,6 +124,25 @@ def _call(name, *args):
 
 def _ptr(t):
     return 0 if t is None else t.data_ptr()
+
+
+ARRIVAL_COUNTERS = 1 << 16
+_arrivals = {}
+
+
+def arrival_counters(device):
+    """Zeroed int32 counters of a device, for kernels whose blocks count themselves in so that the
+    last one finishes a shared result.  Every such kernel leaves them zero again, so all of them
+    share one buffer; launches that use it must not overlap in time (one stream at a time).  It is
+    allocated at the first call, which must not be under graph capture (Runtime() makes that call)."""
+    device = torch.device(device)
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    buf = _arrivals.get(key)
+    if buf is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("arrival_counters: the first call for a device must come before any graph capture")
+        buf = _arrivals[key] = torch.zeros(ARRIVAL_COUNTERS, dtype=torch.int32, device=torch.device("cuda", key))
+    return buf
 
 
 def _check_planes(who, kcache, vcache, nkv, page_size, hd):
@@ -275,10 +294,13 @@ def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache,
     n_splits = max(1, int(n_splits))
     part_o = torch.empty(T * nh * n_splits * hd, dtype=torch.float32, device=out.device)
     part_ml = torch.empty(T * nh * n_splits * 2, dtype=torch.float32, device=out.device)
+    arrivals = arrival_counters(out.device)
+    if T * nkv * ((nh // nkv + 15) // 16) > arrivals.numel():
+        raise KernelError(f"attn_decode: {T} tokens x {nkv} key-value heads need more than {arrivals.numel()} counters")
     _call("blm_attn_decode", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
           page_size, T, nh, nkv, hd, float(scale), int(window), n_splits, part_o.data_ptr(), part_ml.data_ptr(),
-          _stream())
+          arrivals.data_ptr(), _stream())
     return out
 
 

@@ -41,6 +41,7 @@ class Runtime:
         self.page_size = page_size
         self.ops = ops
         ops.library()  # fail now, loudly, if the kernel library cannot be had
+        ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
 
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)

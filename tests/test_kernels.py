@@ -223,6 +223,36 @@ def _paged_case(g, lens, nkv, hd, page=64, n_pages=40, far_key=None):
     return table, keys, values, kc.bfloat16(), vc.bfloat16()
 
 
+def test_attn_decode_merge_by_the_last_split_over_many_calls(ops):
+    """The splits of a (token, key-value head) are merged by whichever of their blocks finishes last,
+    through counters that every call must leave at zero.  A chip-filling case (8 tokens x 8 heads x 16
+    splits) run 40 times with fresh queries and a changing number of splits, every result checked; a
+    stale partial result or a counter left over from the call before would show."""
+    g = torch.Generator().manual_seed(33)
+    nh, nkv, hd = 32, 8, 64
+    lens = [1500, 1024, 700, 1333, 64, 999, 1471, 300]
+    table, keys, values, kc, vc = _paged_case(g, lens, nkv, hd, n_pages=160)
+    positions = dev(torch.tensor([L - 1 for L in lens], dtype=torch.int32))
+    token_seq = dev(torch.arange(len(lens), dtype=torch.int32))
+    table, kc, vc = dev(table), dev(kc), dev(vc)
+    stride = (nh + 2 * nkv) * hd
+    scale = 1.0 / math.sqrt(hd)
+    K = [k.cuda().float() for k in keys]
+    V = [v.cuda().float() for v in values]
+    counters = ops.arrival_counters("cuda")
+    for it in range(40):
+        qkv = dev(torch.randn(len(lens), stride, generator=g).bfloat16())
+        out = torch.full((len(lens), nh * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.attn_decode(qkv, stride, out, positions, token_seq, table, kc, vc, 64, nh, nkv, hd, scale, 0, (16, 3, 24, 8)[it % 4])
+        for b in range(len(lens)):
+            q = qkv[b, : nh * hd].float().reshape(nkv, nh // nkv, hd)
+            sc = torch.einsum("kgd,lkd->kgl", q, K[b]) * scale
+            want = torch.einsum("kgl,lkd->kgd", torch.softmax(sc, -1), V[b]).reshape(nh * hd)
+            err = float((out[b].float() - want).abs().max() / want.abs().max())
+            assert err <= 1.5e-2, f"call {it} sequence {b}: {err:.3g}"
+    assert int(counters.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("nh,nkv,hd,window,splits", [(4, 2, 16, 0, 3), (6, 1, 32, 0, 1), (5, 5, 64, 0, 4), (8, 2, 128, 0, 16),
                                                       (32, 1, 64, 0, 2), (20, 1, 32, 0, 5), (4, 2, 32, 100, 2)])
 def test_attn_decode(ops, nh, nkv, hd, window, splits):
