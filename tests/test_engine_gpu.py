@@ -425,3 +425,30 @@ def test_sampled_tokens_follow_the_plain_probabilities(folders):
             u = uniform(11, i, n)
             assert (cdf[k - 1] if k else 0.0) - 1e-4 <= u <= cdf[k] + 1e-4, f"request {i} token {n}"
             seq.append(tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_fed_in_uneven_chunks_beside_a_decoding_neighbour(folders, dtype):
+    """Any cut of a sequence into steps gives the same logits: a 300-token prompt in chunks of 100, 28,
+    64, 1, 90 and 17 tokens (chunk ends on, before and after page edges), while a second sequence in
+    the same steps goes on one token at a time."""
+    cfg, seed = TINIES["A"]
+    plain = P.load_model_folder(folders["A"])
+    eng = load(folders["A"], dtype, max_tokens=2048)
+    long_req = random_tokens(700, cfg["vocab_size"], 300)
+    short = random_tokens(701, cfg["vocab_size"], 40)
+    want_long = P.transformer_forward([long_req], plain)[0]
+    want_short = P.transformer_forward([short], plain)[0]
+    a, b = eng.open(), eng.open()
+    got = eng.step([(b, short[:34], [33])]).double().cpu().numpy()
+    assert rel_err(got[0], want_short[33]) <= TOL[dtype]
+    at, k = 0, 34
+    for n in (100, 28, 64, 1, 90, 17):
+        rows = sorted({0, n // 2, n - 1})
+        got = eng.step([(a, long_req[at:at + n], rows), (b, [short[k]], [0])]).double().cpu().numpy()
+        for j, r in enumerate(rows):
+            assert rel_err(got[j], want_long[at + r]) <= TOL[dtype], f"{dtype} chunk at {at} row {r}"
+        assert rel_err(got[len(rows)], want_short[k]) <= TOL[dtype], f"{dtype} neighbour at {k}"
+        at += n
+        k += 1
+    assert at == 300
