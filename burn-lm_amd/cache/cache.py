@@ -14,6 +14,9 @@ kv_cache.rs:14-33) and never clears it on reset (cache.rs:45-48); neither does t
 what a sequence may read is decided by its length alone, never by the bytes left in a page.
 
 All bookkeeping is on the host and needs no GPU; only the storage tensors live on the device.
+It is kept by the native core (csrc/host/cache_core.cpp, bound in core.py): slots, lengths, pools
+and page tables, and the assembly of a step's index arrays; this module owns the tensors and
+turns the core's failure codes into exceptions.
 """
 from __future__ import annotations
 
@@ -23,6 +26,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..parts.base import KVNeed, StateNeed
+from . import core as _core
 
 
 class CacheError(RuntimeError):
@@ -41,45 +45,87 @@ class ContextOverflow(CacheError):
         self.actual, self.maximum = actual, maximum
 
 
+def _raise(code: int):
+    """Turns a failure code of the native core into this module's exceptions."""
+    msg = _core.last_error()
+    if code == _core.E_FULL:
+        raise CacheFull(msg)
+    raise CacheError(msg)
+
+
 class PagePool:
     """Free list of page numbers that knows which pages are out, so a page cannot be handed out
-    twice or given back twice."""
+    twice or given back twice.  The list lives in the native core; a group's pool is a view of
+    the one inside the cache's core."""
 
-    def __init__(self, n_pages: int):
+    def __init__(self, n_pages: int, _native=None):
         self.n_pages = n_pages
-        self._free = list(range(n_pages - 1, -1, -1))
-        self._out = set()
+        self._native = _native if _native is not None else _core.NativePool(n_pages)
 
     @property
     def n_free(self):
-        return len(self._free)
+        return self._native.n_free
 
     def take(self, n: int) -> List[int]:
-        if n > len(self._free):
-            raise CacheFull(f"{n} pages wanted, {len(self._free)} free of {self.n_pages}")
-        pages = [self._free.pop() for _ in range(n)]
-        self._out.update(pages)
+        code, pages = self._native.take(n)
+        if code:
+            _raise(code)
         return pages
 
     def give(self, pages: Sequence[int]) -> None:
-        for p in pages:
-            if p not in self._out:
-                raise CacheError(f"page {p} given back but not handed out (freed twice?)")
-        for p in pages:
-            self._out.remove(p)
-            self._free.append(p)
+        code = self._native.give(pages)
+        if code:
+            _raise(code)
+
+    # what tests look at: the free pages (the next to be handed out last) and the pages that are out
+    @property
+    def _free(self):
+        return self._native.free_list()
+
+    @property
+    def _out(self):
+        return self._native.out_set()
+
+
+class _Tables:
+    """Read-only mapping slot -> pages of each page index (-1 once released) of one group."""
+
+    def __init__(self, cache, group_index):
+        self._cache, self._gi = cache, group_index
+
+    def __getitem__(self, slot):
+        return self._cache._table(self._gi, slot)
+
+    def __contains__(self, slot):
+        return slot in self._cache.live_slots
+
+    def __iter__(self):
+        return iter(self._cache.live_slots)
+
+    def __len__(self):
+        return len(self._cache.live_slots)
+
+    def keys(self):
+        return self._cache.live_slots
+
+    def values(self):
+        return [self[s] for s in self._cache.live_slots]
+
+    def items(self):
+        return [(s, self[s]) for s in self._cache.live_slots]
 
 
 class KVGroup:
     def __init__(self, need: KVNeed, places: List[int], n_pages: int, page_size: int, dtype, device):
         self.need, self.places = need, places
         self.page_size = page_size
-        self.pool = PagePool(n_pages)
+        self.n_pages = n_pages
         # [place in group, key|value, page, kv head, token in page * head_dim]; a key page is
         # [token][head_dim], a value page is stored transposed, [head_dim][token]
         self.storage = torch.empty(len(places), 2, n_pages, need.n_kv_heads, page_size * need.head_dim,
                                    dtype=dtype, device=device)
-        self.tables: Dict[int, List[int]] = {}  # slot -> page of each page index (-1 once released)
+        self.pool: Optional[PagePool] = None      # set by the cache once its core exists
+        self.tables: Optional[_Tables] = None
 
     def pages_for(self, length: int) -> int:
         return (length + self.page_size - 1) // self.page_size
@@ -90,11 +136,6 @@ class KVGroup:
             return 0
         first_key = max(0, length_after - self.need.window + 1)  # oldest key the next token may see
         return first_key // self.page_size
-
-
-@dataclass
-class _Seq:
-    length: int = 0
 
 
 class KVView:
@@ -166,96 +207,116 @@ class Cache:
                 t = torch.zeros(max_seqs, *need.shape, dtype=need.dtype, device=device)
                 self.state_tensors.append(t)
                 self.views[i] = StateView(t)
-        self._free_slots = list(range(max_seqs - 1, -1, -1))
-        self._seqs: Dict[int, _Seq] = {}
+        lib = _core.library()
+        self._lib = lib
+        self._h = lib.blm_cache_new(len(self.groups), _core.ints([g.n_pages for g in self.groups]),
+                                    _core.ints([g.need.window for g in self.groups]), page_size, max_seqs, max_context)
+        if not self._h:
+            raise CacheError("the native cache core refused these sizes")
+        for gi, g in enumerate(self.groups):
+            g.pool = PagePool(g.n_pages, _native=_core.NativePool(g.n_pages, handle=lib.blm_cache_pool(self._h, gi)))
+            g.tables = _Tables(self, gi)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.blm_cache_free(h)
 
     # ---- slots -----------------------------------------------------------------------------
     @property
     def free_slots(self):
-        return len(self._free_slots)
+        return self._lib.blm_cache_n_free_slots(self._h)
+
+    @property
+    def _free_slots(self):
+        out = (_core.ctypes.c_int * self.max_seqs)()
+        n = self._lib.blm_cache_free_slots(self._h, out)
+        return list(out[:n])
 
     @property
     def live_slots(self):
-        return sorted(self._seqs)
+        out = (_core.ctypes.c_int * self.max_seqs)()
+        n = self._lib.blm_cache_live_slots(self._h, out)
+        return list(out[:n])
 
     def open(self) -> int:
-        if not self._free_slots:
-            raise CacheFull(f"all {self.max_seqs} sequence slots are in use")
-        slot = self._free_slots.pop()
-        self._seqs[slot] = _Seq()
-        for g in self.groups:
-            g.tables[slot] = []
+        slot = _core.ctypes.c_int(-1)
+        code = self._lib.blm_cache_open(self._h, _core.ctypes.byref(slot))
+        if code:
+            _raise(code)
         for t in self.state_tensors:
-            t[slot].zero_()
-        return slot
+            t[slot.value].zero_()
+        return slot.value
 
     def close(self, slot: int) -> None:
-        if slot not in self._seqs:
-            raise CacheError(f"slot {slot} is not open (closed twice?)")
-        for g in self.groups:
-            g.pool.give([p for p in g.tables.pop(slot) if p >= 0])
-        del self._seqs[slot]
-        self._free_slots.append(slot)
+        code = self._lib.blm_cache_close(self._h, int(slot))
+        if code:
+            _raise(code)
 
     def length(self, slot: int) -> int:
-        try:
-            return self._seqs[slot].length
-        except KeyError:
-            raise CacheError(f"slot {slot} is not open") from None
+        n = self._lib.blm_cache_length(self._h, int(slot))
+        if n < 0:
+            raise CacheError(f"slot {slot} is not open")
+        return n
 
     def room(self, slot: int) -> int:
         return self.max_context - self.length(slot)
+
+    def _table(self, group_index: int, slot: int) -> List[int]:
+        n = self._lib.blm_cache_table_len(self._h, group_index, int(slot))
+        if n < 0:
+            raise KeyError(slot)
+        out = (_core.ctypes.c_int * max(n, 1))()
+        self._lib.blm_cache_table(self._h, group_index, int(slot), out)
+        return list(out[:n])
 
     # ---- growth ----------------------------------------------------------------------------
     def reserve(self, growth: Sequence) -> None:
         """growth: (slot, n_new) pairs of one step.  Hands out the pages all of them need, or
         raises before anything changed."""
-        seen = set()
-        wanted = [0] * len(self.groups)
-        for slot, n in growth:
-            if slot in seen:
-                raise CacheError(f"slot {slot} appears twice in one step")
-            seen.add(slot)
-            length = self.length(slot)
-            if n <= 0:
-                raise CacheError(f"slot {slot}: a step must bring at least one token")
-            if length + n > self.max_context:
-                raise ContextOverflow(length + n, self.max_context)
-            for gi, g in enumerate(self.groups):
-                wanted[gi] += g.pages_for(length + n) - len(g.tables[slot])
-        for gi, g in enumerate(self.groups):
-            if wanted[gi] > g.pool.n_free:
-                raise CacheFull(f"the step needs {wanted[gi]} more pages of {self.page_size} tokens, "
-                                f"{g.pool.n_free} are free of {g.pool.n_pages}")
-        for slot, n in growth:
-            length = self._seqs[slot].length
-            for g in self.groups:
-                more = g.pages_for(length + n) - len(g.tables[slot])
-                if more > 0:
-                    g.tables[slot].extend(g.pool.take(more))
+        growth = list(growth)
+        detail = (_core.ctypes.c_int * 2)()
+        code = self._lib.blm_cache_reserve(self._h, len(growth), _core.ints([int(s) for s, _ in growth]),
+                                           _core.ints([int(n) for _, n in growth]), detail)
+        if code == _core.E_OVERFLOW:
+            raise ContextOverflow(detail[0], detail[1])
+        if code:
+            _raise(code)
 
     def advance(self, slot: int, n: int) -> None:
         """The step that reserved n tokens for the slot has run: the sequence is n longer."""
-        seq = self._seqs[slot]
-        seq.length += n
-        for g in self.groups:
-            first = g.first_needed_page(seq.length)
-            table = g.tables[slot]
-            gone = [table[i] for i in range(min(first, len(table))) if table[i] >= 0]
-            if gone:
-                g.pool.give(gone)
-                for i in range(min(first, len(table))):
-                    table[i] = -1
+        code = self._lib.blm_cache_advance(self._h, int(slot), int(n))
+        if code:
+            _raise(code)
 
     def page_table(self, group_index: int, slots: Sequence[int], width: int) -> List[List[int]]:
-        g = self.groups[group_index]
-        rows = []
-        for s in slots:
-            t = g.tables[s] if s >= 0 else []
-            if len(t) > width:
-                raise CacheError("page table wider than asked for")
-            rows.append(t + [-1] * (width - len(t)))
-        return rows
+        slots = [int(s) for s in slots]
+        out = (_core.ctypes.c_int * max(len(slots) * width, 1))()
+        code = self._lib.blm_cache_page_table(self._h, group_index, len(slots), _core.ints(slots), width, out)
+        if code:
+            _raise(code)
+        return [list(out[i * width:(i + 1) * width]) for i in range(len(slots))]
+
+    def fill_step(self, entries, pad_to: int, width: int, out_ptr: int, capacity: int):
+        """Writes the index arrays of a step for entries (slot, tokens, want) into int32 host memory
+        at out_ptr (see blm_step_fill in csrc/host/cache_core.h for the layout) and returns
+        (tokens, wanted rows, most tokens of one sequence, greatest length after the step)."""
+        slots, counts, tokens, want_counts, wants = [], [], [], [], []
+        for slot, toks, want in entries:
+            slots.append(slot)
+            counts.append(len(toks))
+            tokens.extend(toks)
+            want_counts.append(len(want))
+            wants.extend(want)
+        meta = (_core.ctypes.c_int * 4)()
+        code = self._lib.blm_step_fill(self._h, len(slots), _core.ints(slots), _core.ints(counts), _core.ints(tokens),
+                                       _core.ints(want_counts), _core.ints(wants), pad_to, width, out_ptr, capacity, meta)
+        if code:
+            _raise(code)
+        return tuple(meta)
+
+    def step_size(self, T: int, B: int, R: int, width: int) -> int:
+        return int(self._lib.blm_step_size(len(self.groups), T, B, R, width))
 
     def pages_in_use(self) -> int:
         return sum(g.pool.n_pages - g.pool.n_free for g in self.groups)

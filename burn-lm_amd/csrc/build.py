@@ -1,6 +1,11 @@
-"""Builds the HIP kernel library for gfx950 with hipcc: one object per source, compiled in
-parallel, linked into ``libburnlm_hip.so`` next to the sources.  No other build system and no
-torch headers are involved, so a first build takes about a minute."""
+"""Builds the two native libraries next to their sources.
+
+* ``libburnlm_hip.so``: the HIP kernels for gfx950, one object per ``.hip`` source compiled in
+  parallel by hipcc and linked.
+* ``libburnlm_host.so``: the host-side core (cache bookkeeping, step assembly) from ``host/*.cpp``
+  with the C++ compiler; it needs no GPU and no ROCm.
+
+No other build system and no torch headers are involved; a first build takes well under a minute."""
 from __future__ import annotations
 
 import hashlib
@@ -30,6 +35,26 @@ def source_hash():
         with open(os.path.join(HERE, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+HOST_LIB_NAME = "libburnlm_host.so"
+HOST_DIR = os.path.join(HERE, "host")
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+
+def host_sources():
+    return sorted(f for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+
+
+def host_hash():
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(HOST_DIR)):
+        if name.endswith((".cpp", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(HOST_DIR, name), "rb") as f:
+                h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
     return h.hexdigest()
 
 
@@ -70,6 +95,55 @@ def is_current():
         return False
 
 
+def host_lib_path():
+    return os.path.join(out_dir(), HOST_LIB_NAME)
+
+
+def _host_hash_path():
+    return os.path.join(out_dir(), "_build", "host.sha256")
+
+
+def host_is_current():
+    try:
+        with open(_host_hash_path()) as f:
+            return os.path.exists(host_lib_path()) and f.read().strip() == host_hash()
+    except OSError:
+        return False
+
+
+def find_cxx():
+    for cand in (os.environ.get("CXX"), "g++", "c++", "clang++", "/opt/rocm/llvm/bin/clang++"):
+        path = cand and (cand if os.path.isabs(cand) and os.path.exists(cand) else shutil.which(cand))
+        if path:
+            return path
+    raise RuntimeError("no C++ compiler found (looked at $CXX, g++, c++, clang++): the host library cannot be built")
+
+
+def build_host(verbose=True):
+    """Compile the host-side core.  Always compiles; returns the library path."""
+    cxx = find_cxx()
+    od = out_dir()
+    tmp = os.path.join(od, "_build", HOST_LIB_NAME + f".{os.getpid()}.tmp")
+    t0 = time.time()
+    r = subprocess.run([cxx, *HOST_FLAGS, "-I", HOST_DIR, *[os.path.join(HOST_DIR, s) for s in host_sources()], "-o", tmp],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"{cxx} failed on the host library:\n{r.stdout}")
+    os.replace(tmp, os.path.join(od, HOST_LIB_NAME))
+    with open(_host_hash_path(), "w") as f:
+        f.write(host_hash())
+    if verbose:
+        print(f"[burn-lm_amd build] built {os.path.join(od, HOST_LIB_NAME)} in {time.time() - t0:.1f} s",
+              file=sys.stderr, flush=True)
+    return os.path.join(od, HOST_LIB_NAME)
+
+
+def ensure_host_built(verbose=True):
+    if host_is_current():
+        return host_lib_path()
+    return build_host(verbose=verbose)
+
+
 def find_hipcc():
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.exists(cand):
@@ -79,7 +153,9 @@ def find_hipcc():
 
 
 def build(verbose=True, jobs=None):
-    """Compile every source and link the library.  Always compiles; returns the library path."""
+    """Compile every HIP source and link the kernel library, and compile the host library.  Always
+    compiles; returns the kernel library's path."""
+    build_host(verbose=verbose)
     hipcc = find_hipcc()
     od = out_dir()
     bdir = os.path.join(od, "_build")

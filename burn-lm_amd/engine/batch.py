@@ -27,33 +27,19 @@ class Step:
     is_decode: bool = False      # every sequence brings exactly one token
     host_slots: List[int] = field(default_factory=list)
     host_new: List[int] = field(default_factory=list)
+    host_image: object = None    # the pinned host buffer the index arrays were copied from
 
 
 def build_step(entries: Sequence, lengths: Sequence[int], cache, device) -> Step:
-    """entries: (slot, tokens, want) per sequence; lengths: what each already holds.  All index
-    arrays go to the device in one copy."""
-    tok, pos, seq, rows, cu, after, slots = [], [], [], [], [0], [], []
-    for b, ((slot, tokens, want), past) in enumerate(zip(entries, lengths)):
-        n = len(tokens)
-        base = len(tok)
-        tok.extend(tokens)
-        pos.extend(range(past, past + n))
-        seq.extend([b] * n)
-        rows.extend(base + w for w in want)
-        cu.append(base + n)
-        after.append(past + n)
-        slots.append(slot)
-    T, B, R = len(tok), len(entries), len(rows)
-    max_after = max(after)
+    """entries: (slot, tokens, want) per sequence; lengths: what each already holds.  The native
+    core writes all index arrays into one host buffer, which goes to the device in one copy."""
+    news = [len(e[1]) for e in entries]
+    T, B, R = sum(news), len(entries), sum(len(e[2]) for e in entries)
+    max_after = max(past + n for past, n in zip(lengths, news))
     width = max(1, (max_after + cache.page_size - 1) // cache.page_size)
-    tables = [cache.page_table(gi, slots, width) for gi in range(len(cache.groups))]
-    flat = tok + pos + seq + slots + cu + after + rows
-    for t in tables:
-        for r in t:
-            flat.extend(r)
-    host = torch.tensor(flat, dtype=torch.int32)
-    if device.type == "cuda":
-        host = host.pin_memory()
+    size = cache.step_size(T, B, R, width)
+    host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
+    cache.fill_step(entries, 0, width, host.data_ptr(), size)
     dev = host.to(device, non_blocking=True)
     o = 0
 
@@ -65,9 +51,10 @@ def build_step(entries: Sequence, lengths: Sequence[int], cache, device) -> Step
 
     token_ids, positions, token_seq = take(T), take(T), take(T)
     seq_slots, cu_seqlens, lens_after, want_rows = take(B), take(B + 1), take(B), take(R)
-    block_tables = {gi: take(B * width).view(B, width) for gi in range(len(tables))}
-    news = [len(e[1]) for e in entries]
-    return Step(n_tokens=T, n_seqs=B, n_wanted=R, token_ids=token_ids, positions=positions, token_seq=token_seq,
+    block_tables = {gi: take(B * width).view(B, width) for gi in range(len(cache.groups))}
+    step = Step(n_tokens=T, n_seqs=B, n_wanted=R, token_ids=token_ids, positions=positions, token_seq=token_seq,
                 seq_slots=seq_slots, cu_seqlens=cu_seqlens, lens_after=lens_after, want_rows=want_rows,
                 block_tables=block_tables, max_new=max(news), max_position=max_after - 1, max_len_after=max_after,
-                is_decode=all(n == 1 for n in news), host_slots=slots, host_new=news)
+                is_decode=all(n == 1 for n in news), host_slots=[e[0] for e in entries], host_new=news)
+    step.host_image = host   # the pinned source of the copy stays alive as long as the step
+    return step

@@ -79,21 +79,15 @@ class _Captured:
         torch.cuda.synchronize()
 
     def fill(self, entries, lengths, cache):
-        """Host image of the index buffer for these (slot, [token], [0]) entries, rest padding."""
+        """Host image of the index buffer for these (slot, [token], [0]) entries, the rest padding;
+        written by the native core straight into the pinned buffer."""
         B, W = self.B, self.W
-        n = len(entries)
-        pad = B - n
-        tok = [e[1][0] for e in entries] + [0] * pad
-        pos = list(lengths) + [0] * pad
-        seq = list(range(n)) + [-1] * pad
-        slots = [e[0] for e in entries] + [-1] * pad
-        cu = list(range(B + 1))
-        after = [l + 1 for l in lengths] + [0] * pad
-        rows = list(range(B))
-        flat = tok + pos + seq + slots + cu + after + rows
-        for gi in range(len(cache.groups)):
-            for r in cache.page_table(gi, slots, W):
-                flat.extend(r)
+        if entries:
+            cache.fill_step(entries, B, W, self.host.data_ptr(), self.host.numel())
+            return
+        # all padding (used while recording): token 0, position 0, no sequence, no slot, no pages
+        flat = [0] * B + [0] * B + [-1] * B + [-1] * B + list(range(B + 1)) + [0] * B + list(range(B))
+        flat += [-1] * (len(cache.groups) * B * W)
         self.host.copy_(torch.tensor(flat, dtype=torch.int32))
 
     def run(self, entries, lengths, cache):

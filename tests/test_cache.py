@@ -165,3 +165,62 @@ def test_random_traffic_keeps_the_books():
     for s in list(live):
         c.close(s)
     assert c.pages_in_use() == 0 and c.free_slots == 5
+
+
+def _fill(c, entries, pad_to, width):
+    T = max(sum(len(t) for _, t, _ in entries), pad_to)
+    B = max(len(entries), pad_to)
+    R = max(sum(len(w) for _, _, w in entries), pad_to)
+    size = c.step_size(T, B, R, width)
+    host = torch.full((size,), 12345, dtype=torch.int32)
+    meta = c.fill_step(entries, pad_to, width, host.data_ptr(), size)
+    return host.tolist(), meta
+
+
+def test_step_assembly_of_unequal_prompts():
+    """The index arrays the native core writes for a step: tokens, positions, sequence of each token,
+    slots, first token of each sequence, lengths after, wanted rows, one page table per group."""
+    c = make([KVNeed(2, 8), KVNeed(2, 8, window=24)], max_tokens=320, max_seqs=5, max_context=96)
+    a, b = c.open(), c.open()
+    c.reserve([(a, 20)]); c.advance(a, 20)                     # a already holds 20 tokens
+    entries = [(b, [7, 8, 9], [0, 2]), (a, [5, 6], [1])]
+    c.reserve([(b, 3), (a, 2)])
+    flat, meta = _fill(c, entries, 0, 3)
+    assert meta == (5, 3, 3, 22)
+    want = ([7, 8, 9, 5, 6] + [0, 1, 2, 20, 21] + [0, 0, 0, 1, 1] + [b, a] + [0, 3, 5] + [3, 22] + [0, 2, 4])
+    for gi in range(2):
+        for row in c.page_table(gi, [b, a], 3):
+            want += row
+    assert flat == want
+    assert c.groups[0].tables[a] == c.page_table(0, [a], 2)[0] and len(c.groups[0].tables[a]) == 2
+
+
+def test_step_assembly_pads_a_decode_step_to_a_recorded_shape():
+    c = make(max_seqs=4)
+    a, b = c.open(), c.open()
+    c.reserve([(a, 17), (b, 3)]); c.advance(a, 17); c.advance(b, 3)
+    c.reserve([(a, 1), (b, 1)])
+    flat, meta = _fill(c, [(a, [40], [0]), (b, [41], [0])], 4, 8)
+    assert meta == (4, 4, 1, 18)
+    want = [40, 41, 0, 0] + [17, 3, 0, 0] + [0, 1, -1, -1] + [a, b, -1, -1] + [0, 1, 2, 3, 4] + [18, 4, 0, 0] + [0, 1, 2, 3]
+    for row in c.page_table(0, [a, b, -1, -1], 8):
+        want += row
+    assert flat == want and want[-8:] == [-1] * 8
+
+
+def test_step_assembly_refuses_what_it_cannot_lay_out():
+    c = make(max_seqs=4)
+    a = c.open()
+    c.reserve([(a, 4)])
+    host = torch.zeros(64, dtype=torch.int32)
+    with pytest.raises(CacheError, match="padded"):
+        c.fill_step([(a, [1, 2], [0])], 4, 2, host.data_ptr(), 64)
+    with pytest.raises(CacheError, match="too small"):
+        c.fill_step([(a, [1, 2, 3, 4], [0])], 0, 2, host.data_ptr(), 5)
+    with pytest.raises(CacheError, match="outside"):
+        c.fill_step([(a, [1, 2], [2])], 0, 2, host.data_ptr(), 64)
+    with pytest.raises(CacheError, match="not open"):
+        c.fill_step([(3, [1], [0])], 0, 2, host.data_ptr(), 64)
+    with pytest.raises(CacheError, match="wider"):
+        c.reserve([(a, 40)])
+        c.fill_step([(a, [1], [0])], 0, 1, host.data_ptr(), 64)
