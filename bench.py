@@ -59,18 +59,30 @@ def time_decode(engine, sampler, batch, context, steps, warmup):
     import torch
     for s in list(engine.cache.live_slots):
         engine.close(s)
-    start = context - (steps + warmup)
+    start = context - (steps + warmup + 1)
     slots = fill_cache(engine, batch, start)
-    toks = [1] * batch
     reqs = list(range(batch))
-    for i in range(warmup):
-        logits = engine.step([(s, [t], [0]) for s, t in zip(slots, toks)])
-        toks = sampler.pick(logits, reqs, [i] * batch)
+    rows = list(range(batch))
+
+    def run(n, first_index, picked):
+        """n decode steps the way the generation loop runs them: the next step starts from the tokens
+        left on the GPU, then the host reads the tokens of the step before."""
+        for i in range(n):
+            logits = engine.step_ahead(slots, rows, picked)
+            if logits is None:      # a shape without a recorded graph yet: the plain step, which records it
+                logits = engine.step([(s, [t], [0]) for s, t in zip(slots, picked.tokens())])
+            nxt = sampler.pick_device(logits, reqs, [first_index + i] * batch)
+            picked.tokens()
+            picked = nxt
+        return picked
+
+    logits = engine.step([(s, [1], [0]) for s in slots])
+    picked = run(warmup, 0, sampler.pick_device(logits, reqs, [0] * batch))
+    picked.tokens()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(steps):
-        logits = engine.step([(s, [t], [0]) for s, t in zip(slots, toks)])
-        toks = sampler.pick(logits, reqs, [warmup + i] * batch)
+    picked = run(steps, warmup, picked)
+    picked.tokens()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     for s in slots:

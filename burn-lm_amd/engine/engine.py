@@ -86,6 +86,29 @@ class Engine:
             self.cache.advance(s, len(t))
         return logits
 
+    def step_ahead(self, slots: Sequence[int], rows: Sequence[int], picked) -> Optional[torch.Tensor]:
+        """One more token for each of the sequences in slots, without the host knowing the tokens
+        yet: sequence i's token is ``picked.device[rows[i]]`` (what a sampler left on the GPU for
+        the step before).  Returns the logits of these tokens, or None, with nothing changed, if
+        the step's shape has no recorded graph (the caller then reads the tokens and uses step()).
+        The logits are the recorded graph's own buffer: work queued on the stream before the next
+        step (a sampler's pick) reads them safely, a caller that keeps them longer must copy them."""
+        if self.graphs is None:
+            return None
+        slots = [int(s) for s in slots]
+        rows = [int(r) for r in rows]
+        if not slots or len(rows) != len(slots) or any(not 0 <= r < picked.device.shape[0] for r in rows):
+            raise StepError("step_ahead needs one row of the picked tokens for every sequence")
+        lengths = [self.cache.length(s) for s in slots]
+        key = self.graphs.key_for([(s, [0], [0]) for s in slots], lengths)
+        if key is None or key not in self.graphs.captured:
+            return None
+        self.cache.reserve([(s, 1) for s in slots])  # raises before any change
+        logits = self.graphs.run_ahead(key, slots, rows, picked.device)
+        for s in slots:
+            self.cache.advance(s, 1)
+        return logits
+
     def build_step(self, entries, lengths):
         from .batch import build_step
         return build_step(entries, lengths, self.cache, self.rt.device)

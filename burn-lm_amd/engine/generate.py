@@ -9,13 +9,18 @@ slots, until every request is served.
 The reference's loop is ``Llama::generate`` (crates/burn-lm-llama/src/generation/generate.rs:
 37-110): one request, ``reset()`` first, prompt step, then one token per step up to
 ``sample_len``, with the stop token found asynchronously by a decoder thread
-(generation/context.rs:142-170) so that one more step may run.  Here the stop is seen on the
-host in the same step and no extra step runs; like the reference the stop token is counted and
-returned but is not text.  Where the reference slides its window when the context is full
-(nn/transformer.rs:156-163), a sequence here ends with the reason ``length``.
+(generation/context.rs:142-170) so that one more step may run.  Like the reference the stop token
+is counted and returned but is not text.  Where the reference slides its window when the
+context is full (nn/transformer.rs:156-163), a sequence here ends with the reason ``length``.
 
 The loop needs of its engine only ``open / close / step / length / max_context / cache`` and of
-its sampler only ``pick``, so its decisions are testable without a GPU.
+its sampler only ``pick``, so its decisions are testable without a GPU.  With those alone the
+stop is seen on the host in the same step and no extra step runs.  If the engine also has
+``step_ahead`` and the sampler ``pick_device``, the loop keeps the GPU busy while the host reads
+tokens: the tokens picked for a step stay on the GPU and feed the next step at once, and the
+host looks at them one step late.  A sequence that met a stop token has then, as in the
+reference, run one step too many, whose token is dropped; ends that are known beforehand
+(``sample_len``, the end of the context) cost no extra step.  The tokens are the same either way.
 """
 from __future__ import annotations
 
@@ -90,9 +95,16 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
     cache = engine.cache
     batches = plan_batches([len(prompts[i]) for i in runnable], sample_len, batch_size, engine.max_context,
                            cache.page_size, cache.n_pages, cache.max_seqs)
+    ahead = hasattr(engine, "step_ahead") and hasattr(sampler, "pick_device")
     for batch in batches:
         ids = [runnable[j] for j in batch]
         live = [(i, engine.open()) for i in ids]
+        open_slots = {slot for _, slot in live}
+
+        def close(slot):
+            open_slots.discard(slot)
+            engine.close(slot)
+
         try:
             t0 = clock()
             logits = engine.step([(slot, list(prompts[i]), [len(prompts[i]) - 1]) for i, slot in live])
@@ -100,14 +112,33 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
             stats.prompt_tokens += sum(len(prompts[i]) for i, _ in live)
             stats.prompt_seconds += clock() - t0
             stats.steps += 1
-            first = True
+            t0 = clock()
+            from_prompt = True
+            dropped = set()     # requests among `live` that ended before the step in flight: their token is ignored
             while True:
-                nxt = []
-                for (i, slot), tok in zip(live, picked):
+                # the step after the one whose tokens are still on their way, for every sequence that
+                # cannot end at that token for a reason known beforehand
+                launched = None
+                if ahead and hasattr(picked, "tokens"):
+                    rows = [k for k, (i, slot) in enumerate(live)
+                            if i not in dropped and len(results[i].tokens) + 1 < sample_len
+                            and engine.length(slot) + 1 <= engine.max_context]
+                    if rows:
+                        logits = engine.step_ahead([live[k][1] for k in rows], rows, picked)
+                        if logits is not None:
+                            nxt = [live[k] for k in rows]
+                            launched = (nxt, sampler.pick_device(logits, [i for i, _ in nxt],
+                                                                 [len(results[i].tokens) + 1 for i, _ in nxt]))
+                            stats.steps += 1
+                tokens = picked.tokens() if hasattr(picked, "tokens") else picked
+                survivors = []
+                for (i, slot), tok in zip(live, tokens):
+                    if i in dropped:
+                        continue
                     r = results[i]
                     r.tokens.append(tok)
                     stats.generated_tokens += 1
-                    if not first:
+                    if not from_prompt:
                         stats.decode_tokens += 1
                     if on_token is not None:
                         on_token(i, tok)
@@ -115,23 +146,29 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
                         r.finish_reason = "stop"
                     elif len(r.tokens) >= sample_len:
                         r.finish_reason = "length"
-                    elif engine.length(slot) + 1 > engine.max_context:
+                    elif engine.length(slot) + (0 if launched and (i, slot) in launched[0] else 1) > engine.max_context:
                         r.finish_reason = "length"
                     if r.finish_reason is None:
-                        nxt.append((i, slot))
+                        survivors.append((i, slot))
                     else:
-                        engine.close(slot)
-                live = nxt
+                        close(slot)
+                from_prompt = False
+                if launched is not None:
+                    live, picked = launched
+                    dropped = {i for i, _ in live if results[i].finish_reason is not None}
+                    if len(dropped) == len(live):
+                        break
+                    continue
+                live, dropped = survivors, set()
                 if not live:
                     break
-                first = False
-                t0 = clock()
                 logits = engine.step([(slot, [results[i].tokens[-1]], [0]) for i, slot in live])
-                picked = sampler.pick(logits, [i for i, _ in live], [len(results[i].tokens) for i, _ in live])
-                stats.decode_seconds += clock() - t0
+                requests, indices = [i for i, _ in live], [len(results[i].tokens) for i, _ in live]
+                picked = sampler.pick_device(logits, requests, indices) if ahead else sampler.pick(logits, requests, indices)
                 stats.steps += 1
+            stats.decode_seconds += clock() - t0
         except BaseException:
-            for _, slot in live:
+            for slot in list(open_slots):
                 try:
                     engine.close(slot)
                 except Exception:

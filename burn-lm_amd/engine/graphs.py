@@ -43,9 +43,11 @@ class _Captured:
         G = len(cache.groups)
         self.B, self.W = B, W
         self.copied = None
-        n = 7 * B + 1 + G * B * W
-        self.host = torch.zeros(n, dtype=torch.int32).pin_memory()
-        self.dev = torch.zeros(n, dtype=torch.int32, device=dev)
+        n = 7 * B + 1 + G * B * W          # the step's index arrays ...
+        self.src_at = n                    # ... and behind them, for run_ahead, where each row's token comes from
+        self.host = torch.zeros(n + B, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(n + B, dtype=torch.int32, device=dev)
         o = 0
 
         def take(k):
@@ -57,6 +59,7 @@ class _Captured:
         token_ids, positions, token_seq, seq_slots = take(B), take(B), take(B), take(B)
         cu, after, rows = take(B + 1), take(B), take(B)
         tables = {gi: take(B * W).view(B, W) for gi in range(G)}
+        self.src_rows = take(B)
         span = min(W * cache.page_size, cache.max_context)
         self.step = Step(n_tokens=B, n_seqs=B, n_wanted=B, token_ids=token_ids, positions=positions,
                          token_seq=token_seq, seq_slots=seq_slots, cu_seqlens=cu, lens_after=after, want_rows=rows,
@@ -83,12 +86,12 @@ class _Captured:
         written by the native core straight into the pinned buffer."""
         B, W = self.B, self.W
         if entries:
-            cache.fill_step(entries, B, W, self.host.data_ptr(), self.host.numel())
+            cache.fill_step(entries, B, W, self.host.data_ptr(), self.src_at)
             return
         # all padding (used while recording): token 0, position 0, no sequence, no slot, no pages
         flat = [0] * B + [0] * B + [-1] * B + [-1] * B + list(range(B + 1)) + [0] * B + list(range(B))
         flat += [-1] * (len(cache.groups) * B * W)
-        self.host.copy_(torch.tensor(flat, dtype=torch.int32))
+        self.host[: self.src_at].copy_(torch.tensor(flat, dtype=torch.int32))
 
     def run(self, entries, lengths, cache):
         if self.copied is not None:
@@ -99,6 +102,21 @@ class _Captured:
         self.copied.record()
         self.graph.replay()
         return self.logits[: len(entries)].clone()   # the graph's own output buffer is overwritten by the next replay
+
+    def run_ahead(self, slots, rows, tokens_dev, cache):
+        """Like run(), but row i's token is tokens_dev[rows[i]], taken on the device: the host
+        need not have seen the tokens of the step before.  The logits come back without a copy."""
+        if self.copied is not None:
+            self.copied.synchronize()
+        n = len(slots)
+        self.fill([(s, [0], [0]) for s in slots], None, cache)
+        self.host_np[self.src_at: self.src_at + n] = rows
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        torch.index_select(tokens_dev, 0, self.src_rows[:n], out=self.step.token_ids[:n])
+        self.graph.replay()
+        return self.logits[:n]      # the graph's own buffer: good until the next replay of this shape
 
 
 class DecodeGraphs:
@@ -131,6 +149,14 @@ class DecodeGraphs:
             return None
         self.replays += 1
         return c.run(entries, lengths, self._engine().cache)
+
+    def run_ahead(self, key, slots, rows, tokens_dev):
+        """Replays a recorded shape with the tokens taken on the device; None if it is not recorded."""
+        c = self.captured.get(key)
+        if c is None:
+            return None
+        self.replays += 1
+        return c.run_ahead(slots, rows, tokens_dev, self._engine().cache)
 
     def after_eager(self, key):
         """The shape has just run eagerly (so every kernel and library handle it needs exists):

@@ -31,6 +31,23 @@ def uniform(seed: int, request: int, index: int) -> float:
     return (x >> 40) / float(1 << 24)
 
 
+class Picked:
+    """The tokens picked for the rows of one step.  ``device`` (int32 [rows], on the GPU) can feed
+    the next step without the host having seen the tokens; ``tokens()`` waits for their copy to
+    the host, which was started when they were picked, and returns them as a list."""
+
+    def __init__(self, device_tokens: torch.Tensor):
+        self.device = device_tokens
+        self._host = torch.empty(device_tokens.shape, dtype=device_tokens.dtype, pin_memory=True)
+        self._host.copy_(device_tokens, non_blocking=True)
+        self._done = torch.cuda.Event()
+        self._done.record()
+
+    def tokens(self) -> List[int]:
+        self._done.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
     """temperature == 0: greedy, lowest index wins ties.  temperature > 0: temperature softmax,
     nucleus of mass top_p (1.0 keeps everything), inverse-CDF draw."""
@@ -52,8 +69,9 @@ class Sampler:
     def uniforms(self, requests: Sequence[int], indices: Sequence[int]) -> List[float]:
         return [uniform(self.seed, r, i) for r, i in zip(requests, indices)]
 
-    def pick(self, logits: torch.Tensor, requests: Sequence[int], indices: Sequence[int]) -> List[int]:
-        """logits float32 [rows, vocab] on the GPU -> one token per row, as host integers."""
+    def pick_device(self, logits: torch.Tensor, requests: Sequence[int], indices: Sequence[int]) -> Picked:
+        """logits float32 [rows, vocab] on the GPU -> one token per row, left on the GPU; nothing here
+        waits for the GPU."""
         ops = self._ops
         if ops is None:
             from ..csrc import ops
@@ -61,6 +79,11 @@ class Sampler:
         if self.greedy:
             out = ops.argmax(logits)
         else:
-            u = torch.tensor(self.uniforms(requests, indices), dtype=torch.float32).to(logits.device)
-            out = ops.sample(logits, u, self.temperature, self.top_p)
-        return out.tolist()
+            # through pinned memory, so that the copy does not wait for the work already queued
+            u = torch.tensor(self.uniforms(requests, indices), dtype=torch.float32).pin_memory()
+            out = ops.sample(logits, u.to(logits.device, non_blocking=True), self.temperature, self.top_p)
+        return Picked(out)
+
+    def pick(self, logits: torch.Tensor, requests: Sequence[int], indices: Sequence[int]) -> List[int]:
+        """logits float32 [rows, vocab] on the GPU -> one token per row, as host integers."""
+        return self.pick_device(logits, requests, indices).tokens()

@@ -166,3 +166,78 @@ def test_sampler_is_told_request_and_token_index():
     s = HostArgmax()
     generate(eng, [[1], [20], [3]], s, sample_len=4, stop_ids=[expected([20], 4)[1]], batch_size=4)
     assert s.last == ([0, 2], [3, 3])
+
+
+class AheadEngine(ToyEngine):
+    """A stand-in with step_ahead: a shape (number of sequences) can run ahead once a plain decode
+    step of that shape has run, as a recorded graph would allow."""
+
+    def __init__(self, **kw):
+        super().__init__(**kw)
+        self.recorded, self.ahead_steps = set(), 0
+
+    def step(self, entries):
+        if all(len(t) == 1 for _, t, _ in entries):
+            self.recorded.add(len(entries))
+        return super().step(entries)
+
+    def step_ahead(self, slots, rows, picked):
+        if len(slots) not in self.recorded:
+            return None
+        self.ahead_steps += 1
+        toks = picked.tokens()      # the stand-in may look; the real engine takes them on the device
+        return super().step([(s, [toks[r]], [0]) for s, r in zip(slots, rows)])
+
+
+class ToyPicked:
+    def __init__(self, toks):
+        self._toks = toks
+        self.read = False
+
+    def tokens(self):
+        self.read = True
+        return list(self._toks)
+
+
+class AheadArgmax(HostArgmax):
+    def pick_device(self, logits, requests, indices):
+        self.calls = getattr(self, "calls", []) + [(list(requests), list(indices))]
+        return ToyPicked(self.pick(logits, requests, indices))
+
+
+def test_running_ahead_gives_the_same_tokens_and_at_most_one_dropped_step_per_stop():
+    prompts = [[1, 2, 3], [5, 5], [9], [2, 7, 1, 1]]
+    free = [expected(p, 9) for p in prompts]
+    stop = free[1][2]
+    want = [expected(p, 9, stop=(stop,)) for p in prompts]
+    plain_eng = ToyEngine()
+    plain, _ = generate(plain_eng, prompts, HostArgmax(), sample_len=9, stop_ids=[stop], batch_size=4)
+    eng, sampler = AheadEngine(), AheadArgmax()
+    res, stats = generate(eng, prompts, sampler, sample_len=9, stop_ids=[stop], batch_size=4)
+    assert [r.tokens for r in res] == want == [r.tokens for r in plain]
+    assert [r.finish_reason for r in res] == [r.finish_reason for r in plain]
+    assert eng.ahead_steps > 0, "no step ran ahead"
+    # a sequence that met its stop token was in one more step than without running ahead; one that
+    # ended at sample_len was not
+    def steps_of(e, k):
+        return sum(1 for st in e.steps for s, _ in st if s == e.opened[k])
+    for k, r in enumerate(res):
+        extra = steps_of(eng, k) - steps_of(plain_eng, k)
+        assert extra == (1 if r.finish_reason == "stop" else 0), (k, r.finish_reason, extra)
+    assert stats.generated_tokens == sum(len(w) for w in want)
+    assert stats.decode_tokens == stats.generated_tokens - len(prompts)
+    # the random number of a draw is that of the token's index in its request, also when picked ahead
+    for requests, indices in sampler.calls:
+        assert len(requests) == len(indices)
+    assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 4
+
+
+def test_running_ahead_stops_at_the_end_of_the_context_without_an_extra_step():
+    eng = AheadEngine(max_context=12, max_tokens=64)
+    res, _ = generate(eng, [[1] * 10, [3]], AheadArgmax(), sample_len=50, batch_size=4)
+    assert res[0].finish_reason == "length" and res[0].tokens == expected([1] * 10, 3)
+    assert res[1].finish_reason == "length" and len(res[1].tokens) == 12
+    assert eng.cache.pages_in_use() == 0
+    assert max(n for st in eng.steps for _, n in st if n == 1) == 1
+    for s in eng.opened:
+        assert s not in eng.cache.live_slots
