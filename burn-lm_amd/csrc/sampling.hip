@@ -1,9 +1,18 @@
-// Token choice from float logits, one block per row.
-//   argmax : first index of the maximum (lowest index wins ties).
+// Token choice from float logits.
+//   argmax : first index of the maximum (lowest index wins ties); a row is searched by 32 blocks.
 //   sample : softmax(logits / temperature) in float, nucleus (top-p) cut, inverse-CDF pick at a
-//            uniform number u given by the caller, walking the kept tokens in index order.
+//            uniform number u given by the caller, walking the kept tokens in index order; one
+//            block per row.
 // Nucleus rule: a token is kept while the probability mass of the tokens strictly more likely
 // than it is below p; so the token that crosses p is kept, and tokens tied with it are too.
+//
+// The weight of a token is e = 2^((x - max) * log2(e) / temperature), in (0, 1].  The smallest
+// kept weight is found by a radix selection over the bit pattern of e (positive floats order like
+// their bits): three passes over the row with histograms of 11, 11 and 8 bits, each bin holding
+// the mass of its tokens.  Mass is summed as 64-bit integers (e * 2^32, truncated), so the sums do
+// not depend on the order in which the shared-memory atomics land and the same logits always give
+// the same cut; a token lighter than 2^-32 of the heaviest one counts as no mass.  The pick then
+// walks the kept tokens in index order: every wavefront owns a contiguous range of the row.
 #include "common.h"
 
 #define SMP_THREADS 1024
@@ -70,79 +79,276 @@ extern "C" int blm_argmax(const float* logits, int* out, int R, int V, int ld, f
   return 0;
 }
 
+#define SMP_BINS 2048
+#define SMP_MAX_CHUNKS 256   // chunks of 256 elements per wavefront: rows of up to 16 * 256 * 256 elements
+
+// All elements of a row, coalesced: with VEC four consecutive floats per lane, and four such loads
+// in flight per lane (a loop that waits for every load in turn spends a memory round trip on each).
+// Places past the row's end read as -infinity, which BODY must take as "no token".
+#define SMP_FOR_EACH(BODY)                                                                          \
+  if (VEC) {                                                                                        \
+    const float4* x4 = reinterpret_cast<const float4*>(x);                                          \
+    const int n4 = V / 4;                                                                           \
+    for (int i4 = tid; i4 < n4; i4 += 4 * SMP_THREADS) {                                            \
+      float4 v4[4];                                                                                 \
+      _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                               \
+        const int j = i4 + u * SMP_THREADS;                                                         \
+        v4[u] = j < n4 ? x4[j] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);           \
+      }                                                                                             \
+      _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                               \
+        { const float xv = v4[u].x; BODY }                                                          \
+        { const float xv = v4[u].y; BODY }                                                          \
+        { const float xv = v4[u].z; BODY }                                                          \
+        { const float xv = v4[u].w; BODY }                                                          \
+      }                                                                                             \
+    }                                                                                               \
+    if (tid < (V & 3)) { const float xv = x[(V & ~3) + tid]; BODY }                                 \
+  } else {                                                                                          \
+    for (int i = tid; i < V; i += 4 * SMP_THREADS) {                                                \
+      float v1[4];                                                                                  \
+      _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                               \
+        const int j = i + u * SMP_THREADS;                                                          \
+        v1[u] = j < V ? x[j] : -INFINITY;                                                           \
+      }                                                                                             \
+      _Pragma("unroll") for (int u = 0; u < 4; ++u) { const float xv = v1[u]; BODY }                \
+    }                                                                                               \
+  }
+
+__device__ __forceinline__ unsigned long long shfl_down_u64(unsigned long long v, int d) {
+  const uint32_t lo = __shfl_down((uint32_t)v, d, BLM_WAVE), hi = __shfl_down((uint32_t)(v >> 32), d, BLM_WAVE);
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+// The lowest bin b of hist[0 .. SMP_BINS) with carry + (mass of the bins above b) < target, and
+// that sum for it.  Every thread gets both.  Thread t looks after bins 2t and 2t + 1.
+__device__ __forceinline__ void lowest_bin_below(const unsigned long long* hist, unsigned long long carry,
+                                                 unsigned long long target, unsigned long long* wave_tot, int* found,
+                                                 int& bin, unsigned long long& above) {
+  const int tid = threadIdx.x, lane = tid & (BLM_WAVE - 1), w = tid / BLM_WAVE;
+  const unsigned long long m0 = hist[2 * tid], m1 = hist[2 * tid + 1];
+  unsigned long long suf = m0 + m1;   // becomes the mass of this thread's bins and of all higher threads' bins
+#pragma unroll
+  for (int d = 1; d < BLM_WAVE; d <<= 1) {
+    const unsigned long long o = shfl_down_u64(suf, d);
+    if (lane + d < BLM_WAVE) suf += o;
+  }
+  if (tid == 0) *found = 0x7fffffff;
+  if (lane == 0) wave_tot[w] = suf;
+  __syncthreads();
+  for (int k = w + 1; k < SMP_THREADS / BLM_WAVE; ++k) suf += wave_tot[k];
+  const unsigned long long above1 = carry + suf - m0 - m1;   // above bin 2t + 1
+  const unsigned long long above0 = above1 + m1;             // above bin 2t
+  if (above0 < target) atomicMin(found, 2 * tid);
+  else if (above1 < target) atomicMin(found, 2 * tid + 1);
+  __syncthreads();
+  bin = *found;
+  // the thread that owns the bin publishes its sum through wave_tot[0] (all reads of it are done)
+  if (bin == 2 * tid) wave_tot[0] = above0;
+  if (bin == 2 * tid + 1) wave_tot[0] = above1;
+  __syncthreads();
+  above = wave_tot[0];
+  __syncthreads();
+}
+
+template <bool VEC>
 __global__ void __launch_bounds__(SMP_THREADS)
-    sample_kernel(const float* __restrict__ logits, const float* __restrict__ uniforms,
-                  int* __restrict__ out, int V, int ld, float inv_temperature, float top_p) {
+    sample_kernel(const float* __restrict__ logits, const float* __restrict__ uniforms, int* __restrict__ out, int V,
+                  int ld, float k2, float top_p) {
+  __shared__ unsigned long long hist[SMP_BINS];
+  __shared__ unsigned long long wave_tot[SMP_THREADS / BLM_WAVE];
   __shared__ float red[17];
-  __shared__ float seg[SMP_THREADS];
-  __shared__ int pick[2];
+  __shared__ float wsum[SMP_THREADS / BLM_WAVE];
+  __shared__ int found, pick, last_kept;
   const float* x = logits + (size_t)blockIdx.x * ld;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & (BLM_WAVE - 1), w = tid / BLM_WAVE;
 
   float mx = -INFINITY;
-  for (int i = tid; i < V; i += blockDim.x) mx = fmaxf(mx, x[i]);
+  SMP_FOR_EACH(mx = fmaxf(mx, xv);)
   mx = block_max(mx, red);
 
-  float z = 0.f;
-  for (int i = tid; i < V; i += blockDim.x) z += expf((x[i] - mx) * inv_temperature);
-  z = block_sum(z, red);
-
-  // smallest kept weight tau: the smallest float t with mass{e > t} < top_p * z
-  float tau = 0.f;
+  // smallest kept weight, as a bit pattern; 0 keeps everything
+  uint32_t tau = 0u;
   if (top_p < 1.0f) {
-    const float target = top_p * z;
-    uint32_t lo = 0u, hi = 0x3f800000u;  // e <= 1, so mass{e > 1} = 0 < target
-    // f(0) >= target unless everything underflowed; then tau collapses to the smallest float
-    while (hi - lo > 1u) {
-      const uint32_t mid = lo + ((hi - lo) >> 1);
-      const float t = __uint_as_float(mid);
-      float mass = 0.f;
-      for (int i = tid; i < V; i += blockDim.x) {
-        const float e = expf((x[i] - mx) * inv_temperature);
-        mass += e > t ? e : 0.f;
+    unsigned long long carry = 0ull, target = 0ull;
+    uint32_t prefix = 0u;
+    // bits 29..19, then 18..8, then 7..0 (e <= 1, so bits 31 and 30 are clear)
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 19 : (level == 1 ? 8 : 0);
+      const uint32_t mask = level == 2 ? 0xffu : 0x7ffu;
+      hist[2 * tid] = 0ull;
+      hist[2 * tid + 1] = 0ull;
+      __syncthreads();
+      SMP_FOR_EACH(
+        const float e = __builtin_amdgcn_exp2f((xv - mx) * k2);
+        const uint32_t key = __float_as_uint(e);
+        // the digits above this level must be the ones already chosen (none at the first level)
+        if (level == 0 || (key >> (shift + (level == 1 ? 11 : 8))) == prefix) {
+          const unsigned long long q = (unsigned long long)(e * 4294967296.0f);
+          if (q) atomicAdd(&hist[(key >> shift) & mask], q);
+        }
+      )
+      __syncthreads();
+      if (level == 0) {
+        // the whole mass: what every bin holds
+        unsigned long long z = hist[2 * tid] + hist[2 * tid + 1];
+#pragma unroll
+        for (int d = 1; d < BLM_WAVE; d <<= 1) {
+          const unsigned long long o = shfl_down_u64(z, d);
+          if (lane + d < BLM_WAVE) z += o;
+        }
+        if (lane == 0) wave_tot[w] = z;
+        __syncthreads();
+        unsigned long long total = 0ull;
+        for (int k = 0; k < SMP_THREADS / BLM_WAVE; ++k) total += wave_tot[k];
+        __syncthreads();
+        target = (unsigned long long)((double)top_p * (double)total);
+        if (target < 1ull) target = 1ull;
       }
-      mass = block_sum(mass, red);
-      if (mass < target) hi = mid; else lo = mid;
+      int bin;
+      unsigned long long above;
+      lowest_bin_below(hist, carry, target, wave_tot, &found, bin, above);
+      carry = above;
+      prefix = (prefix << (level == 2 ? 8 : 11)) | (uint32_t)bin;
     }
-    tau = __uint_as_float(hi);
+    tau = prefix;
   }
 
-  // contiguous segment per thread, so the walk is in index order
-  const int per = (V + blockDim.x - 1) / blockDim.x;
-  const int beg = tid * per, end = min(V, beg + per);
+  // The pick, in index order.  Wavefront w owns elements [w * span, (w + 1) * span), span a
+  // multiple of 256; it reads them 256 at a time, lane l the four from offset 4 l of each chunk,
+  // and remembers the kept mass of every chunk (chunk c in lane c % 64, register c / 64).
+  const int span = (((V + SMP_THREADS / BLM_WAVE - 1) / (SMP_THREADS / BLM_WAVE)) + 255) / 256 * 256;
+  const int begin = w * span, end = min(V, begin + span);
+  const int n_chunks = end > begin ? (end - begin + 255) / 256 : 0;   // at most SMP_MAX_CHUNKS (checked on the host)
+  float chunk_mass[SMP_MAX_CHUNKS / BLM_WAVE];
+#pragma unroll
+  for (int g = 0; g < SMP_MAX_CHUNKS / BLM_WAVE; ++g) chunk_mass[g] = 0.f;
+  int my_last = -1;
+  // kept weights of the four elements of this lane in chunk ci (0 where there is no kept token)
+#define SMP_LOAD_CHUNK(ci, xs)                                                                       \
+  {                                                                                                 \
+    const int i0_ = begin + (ci) * 256 + lane * 4;                                                  \
+    if (VEC && i0_ + 3 < end) {                                                                     \
+      const float4 v4_ = *reinterpret_cast<const float4*>(x + i0_);                                 \
+      xs[0] = v4_.x; xs[1] = v4_.y; xs[2] = v4_.z; xs[3] = v4_.w;                                   \
+    } else {                                                                                        \
+      _Pragma("unroll") for (int k = 0; k < 4; ++k) xs[k] = i0_ + k < end ? x[i0_ + k] : -INFINITY; \
+    }                                                                                               \
+  }
+#define SMP_KEPT(xv) ([&](float v_) { const float e_ = __builtin_amdgcn_exp2f((v_ - mx) * k2); \
+                                      return (__float_as_uint(e_) >= tau && e_ > 0.f) ? e_ : 0.f; }(xv))
+  for (int c0 = 0; c0 < n_chunks; c0 += 4) {
+    float xs[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (c0 + u < n_chunks) { SMP_LOAD_CHUNK(c0 + u, xs[u]) }
+      else { xs[u][0] = xs[u][1] = xs[u][2] = xs[u][3] = -INFINITY; }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int ci = c0 + u;
+      float s4 = 0.f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float e = SMP_KEPT(xs[u][k]);
+        s4 += e;
+        if (e > 0.f) my_last = begin + ci * 256 + lane * 4 + k;
+      }
+      const float t = wave_sum(s4);
+#pragma unroll
+      for (int g = 0; g < SMP_MAX_CHUNKS / BLM_WAVE; ++g)
+        if (ci < n_chunks && (ci >> 6) == g && (ci & 63) == lane) chunk_mass[g] = t;
+    }
+  }
+  // mass of the wavefront's range: its chunks in order
   float mine = 0.f;
-  int last_kept = -1;
-  for (int i = beg; i < end; ++i) {
-    const float e = expf((x[i] - mx) * inv_temperature);
-    if (e >= tau) { mine += e; last_kept = i; }
+#pragma unroll
+  for (int g = 0; g < SMP_MAX_CHUNKS / BLM_WAVE; ++g) {
+    float incl = chunk_mass[g];
+#pragma unroll
+    for (int d = 1; d < BLM_WAVE; d <<= 1) {
+      const float o = __shfl_up(incl, d, BLM_WAVE);
+      if (lane >= d) incl += o;
+    }
+    mine += __shfl(incl, BLM_WAVE - 1, BLM_WAVE);
   }
-  seg[tid] = mine;
-  if (tid == 0) { pick[0] = 0x7fffffff; pick[1] = -1; }
+  if (tid == 0) { pick = 0x7fffffff; last_kept = -1; }
   __syncthreads();
-  if (tid == 0) {  // exclusive prefix over 1024 segment sums, in order
-    float run = 0.f;
-    for (int k = 0; k < (int)blockDim.x; ++k) { const float s = seg[k]; seg[k] = run; run += s; }
-    red[0] = run;
+  if (lane == 0) wsum[w] = mine;
+  if (my_last >= 0) atomicMax(&last_kept, my_last);
+  __syncthreads();
+  float total = 0.f, before = 0.f;
+  for (int k = 0; k < SMP_THREADS / BLM_WAVE; ++k) {
+    if (k == w) before = total;
+    total += wsum[k];
   }
-  __syncthreads();
-  const float total = red[0];
   const float want = uniforms[blockIdx.x] * total;
-  if (last_kept >= 0) atomicMax(&pick[1], last_kept);
-  const float before = seg[tid];
-  if (mine > 0.f && want >= before && want < before + mine) {
-    float run = before;
-    int chosen = last_kept;
-    for (int i = beg; i < end; ++i) {
-      const float e = expf((x[i] - mx) * inv_temperature);
-      if (e >= tau) {
-        run += e;
-        if (want < run) { chosen = i; break; }
+  if (mine > 0.f && want >= before && want < before + mine) {   // at most one wavefront
+    // which chunk: the first whose running mass passes want
+    float acc = before;
+    int chunk = -1;
+#pragma unroll
+    for (int g = 0; g < SMP_MAX_CHUNKS / BLM_WAVE; ++g) {
+      if (chunk >= 0) continue;
+      float incl = chunk_mass[g];
+#pragma unroll
+      for (int d = 1; d < BLM_WAVE; d <<= 1) {
+        const float o = __shfl_up(incl, d, BLM_WAVE);
+        if (lane >= d) incl += o;
+      }
+      const float group_total = __shfl(incl, BLM_WAVE - 1, BLM_WAVE);
+      const unsigned long long hits = __ballot(chunk_mass[g] > 0.f && want < acc + incl);
+      if (hits) {
+        const int first = __ffsll((long long)hits) - 1;
+        chunk = g * 64 + first;
+        acc += __shfl(incl - chunk_mass[g], first, BLM_WAVE);
+      } else {
+        acc += group_total;
       }
     }
-    atomicMin(&pick[0], chosen);
+    if (chunk >= 0) {
+      float xs[4], es[4];
+      SMP_LOAD_CHUNK(chunk, xs)
+      float s4 = 0.f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { es[k] = SMP_KEPT(xs[k]); s4 += es[k]; }
+      float incl = s4;   // inclusive prefix over the lanes, in lane order
+#pragma unroll
+      for (int d = 1; d < BLM_WAVE; d <<= 1) {
+        const float o = __shfl_up(incl, d, BLM_WAVE);
+        if (lane >= d) incl += o;
+      }
+      unsigned long long hits = __ballot(s4 > 0.f && want < acc + incl);
+      const unsigned long long have = __ballot(s4 > 0.f);
+      if (!hits && have) hits = 1ull << (63 - __clzll((long long)have));   // rounding: the chunk's last lane with a kept token
+      if (hits) {
+        const int first = __ffsll((long long)hits) - 1;
+        if (lane == first) {
+          const int i0 = begin + chunk * 256 + lane * 4;
+          float run = acc + incl - s4;
+          int chosen = -1, last = -1;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (es[k] > 0.f) {
+              run += es[k];
+              last = i0 + k;
+              if (want < run && chosen < 0) chosen = i0 + k;
+            }
+          }
+          atomicMin(&pick, chosen >= 0 ? chosen : last);   // rounding may leave want at the lane's upper edge
+        }
+      }
+    } else {
+      // rounding left want at the upper edge of the wavefront's range: its last kept token
+      int m = my_last;
+#pragma unroll
+      for (int d = BLM_WAVE / 2; d > 0; d >>= 1) m = max(m, __shfl_xor(m, d, BLM_WAVE));
+      if (lane == 0 && m >= 0) atomicMin(&pick, m);
+    }
   }
+#undef SMP_LOAD_CHUNK
+#undef SMP_KEPT
   __syncthreads();
-  if (tid == 0) out[blockIdx.x] = pick[0] != 0x7fffffff ? pick[0] : (pick[1] >= 0 ? pick[1] : 0);
+  if (tid == 0) out[blockIdx.x] = pick != 0x7fffffff ? pick : (last_kept >= 0 ? last_kept : 0);
 }
 
 extern "C" int blm_sample(const float* logits, const float* uniforms, int* out, int R, int V, int ld,
@@ -150,8 +356,14 @@ extern "C" int blm_sample(const float* logits, const float* uniforms, int* out, 
   BLM_REQUIRE(R > 0 && V > 0 && ld >= V, "sample: bad sizes R=%d V=%d ld=%d", R, V, ld);
   BLM_REQUIRE(temperature > 0.f, "sample: temperature must be > 0 (got %g); use argmax for 0", (double)temperature);
   BLM_REQUIRE(top_p > 0.f, "sample: top_p must be > 0 (got %g)", (double)top_p);
-  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SMP_THREADS), 0, stream, logits, uniforms, out, V, ld,
-                     1.0f / temperature, top_p);
+  BLM_REQUIRE(V <= (SMP_THREADS / BLM_WAVE) * SMP_MAX_CHUNKS * 256, "sample: a vocabulary of %d is more than %d", V,
+              (SMP_THREADS / BLM_WAVE) * SMP_MAX_CHUNKS * 256);
+  const float k2 = 1.4426950408889634f / temperature;
+  const bool vec = ld % 4 == 0 && ((uintptr_t)logits % 16) == 0;
+  if (vec)
+    hipLaunchKernelGGL(sample_kernel<true>, dim3(R), dim3(SMP_THREADS), 0, stream, logits, uniforms, out, V, ld, k2, top_p);
+  else
+    hipLaunchKernelGGL(sample_kernel<false>, dim3(R), dim3(SMP_THREADS), 0, stream, logits, uniforms, out, V, ld, k2, top_p);
   BLM_LAUNCH_CHECK("sample");
   return 0;
 }
