@@ -544,6 +544,35 @@ def test_sample_top_p_keeps_the_nucleus_only(ops):
     assert int(out[3]) == 40000 and all(0 <= int(t) < 50257 for t in out)
 
 
+@pytest.mark.parametrize("V,ld", [(128256, 128256), (32003, 32003), (50257, 50260)])
+def test_sample_large_vocabulary_matches_the_ordered_nucleus(ops, V, ld):
+    """Vocabularies of real size (a multiple of four, an odd one that takes the scalar loads, a padded
+    row stride): every draw lies in the plain implementation's nucleus and is the token at which the
+    cumulative mass of the kept tokens, in index order, passes u; the same inputs give the same draws."""
+    import plain_llama as P
+    g = torch.Generator().manual_seed(41)
+    R, T, p = 512, 0.8, 0.9
+    logits = torch.randn(V, generator=g) * 2.5
+    probs = P.temperature_softmax(logits.double().numpy(), T)
+    kept = np.array(sorted(P.top_p_keep(probs, p)))
+    cdf = np.cumsum(probs[kept]) / probs[kept].sum()
+    u = torch.rand(R, generator=g)
+    wide = torch.full((R, ld), 1e9)              # beyond the vocabulary: must not be looked at
+    wide[:, :V] = logits
+    x = dev(wide)[:, :V]
+    got = ops.sample(x, dev(u), T, p).cpu().numpy()
+    assert set(got.tolist()) <= set(kept.tolist()), "a token outside the nucleus was drawn"
+    want = kept[np.minimum(np.searchsorted(cdf, u.double().numpy(), side="right"), len(kept) - 1)]
+    assert (want == got).mean() > 0.99, f"{(want != got).sum()} of {R} draws differ from the ordered inverse CDF"
+    again = ops.sample(x, dev(u), T, p).cpu().numpy()
+    assert (again == got).all()
+    # p = 1 keeps everything
+    full = ops.sample(x, dev(u), T, 1.0).cpu().numpy()
+    cdf1 = np.cumsum(probs)
+    want1 = np.minimum(np.searchsorted(cdf1, u.double().numpy() * cdf1[-1], side="right"), V - 1)
+    assert (want1 == full).mean() > 0.98
+
+
 @pytest.mark.parametrize("pairing", ["interleaved", "half"])
 @pytest.mark.parametrize("M,K,nh,nkv,hd", [(8, 2048, 4, 2, 64), (5, 264, 3, 1, 32), (16, 3072, 2, 2, 128), (1, 64, 6, 3, 64)])
 def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
