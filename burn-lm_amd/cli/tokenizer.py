@@ -4,7 +4,9 @@
 (crates/burn-lm-llama/src/tokenizer/byte.rs:3-49: bos 0, eos 1, stop ids [2]); it needs a
 vocabulary of at least 256.  Where the reference prints the id list on decode (byte.rs:34-36),
 this one gives the bytes back as text.  A ``tokenizer.json`` in the model folder is used instead
-when the ``tokenizers`` package can read it."""
+when the ``tokenizers`` package can read it; its stop ids are those of the special tokens the
+reference's Llama-3 tokenizer stops at (crates/burn-lm-llama/src/tokenizer/tiktoken.rs:12-15,
+126-132), as far as the file defines them."""
 from __future__ import annotations
 
 import os
@@ -26,18 +28,28 @@ class ByteTokenizer:
 
 
 class FileTokenizer:
+    BOS, EOS = "<|begin_of_text|>", "<|end_of_text|>"
+    STOPS = ("<|end_of_text|>", "<|eom_id|>", "<|eot_id|>")
+
     def __init__(self, path):
         from tokenizers import Tokenizer
         self._tok = Tokenizer.from_file(path)
+        self.bos_id, self.eos_id = self._tok.token_to_id(self.BOS), self._tok.token_to_id(self.EOS)
 
     def encode(self, text, bos=False, eos=False):
-        return self._tok.encode(text, add_special_tokens=False).ids
+        ids = self._tok.encode(text, add_special_tokens=False).ids
+        if bos and self.bos_id is not None:
+            ids = [self.bos_id] + ids
+        if eos and self.eos_id is not None:
+            ids = ids + [self.eos_id]
+        return ids
 
     def decode(self, tokens):
         return self._tok.decode(list(tokens), skip_special_tokens=True)
 
     def stop_ids(self):
-        return []
+        ids = [self._tok.token_to_id(t) for t in self.STOPS]
+        return [i for i in ids if i is not None]
 
 
 def for_folder(folder: str, vocab_size: int):

@@ -122,10 +122,11 @@ class InferenceServer:
 
     # ---- work --------------------------------------------------------------------------------
     def stop_ids(self):
-        ids = list(self.engine.model.plan.stop_ids)
-        if not ids and self.tokenizer is not None:
-            ids = list(self.tokenizer.stop_ids())
-        return ids
+        """The configuration's end-of-sequence ids and the tokenizer's stop ids together."""
+        ids = set(self.engine.model.plan.stop_ids)
+        if self.tokenizer is not None:
+            ids.update(self.tokenizer.stop_ids())
+        return sorted(ids)
 
     def generate(self, prompts: Sequence[Sequence[int]], on_token: Optional[Callable[[int, int], None]] = None,
                  stop_ids: Optional[Sequence[int]] = None, **options):

@@ -114,3 +114,25 @@ def test_presets_are_valid_configurations():
     assert (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads,
             c.intermediate_size, c.vocab_size) == (2048, 16, 32, 8, 8192, 128256)
     assert c.rope_scaling.factor == 32.0 and c.rope_theta == 500000.0
+
+
+def test_tokenizers_for_the_command_line(tmp_path):
+    """Bytes by default; a tokenizer.json in the model folder is used when there is one, with the
+    stop ids of the special tokens it defines (tiktoken.rs:12-15, 126-132)."""
+    from burn_lm_amd.cli.tokenizer import ByteTokenizer, FileTokenizer, for_folder
+    t = for_folder(str(tmp_path), 256)
+    assert isinstance(t, ByteTokenizer) and t.decode(t.encode("héllo")) == "héllo" and t.stop_ids() == [2]
+    assert t.encode("a", bos=True, eos=True) == [0, 97, 1]
+    with pytest.raises(ValueError, match="at least 256"):
+        for_folder(str(tmp_path), 100)
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    vocab = {"hello": 0, "world": 1, "[UNK]": 2, "<|begin_of_text|>": 3, "<|end_of_text|>": 4, "<|eot_id|>": 5}
+    tok = Tokenizer(models.WordLevel(vocab, unk_token="[UNK]"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.add_special_tokens(["<|begin_of_text|>", "<|end_of_text|>", "<|eot_id|>"])
+    tok.save(str(tmp_path / "tokenizer.json"))
+    f = for_folder(str(tmp_path), 6)
+    assert isinstance(f, FileTokenizer)
+    assert f.encode("hello world") == [0, 1] and f.encode("hello", bos=True, eos=True) == [3, 0, 4]
+    assert f.stop_ids() == [4, 5]            # <|eom_id|> is not in this file
+    assert f.decode([3, 0, 1, 5]) == "hello world"
