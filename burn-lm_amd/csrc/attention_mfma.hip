@@ -21,6 +21,7 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
 
 #define AM_WAVES 4
 #define AM_PAGE 64
@@ -181,11 +182,16 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
                              float scale, int window) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
-  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 8;
+  // row strides in shared memory: keys are read 16 bytes per lane from 16 rows (stride = 16 bytes mod
+  // 128 keeps the 32 banks apart), values 8 bytes per lane from 16 rows (stride = 8 bytes mod 128)
+  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 4;
   constexpr int CHUNKS = AM_PAGE * HD / 8;              // 16-byte pieces of a page (keys and values alike)
   constexpr int PER_THREAD = (CHUNKS + AM_WAVES * BLM_WAVE - 1) / (AM_WAVES * BLM_WAVE);
-  __shared__ __align__(16) bf16 k_lds[AM_PAGE * KSTR];
-  __shared__ __align__(16) bf16 v_lds[HD * VSTR];
+  // two buffers for head sizes whose pages fit twice: the next page is written while the current
+  // one is still being used, and one barrier per page is enough
+  constexpr int NBUF = HD <= 128 ? 2 : 1;
+  __shared__ __align__(16) bf16 k_lds[NBUF][AM_PAGE * KSTR];
+  __shared__ __align__(16) bf16 v_lds[NBUF][HD * VSTR];   // HD * VSTR * 2 bytes is a multiple of 16
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int c = lane & 15, kg = lane >> 4;
   const int G = nh / nkv;
@@ -247,30 +253,49 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
       }                                                                                       \
     }                                                                                         \
   }
+#define AM_STAGE(buf)                                                                                         \
+  _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                                      \
+    const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                                        \
+    if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {                                                    \
+      const int kr = j / (HD / 8), kc = j - kr * (HD / 8);           /* key row, 16-byte column */              \
+      *reinterpret_cast<u32x4_t*>(k_lds[buf] + kr * KSTR + kc * 8) = kreg[i];                                   \
+      const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8); /* value row (a dim), 16-byte column */    \
+      u32x2_t* vd = reinterpret_cast<u32x2_t*>(v_lds[buf] + vr * VSTR + vc * 8);   /* rows are 8-byte aligned */  \
+      vd[0] = u32x2_t{vreg[i].x, vreg[i].y};                                                                    \
+      vd[1] = u32x2_t{vreg[i].z, vreg[i].w};                                                                    \
+    }                                                                                                           \
+  }
+#define AM_USE(buf)                                                                                           \
+  if (pi >= my_first && pi <= my_last) {                                                                        \
+    const int key0 = pi * AM_PAGE;                                                                              \
+    /* pages wholly inside every query's range need no mask */                                                  \
+    if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)                                                    \
+      attn_page<HD, true, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, l, o);  \
+    else                                                                                                        \
+      attn_page<HD, false, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, l, o); \
+  }
   AM_FETCH(blk_first);
-  for (int pi = blk_first; pi <= blk_last; ++pi) {
-    __syncthreads();   // the page before has been used by every wavefront
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; ++i) {
-      const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;
-      if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {
-        const int kr = j / (HD / 8), kc = j - kr * (HD / 8);          // key row, 16-byte column
-        *reinterpret_cast<u32x4_t*>(k_lds + kr * KSTR + kc * 8) = kreg[i];
-        const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8);  // value row (a dim), 16-byte column
-        *reinterpret_cast<u32x4_t*>(v_lds + vr * VSTR + vc * 8) = vreg[i];
-      }
-    }
+  if (NBUF == 2) {
+    AM_STAGE(0)
     __syncthreads();
-    if (pi < blk_last) AM_FETCH(pi + 1);   // travels while this page is used
-    if (pi >= my_first && pi <= my_last) {
-      const int key0 = pi * AM_PAGE;
-      // pages wholly inside every query's range need no mask
-      if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)
-        attn_page<HD, true, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
-      else
-        attn_page<HD, false, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, qpos, lo, qpos_last, scale2, m, l, o);
+    for (int pi = blk_first; pi <= blk_last; ++pi) {
+      const int cur = (pi - blk_first) & 1;
+      if (pi < blk_last) AM_FETCH(pi + 1);   // travels while this page is used
+      AM_USE(cur)
+      if (pi < blk_last) { AM_STAGE(cur ^ 1) }   // the other buffer: nobody reads it now
+      __syncthreads();   // the next page is in place, and everybody is done with this one
+    }
+  } else {
+    for (int pi = blk_first; pi <= blk_last; ++pi) {
+      __syncthreads();   // the page before has been used by every wavefront
+      AM_STAGE(0)
+      __syncthreads();
+      if (pi < blk_last) AM_FETCH(pi + 1);   // travels while this page is used
+      AM_USE(0)
     }
   }
+#undef AM_STAGE
+#undef AM_USE
 #undef AM_FETCH
   if (!active) return;
   l += __shfl_xor(l, 16, BLM_WAVE);
