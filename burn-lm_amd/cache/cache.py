@@ -20,7 +20,6 @@ turns the core's failure codes into exceptions.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence
 
 import torch

@@ -11,11 +11,11 @@ reference's loop (crates/burn-lm-llama/src/generation/generate.rs:66-85) is one 
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence, Tuple
+from typing import Optional, Sequence, Tuple
 
 import torch
 
-from ..cache.cache import Cache, CacheError
+from ..cache.cache import Cache
 
 
 class StepError(ValueError):

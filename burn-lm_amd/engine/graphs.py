@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import gc
 import weakref
-from typing import Dict, List, Tuple
+from typing import Dict, Tuple
 
 import torch
 

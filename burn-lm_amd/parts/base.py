@@ -27,7 +27,7 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Optional, Tuple
+from typing import Dict, Tuple
 
 import torch
 

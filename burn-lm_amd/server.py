@@ -16,7 +16,7 @@ import time
 from dataclasses import asdict, dataclass, fields
 from typing import Callable, List, Optional, Sequence
 
-from .engine.generate import ContextLengthExceeded, Generation, generate
+from .engine.generate import ContextLengthExceeded, generate
 from .engine.stats import Stats
 from .sampling.sampler import Sampler
 

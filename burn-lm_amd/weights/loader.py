@@ -10,7 +10,7 @@ server/llama3.rs:526-543.)"""
 from __future__ import annotations
 
 import re
-from typing import Dict, Iterable, Sequence
+from typing import Dict, Sequence
 
 import torch
 

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import plain_llama as P
-from helpers import TINIES, TINY_A, TINY_B, TOL, make_folder, random_tokens, rel_err
+from helpers import TINIES, TINY_A, TOL, make_folder, random_tokens, rel_err
 
 pytestmark = pytest.mark.gpu
 

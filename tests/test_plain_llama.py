@@ -5,7 +5,6 @@ wrong place, scale before the product) fails it."""
 import math
 
 import numpy as np
-import pytest
 import torch
 
 import plain_llama as P

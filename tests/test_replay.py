@@ -2,7 +2,6 @@
 each request whole; with its last 32 tokens one by one; and in batches of unequal lengths whose
 shorter requests end earlier, one batch after another on a cache so small that pages and slots
 are used again.  In 32-bit and in bfloat16, on two tiny configurations."""
-import numpy as np
 import pytest
 
 import plain_llama as P

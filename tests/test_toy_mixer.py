@@ -5,7 +5,6 @@ layer 1 a running decayed sum ``s_t = a * s_{t-1} + x_t W`` kept as fixed-size s
 and the order runs layer 0 twice, the second time reading the first run's keys and values."""
 import json
 import math
-import os
 from dataclasses import dataclass
 
 import numpy as np

@@ -3,11 +3,9 @@ wrong with a checkpoint (no GPU)."""
 import json
 import os
 
-import numpy as np
 import pytest
 import torch
 
-import burn_lm_amd
 from burn_lm_amd import registry
 from burn_lm_amd.engine.model import Model
 from burn_lm_amd.weights import loader, safetensors_io as st
