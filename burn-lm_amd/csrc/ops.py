@@ -366,7 +366,8 @@ def pack_weight(w, gated=False):
 
 
 def gemv_mfma(a, packed, out, K, gated=False):
-    """bfloat16 product for M <= 16 rows on the matrix cores; streams the packed weights once.
+    """bfloat16 product for M <= 64 rows on the matrix cores; streams the packed weights once (17 to 64
+    rows: K at most 2048 per group, see gemv_mfma_group_limit).
     packed: pack_weight(w) of w [N, K].  out: bfloat16 or float32 [M, N], or float32
     [groups, M, N]: K is then cut into that many groups whose partial products fill the planes of
     out (the reader sums them).  gated=True: packed = pack_weight(w, gated=True) of a [2I, K] matrix
