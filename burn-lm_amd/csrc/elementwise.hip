@@ -246,6 +246,90 @@ __global__ void rope_kv_write_kernel(TA* __restrict__ qkv, const int* __restrict
   }
 }
 
+// bf16, head_dim a multiple of 16.  Blocks 0 .. T-1 rotate one token each, eight lanes per thread
+// with 16-byte accesses (pairing 1: lanes i..i+7 with i+half..i+half+7; pairing 0: eight neighbouring
+// lanes = four pairs).  The blocks after them copy the values: a block takes 16 consecutive tokens of
+// one key-value head, reads their rows coalesced into shared memory and writes them transposed, 16
+// lanes to the 16 tokens of one head lane, which are neighbours in the page when the tokens are
+// neighbours in a sequence (the usual case in a prompt), so that a row of the page is written in
+// pieces of 32 bytes and not of 2.
+__global__ void __launch_bounds__(256)
+    rope_kv_write_vec_kernel(bf16* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ token_seq,
+                             const int* __restrict__ block_table, int table_width, const float2* __restrict__ cos_sin,
+                             bf16* __restrict__ kcache, bf16* __restrict__ vcache, int page_size, int T, int nh,
+                             int nkv, int hd, int pairing, int write_kv) {
+  if ((int)blockIdx.x >= T) {   // a tile of values: 16 tokens of one key-value head
+    extern __shared__ bf16 vt[];   // [16][hd + 2]
+    const int tile = blockIdx.x - T;
+    const int head = tile % nkv, t0 = (tile / nkv) * 16;
+    const int vstr = hd + 2;
+    const size_t row_len = (size_t)(nh + 2 * nkv) * hd;
+    for (int e = threadIdx.x; e < 16 * hd / 2; e += blockDim.x) {   // two lanes (4 bytes) per access
+      const int j = e / (hd / 2), d2 = e - j * (hd / 2);
+      if (t0 + j < T)
+        *reinterpret_cast<uint32_t*>(vt + j * vstr + 2 * d2) =
+            *reinterpret_cast<const uint32_t*>(qkv + (size_t)(t0 + j) * row_len + (size_t)(nh + nkv + head) * hd + 2 * d2);
+    }
+    __syncthreads();
+    const int j = threadIdx.x & 15;
+    if (t0 + j >= T) return;
+    const int bj = token_seq[t0 + j];
+    if (bj < 0) return;
+    const int pj = positions[t0 + j];
+    const int pg = block_table[(size_t)bj * table_width + pj / page_size];
+    if (pg < 0) return;
+    bf16* dst = vcache + ((size_t)pg * nkv + head) * hd * page_size + pj % page_size;
+    for (int d = threadIdx.x >> 4; d < hd; d += blockDim.x >> 4) dst[(size_t)d * page_size] = vt[j * vstr + d];
+    return;
+  }
+  const int t = blockIdx.x;
+  const int b = token_seq[t];
+  if (b < 0) return;  // padding token
+  const int pos = positions[t];
+  const int half = hd >> 1;
+  bf16* row = qkv + (size_t)t * (size_t)(nh + 2 * nkv) * hd;
+  const float2* cs = cos_sin + (size_t)pos * half;
+  const int page = block_table[(size_t)b * table_width + pos / page_size];
+  const int slot = pos % page_size;
+  const bool store = write_kv && page >= 0;
+  const int per_head = pairing == 1 ? half / 8 : hd / 8;   // threads per head
+  const int n_units = (nh + nkv) * per_head;
+  for (int w = threadIdx.x; w < n_units; w += blockDim.x) {
+    const int head = w / per_head, u = w - head * per_head;
+    if (head >= nh && !store) continue;
+    bf16* x = row + (size_t)head * hd;
+    bf16* dst = head < nh ? x : kcache + (((size_t)page * nkv + (head - nh)) * page_size + slot) * hd;
+    if (pairing == 1) {
+      const int i = u * 8;
+      const uint4 a = *reinterpret_cast<const uint4*>(x + i), c = *reinterpret_cast<const uint4*>(x + i + half);
+      const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, cw[4] = {c.x, c.y, c.z, c.w};
+      uint32_t o0[4], o1[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float4 f = *reinterpret_cast<const float4*>(cs + i + 2 * k);   // (cos, sin) of two pairs
+        const float x0a = __uint_as_float(aw[k] << 16), x0b = __uint_as_float(aw[k] & 0xffff0000u);
+        const float x1a = __uint_as_float(cw[k] << 16), x1b = __uint_as_float(cw[k] & 0xffff0000u);
+        o0[k] = f32x2_to_bf16x2_bits(x0a * f.x - x1a * f.y, x0b * f.z - x1b * f.w);
+        o1[k] = f32x2_to_bf16x2_bits(x0a * f.y + x1a * f.x, x0b * f.w + x1b * f.z);
+      }
+      *reinterpret_cast<uint4*>(dst + i) = make_uint4(o0[0], o0[1], o0[2], o0[3]);
+      *reinterpret_cast<uint4*>(dst + i + half) = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+    } else {
+      const int i = u * 8;   // lanes i .. i+7 = pairs i/2 .. i/2+3
+      const uint4 a = *reinterpret_cast<const uint4*>(x + i);
+      const uint32_t aw[4] = {a.x, a.y, a.z, a.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float2 f = cs[i / 2 + k];
+        const float x0 = __uint_as_float(aw[k] << 16), x1 = __uint_as_float(aw[k] & 0xffff0000u);
+        o[k] = f32x2_to_bf16x2_bits(x0 * f.x - x1 * f.y, x0 * f.y + x1 * f.x);
+      }
+      *reinterpret_cast<uint4*>(dst + i) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
 extern "C" int blm_rope_kv_write(void* qkv, int act_dtype, const int* positions,
                                  const int* token_seq, const int* block_table, int table_width,
                                  const float* cos_sin, void* kcache, void* vcache, int page_size,
@@ -256,6 +340,16 @@ extern "C" int blm_rope_kv_write(void* qkv, int act_dtype, const int* positions,
   BLM_REQUIRE(page_size > 0 && table_width > 0, "rope_kv_write: bad cache geometry");
   BLM_REQUIRE(pairing == 0 || pairing == 1, "rope_kv_write: pairing %d unknown", pairing);
   dim3 grid(T), block(256);
+  if (act_dtype == BLM_BF16 && hd % 16 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kcache % 16) == 0 &&
+      ((uintptr_t)cos_sin % 16) == 0) {
+    const long long v_tiles = write_kv ? (long long)((T + 15) / 16) * nkv : 0;
+    BLM_REQUIRE(T + v_tiles < 2147483647LL, "rope_kv_write: too many tokens");
+    hipLaunchKernelGGL(rope_kv_write_vec_kernel, dim3((unsigned)(T + v_tiles)), block, (size_t)16 * (hd + 2) * sizeof(bf16),
+                       stream, (bf16*)qkv, positions, token_seq, block_table, table_width, (const float2*)cos_sin,
+                       (bf16*)kcache, (bf16*)vcache, page_size, T, nh, nkv, hd, pairing, write_kv);
+    BLM_LAUNCH_CHECK("rope_kv_write_vec");
+    return 0;
+  }
   if (act_dtype == BLM_F32)
     hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)qkv, positions, token_seq,
                        block_table, table_width, (const float2*)cos_sin, (float*)kcache, (float*)vcache,
