@@ -452,3 +452,68 @@ def test_a_prompt_fed_in_uneven_chunks_beside_a_decoding_neighbour(folders, dtyp
         at += n
         k += 1
     assert at == 300
+
+
+@pytest.mark.parametrize("name,dtype,seed", [("A", "float32", 0), ("B", "float32", 1), ("A", "bfloat16", 2), ("B", "bfloat16", 3)])
+def test_random_schedules_of_steps(folders, name, dtype, seed):
+    """Sequences are opened, fed in random chunks (whole prompts, pieces, single tokens, several
+    sequences per step in random order), and closed at random, on a cache small enough that slots and
+    pages are used again and steps are sometimes refused; every logit asked for is compared with the
+    plain implementation's for that sequence and position."""
+    from burn_lm_amd.cache.cache import CacheFull
+    cfg, _ = TINIES[name]
+    plain = P.load_model_folder(folders[name])
+    rng = np.random.default_rng(100 + seed)
+    max_ctx = min(cfg["max_position_embeddings"], 256)
+    eng = load(folders[name], dtype, max_tokens=768, max_seqs=5, max_context=max_ctx)
+    live = {}        # slot -> [tokens of the sequence, fed so far, plain logits]
+    checked = refused = 0
+    for it in range(60):
+        if len(live) < 5 and (not live or rng.random() < 0.5):
+            try:
+                s = eng.open()
+            except CacheFull:
+                s = None
+            if s is not None:
+                toks = random_tokens(int(rng.integers(1 << 30)), cfg["vocab_size"], int(rng.integers(1, 200)))
+                live[s] = [toks, 0, P.transformer_forward([toks], plain)[0]]
+        picks = [s for s in live if rng.random() < 0.7]
+        rng.shuffle(picks)
+        entries, expect = [], []
+        for s in picks:
+            toks, fed, want = live[s]
+            left = len(toks) - fed
+            if left == 0:
+                continue
+            n = int(min(left, rng.choice([1, 1, 2, 17, 64, 65, 200])))
+            rows = sorted(set(int(r) for r in rng.integers(0, n, size=int(rng.integers(0, 4)))))
+            entries.append((s, toks[fed:fed + n], rows))
+            expect += [want[fed + r] for r in rows]
+        if entries:
+            try:
+                got = eng.step(entries)
+            except CacheFull:
+                refused += 1
+                got = None
+                victim = max(live, key=lambda s: live[s][1])     # make room: the longest sequence goes
+                eng.close(victim)
+                del live[victim]
+                entries = []
+            for s, t, _ in entries:
+                live[s][1] += len(t)
+            if got is not None:
+                got = got.double().cpu().numpy()
+                assert got.shape[0] == len(expect)
+                for g_row, w_row in zip(got, expect):
+                    assert rel_err(g_row, w_row) <= TOL[dtype], f"iteration {it}"
+                    checked += 1
+            elif entries:
+                assert not expect
+        for s in list(live):
+            if live[s][1] == len(live[s][0]) or rng.random() < 0.05:
+                eng.close(s)
+                del live[s]
+    assert checked > 60, f"only {checked} logits were compared"
+    for s in list(live):
+        eng.close(s)
+    assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 5
