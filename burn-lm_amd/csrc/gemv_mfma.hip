@@ -57,7 +57,12 @@ __global__ void __launch_bounds__(MAXT)
     }
   }
 
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+  // a block takes a run of neighbouring column tiles, so that it streams one contiguous piece of the
+  // packed weights (blocks that each read their own region reach a higher memory rate than blocks
+  // that all advance through the matrix side by side)
+  const int tiles_per_block = (n_tiles + gridDim.x - 1) / gridDim.x;
+  const int tile_begin = blockIdx.x * tiles_per_block, tile_end = min(n_tiles, tile_begin + tiles_per_block);
+  for (int tile = tile_begin; tile < tile_end; ++tile) {
     const bf16* wt = Wp + ((size_t)tile * k_steps * 64 + lane) * 8;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     constexpr int CH = KSTEPS < 16 ? KSTEPS : 16;   // weight loads in flight per wavefront
@@ -150,9 +155,12 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) woff[s] = (step0 + s < k_steps ? step0 + s : k_steps - 1) * 512;
 
+  // a block takes a run of neighbouring column tiles: one contiguous piece of the packed weights
+  const int tiles_per_block = (n_tiles + gridDim.x - 1) / gridDim.x;
+  const int tile_begin = blockIdx.x * tiles_per_block, tile_end = min(n_tiles, tile_begin + tiles_per_block);
   uint4 w[KSTEPS], wn[KSTEPS];
   {
-    const bf16* wt = wbase + (size_t)blockIdx.x * k_steps * 512;   // gridDim.x <= n_tiles
+    const bf16* wt = wbase + (size_t)min(tile_begin, n_tiles - 1) * k_steps * 512;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) w[s] = ld16(wt + woff[s]);
   }
@@ -169,9 +177,9 @@ __global__ void __launch_bounds__(512)
     }
   }
 
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+  for (int tile = tile_begin; tile < tile_end; ++tile) {
     {
-      const int next = tile + (int)gridDim.x < n_tiles ? tile + (int)gridDim.x : tile;   // the last round re-reads its own
+      const int next = tile + 1 < tile_end ? tile + 1 : tile;   // the last round re-reads its own
       const bf16* wt = wbase + (size_t)next * k_steps * 512;
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) wn[s] = ld16(wt + woff[s]);
