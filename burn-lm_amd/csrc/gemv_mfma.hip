@@ -126,18 +126,18 @@ __global__ void __launch_bounds__(MAXT)
   }
 }
 
-// 17..64 rows: MT row tiles of 16.  A wavefront keeps the activations of all MT tiles for its 8
-// k-steps in registers (MT * 8 fragments) and runs MT MFMAs per weight fragment, so the weights
-// still stream once.  Blocks have up to 8 wavefronts, so one K-group spans at most 2048.  The
-// weights of the block's next column tile are requested before the current tile is multiplied and
-// reduced (and the first tile's before the activations), so the memory pipeline never idles while
-// the block synchronises.
-#define ROWS_KSTEPS 8
-template <int MT, typename TC>
+// 17..64 rows: MT row tiles of 16.  A wavefront keeps the activations of all MT tiles for its
+// KSTEPS k-steps in registers (MT * KSTEPS fragments, at most 32) and runs MT MFMAs per weight
+// fragment, so the weights still stream once.  Blocks have up to 8 wavefronts, so one K-group
+// spans at most 8 * KSTEPS * 32: 2048 with 8 k-steps, and 4096 with 16, which only two row tiles
+// leave room for.  PREFETCH: the weights of the block's next column tile are requested before the
+// current tile is multiplied and reduced (and the first tile's before the activations), so the
+// memory pipeline never idles while the block synchronises; with 16 k-steps the registers do not
+// allow it.
+template <int MT, int KSTEPS, bool PREFETCH, typename TC>
 __global__ void __launch_bounds__(512)
     gemv_mfma_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wp, TC* __restrict__ C, int M, int N,
                           int K, int lda, int ldc, int n_tiles, int k_steps, int c_mode, int steps_per_group) {
-  constexpr int KSTEPS = ROWS_KSTEPS;
   extern __shared__ float red[];  // [waves][MT][256]
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int n_waves = blockDim.x / BLM_WAVE;
@@ -158,8 +158,8 @@ __global__ void __launch_bounds__(512)
   // a block takes a run of neighbouring column tiles: one contiguous piece of the packed weights
   const int tiles_per_block = (n_tiles + gridDim.x - 1) / gridDim.x;
   const int tile_begin = blockIdx.x * tiles_per_block, tile_end = min(n_tiles, tile_begin + tiles_per_block);
-  uint4 w[KSTEPS], wn[KSTEPS];
-  {
+  uint4 w[KSTEPS], wn[PREFETCH ? KSTEPS : 1];
+  if (PREFETCH) {
     const bf16* wt = wbase + (size_t)min(tile_begin, n_tiles - 1) * k_steps * 512;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) w[s] = ld16(wt + woff[s]);
@@ -178,13 +178,17 @@ __global__ void __launch_bounds__(512)
   }
 
   for (int tile = tile_begin; tile < tile_end; ++tile) {
-    {
-      const int next = tile + 1 < tile_end ? tile + 1 : tile;   // the last round re-reads its own
+    if (PREFETCH) {
+      const int next = tile + 1 < tile_end ? tile + 1 : tile;   // the last round re-reads its own (from the cache)
       const bf16* wt = wbase + (size_t)next * k_steps * 512;
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) wn[s] = ld16(wt + woff[s]);
+    } else {
+      const bf16* wt = wbase + (size_t)tile * k_steps * 512;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) w[s] = ld16(wt + woff[s]);
     }
-    __builtin_amdgcn_sched_barrier(0);   // the next tile's loads are issued before this tile's first MFMA
+    __builtin_amdgcn_sched_barrier(0);   // every load is issued before this tile's first MFMA
     f32x4_t acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -219,8 +223,10 @@ __global__ void __launch_bounds__(512)
       }
     }
     __syncthreads();
+    if (PREFETCH) {
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) w[s] = wn[s];
+      for (int s = 0; s < KSTEPS; ++s) w[s] = wn[s];
+    }
   }
 }
 
@@ -238,7 +244,7 @@ static int plan_k(int K, int* ksteps) {
 // The largest K that one K-group may span for M rows (more rows leave fewer registers per k-step).
 extern "C" int blm_gemv_mfma_group_limit(int M) {
   if (M < 1 || M > 64) return 0;
-  return M <= 16 ? 16384 : 2048;
+  return M <= 16 ? 16384 : (M <= 32 ? 4096 : 2048);
 }
 
 // Whether the product runs with all of K in one group.
@@ -254,18 +260,20 @@ static int launch_mfma(const void* A, const void* Wp, void* C, int M, int N, int
   const int steps_per_group = (k_steps + k_groups - 1) / k_groups;
   if (M > 16) {
     const int mt = (M + 15) / 16;
-    const int waves = (steps_per_group + ROWS_KSTEPS - 1) / ROWS_KSTEPS;   // at most 8 by the group limit
+    const int ks = steps_per_group > 64 ? 16 : 8;   // more than 2048 of K per group: two row tiles at most
+    const int waves = (steps_per_group + ks - 1) / ks;   // at most 8 by the group limit
     int blocks = n_tiles;
     const int cap = 256 / k_groups;
     if (blocks > cap) blocks = cap > 0 ? cap : 1;
     dim3 grid(blocks, k_groups), block(waves * BLM_WAVE);
     const size_t smem = (size_t)waves * mt * 256 * sizeof(float);
-#define BLM_GR(MT)                                                                                              \
-  hipLaunchKernelGGL((gemv_mfma_rows_kernel<MT, TC>), grid, block, smem, stream, (const bf16*)A,                \
+#define BLM_GR(MT, KS, PF)                                                                                      \
+  hipLaunchKernelGGL((gemv_mfma_rows_kernel<MT, KS, PF, TC>), grid, block, smem, stream, (const bf16*)A,        \
                      (const bf16*)Wp, (TC*)C, M, N, K, lda, ldc, n_tiles, k_steps, c_mode, steps_per_group)
-    if (mt == 2) BLM_GR(2);
-    else if (mt == 3) BLM_GR(3);
-    else BLM_GR(4);
+    if (ks == 16) BLM_GR(2, 16, false);
+    else if (mt == 2) BLM_GR(2, 8, true);
+    else if (mt == 3) BLM_GR(3, 8, true);
+    else BLM_GR(4, 8, true);
 #undef BLM_GR
     BLM_LAUNCH_CHECK("gemv_mfma_rows");
     return 0;

@@ -392,7 +392,7 @@ def test_pack_weight_layout(ops):
 @pytest.mark.parametrize("M,N,K", [(1, 1001, 264), (8, 48, 64), (7, 130, 144), (16, 16, 512), (11, 333, 520),
                                    (8, 257, 2048), (3, 40, 8192), (16, 100, 8200), (5, 31, 14336), (9, 77, 4104),
                                    (2, 9000, 264), (8, 8200, 1024), (6, 100, 4096), (4, 52, 600),
-                                   (17, 130, 264), (32, 48, 2048), (29, 5000, 2040), (33, 77, 2048), (48, 257, 520),
+                                   (17, 130, 264), (32, 48, 2048), (29, 5000, 2040), (33, 77, 2048), (32, 200, 4096), (20, 1000, 3072), (48, 257, 520),
                                    (47, 16, 64), (49, 300, 1032), (64, 4200, 2048), (61, 40, 136)])
 def test_gemv_mfma(ops, out_dtype, M, N, K):
     """Matrix-core skinny product: every way K is cut among wavefronts, tails in N, K and M; above 16
@@ -452,7 +452,7 @@ def test_gemv_mfma_partial_products_are_summed_by_the_norm(ops, M, N, K, groups)
 
 
 @pytest.mark.parametrize("M,I,K", [(8, 176, 64), (3, 384, 144), (16, 8, 520), (5, 1000, 2048), (1, 64, 4104),
-                                   (64, 1000, 2048), (20, 176, 1544), (37, 384, 144), (50, 8, 520)])
+                                   (64, 1000, 2048), (20, 176, 1544), (37, 384, 144), (50, 8, 520), (32, 176, 4096)])
 def test_gemv_mfma_gated(ops, M, I, K):
     """The SwiGLU gating in the epilogue of the product that computes gate and up: the packed copy pairs
     every 8 gate rows with their 8 up rows, the result is silu(x gate^T) * (x up^T)."""
@@ -474,9 +474,9 @@ def test_gemv_mfma_refuses_what_it_cannot_do(ops):
     assert not ops.gemv_mfma_supported(65, 64, 64) and not ops.gemv_mfma_supported(4, 64, 60)
     assert not ops.gemv_mfma_supported(4, 64, 16392)
     # more rows leave fewer registers for each k-step: the K of one group shrinks
-    assert ops.gemv_mfma_supported(16, 64, 4096) and not ops.gemv_mfma_supported(17, 64, 4096)
-    assert ops.gemv_mfma_supported(64, 64, 2048) and not ops.gemv_mfma_supported(17, 64, 2056)
-    assert [ops.gemv_mfma_group_limit(m) for m in (0, 1, 16, 17, 64, 65)] == [0, 16384, 16384, 2048, 2048, 0]
+    assert ops.gemv_mfma_supported(32, 64, 4096) and not ops.gemv_mfma_supported(33, 64, 4096)
+    assert ops.gemv_mfma_supported(64, 64, 2048) and not ops.gemv_mfma_supported(17, 64, 4104)
+    assert [ops.gemv_mfma_group_limit(m) for m in (0, 1, 16, 17, 32, 33, 64, 65)] == [0, 16384, 16384, 4096, 4096, 2048, 2048, 0]
     wp = ops.pack_weight(dev(torch.zeros(8, 64).bfloat16()))
     with pytest.raises(KernelError, match="1..64"):
         ops.gemv_mfma(dev(torch.zeros(65, 64).bfloat16()), wp, torch.zeros(65, 8, dtype=torch.bfloat16, device="cuda"), 64)
