@@ -7,6 +7,12 @@
 //
 // Visibility: the query at position p of its sequence sees keys j of the same sequence with
 // j <= p and, if window > 0, p - j < window.
+//
+// With n_splits > 1 (few query tokens over long key ranges: decode) the key range of every
+// (token, head) is cut into that many pieces handled by different wavefronts (blockIdx.y).  Each
+// writes its partial maximum, sum and output with stores that reach device-coherent memory, waits
+// for them to complete and counts itself in; the wavefront that finds all the others counted reads
+// their partial results back and writes the output.  Nobody waits for anybody.
 #include "common.h"
 
 template <typename T>
@@ -39,7 +45,8 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
                       const int* __restrict__ positions, const int* __restrict__ token_seq,
                       const int* __restrict__ block_table, int table_width,
                       const TA* __restrict__ kcache, const TA* __restrict__ vcache, int page_size,
-                      int T, int nh, int nkv, int hd, float scale, int window) {
+                      int T, int nh, int nkv, int hd, float scale, int window, int n_splits, float* part_o,
+                      float* part_ml, int* arrivals) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const long long w = (long long)blockIdx.x * ATTN_WAVES + wave;
@@ -63,13 +70,19 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
   const int kvh = head / (nh / nkv);
   const int* bt = block_table + (size_t)b * table_width;
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  // this wavefront's piece of the key range, in chunks of one wavefront's width
+  const int split = blockIdx.y;
+  const int n_chunks = (pos - first) / BLM_WAVE + 1;
+  const int per_split = (n_chunks + n_splits - 1) / n_splits;
+  const int j_begin = first + split * per_split * BLM_WAVE;
+  const int j_end = min(pos, j_begin + per_split * BLM_WAVE - 1);   // last key of the piece
 
   float m = -INFINITY, l = 0.f;
   float acc[ATTN_MAX_HD / BLM_WAVE] = {0.f, 0.f, 0.f, 0.f};
 
-  for (int j0 = first; j0 <= pos; j0 += BLM_WAVE) {
+  for (int j0 = j_begin; j0 <= j_end; j0 += BLM_WAVE) {
     const int j = j0 + lane;
-    const bool valid = j <= pos;
+    const bool valid = j <= j_end;
     float s = -INFINITY;
     if (valid) {
       const int page = bt[j / page_size];
@@ -93,7 +106,7 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
     l = l * corr + wave_sum(p);
 #pragma unroll
     for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) acc[i] *= corr;
-    const int cnt = (pos - j0 + 1) < BLM_WAVE ? (pos - j0 + 1) : BLM_WAVE;
+    const int cnt = (j_end - j0 + 1) < BLM_WAVE ? (j_end - j0 + 1) : BLM_WAVE;
     for (int jj = 0; jj < cnt; ++jj) {
       const float pj = __shfl(p, jj, BLM_WAVE);
       const int ja = j0 + jj;
@@ -107,34 +120,88 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
     }
     m = m_new;
   }
-  const float inv = 1.0f / l;
+  if (n_splits == 1) {
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) {
+      const int d = lane + i * BLM_WAVE;
+      if (d < hd) orow[d] = from_float<TA>(acc[i] * inv);
+    }
+    return;
+  }
+  // publish this piece (an empty piece has m = -inf, l = 0 and counts for nothing)
+  const size_t item = (size_t)t * nh + head;
+  float* po = part_o + (item * n_splits + split) * hd;
 #pragma unroll
   for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) {
     const int d = lane + i * BLM_WAVE;
-    if (d < hd) orow[d] = from_float<TA>(acc[i] * inv);
+    if (d < hd) __hip_atomic_store(po + d, acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (lane == 0) {
+    __hip_atomic_store(part_ml + (item * n_splits + split) * 2, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(part_ml + (item * n_splits + split) * 2 + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the wavefront's stores have been acknowledged
+  int last = 0;
+  if (lane == 0) {
+    const int before = __hip_atomic_fetch_add(arrivals + item, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = before == n_splits - 1;
+    if (last) __hip_atomic_store(arrivals + item, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero again for the next launch
+  }
+  last = __shfl(last, 0, BLM_WAVE);
+  if (!last) return;
+  float M = -INFINITY, L = 0.f;
+  float O[ATTN_MAX_HD / BLM_WAVE] = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < n_splits; ++sp) {
+    const float* ml = part_ml + (item * n_splits + sp) * 2;
+    const float ms = __hip_atomic_load(ml, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float ls = __hip_atomic_load(ml + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (ls == 0.f) continue;
+    const float Mn = fmaxf(M, ms);
+    const float keep = expf(M - Mn), take = expf(ms - Mn);   // exp(-inf) = 0 on the first piece
+    L = L * keep + ls * take;
+    const float* ps = part_o + (item * n_splits + sp) * hd;
+#pragma unroll
+    for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) {
+      const int d = lane + i * BLM_WAVE;
+      if (d < hd) O[i] = O[i] * keep + __hip_atomic_load(ps + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * take;
+    }
+    M = Mn;
+  }
+  const float inv = 1.0f / L;
+#pragma unroll
+  for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) {
+    const int d = lane + i * BLM_WAVE;
+    if (d < hd) orow[d] = from_float<TA>(O[i] * inv);
   }
 }
 
+// part_o: T*nh*n_splits*hd floats, part_ml: T*nh*n_splits*2 floats, arrivals: T*nh ints that are
+// zero before the first call (every call leaves them zero again); all three may be null when
+// n_splits is 1.  Calls that share the arrivals buffer must not overlap in time.
 extern "C" int blm_attn_paged(const void* q, int q_row_stride, void* out, int act_dtype,
                               const int* positions, const int* token_seq, const int* block_table,
                               int table_width, const void* kcache, const void* vcache,
                               int page_size, int T, int nh, int nkv, int hd, float scale,
-                              int window, hipStream_t stream) {
+                              int window, int n_splits, float* part_o, float* part_ml, int* arrivals,
+                              hipStream_t stream) {
   BLM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && nh % nkv == 0,
               "attn_paged: bad sizes T=%d heads=%d kv_heads=%d (heads must be a multiple of kv_heads)", T, nh, nkv);
   BLM_REQUIRE(hd > 0 && hd % 2 == 0 && hd <= ATTN_MAX_HD,
               "attn_paged: head_dim %d not supported (even, at most %d)", hd, ATTN_MAX_HD);
   BLM_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attn_paged: bad cache geometry");
+  BLM_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml && arrivals)),
+              "attn_paged: %d splits need their workspace", n_splits);
   const long long items = (long long)T * nh;
   const long long blocks = (items + ATTN_WAVES - 1) / ATTN_WAVES;
   BLM_REQUIRE(blocks < 2147483647LL, "attn_paged: too many (token, head) pairs: %lld", items);
-  dim3 grid((unsigned)blocks), block(ATTN_WAVES * BLM_WAVE);
+  dim3 grid((unsigned)blocks, (unsigned)n_splits), block(ATTN_WAVES * BLM_WAVE);
   const size_t smem = (size_t)ATTN_WAVES * hd * sizeof(float);
   const bool vec = (hd % 8) == 0 && (q_row_stride % 8) == 0;
 #define BLM_ATTN_CASE(TA, V)                                                                        \
   hipLaunchKernelGGL((attn_paged_kernel<TA, V>), grid, block, smem, stream, (const TA*)q, q_row_stride, \
                      (TA*)out, positions, token_seq, block_table, table_width, (const TA*)kcache,    \
-                     (const TA*)vcache, page_size, T, nh, nkv, hd, scale, window)
+                     (const TA*)vcache, page_size, T, nh, nkv, hd, scale, window, n_splits, part_o, part_ml, arrivals)
   if (act_dtype == BLM_F32) {
     if (vec) BLM_ATTN_CASE(float, true); else BLM_ATTN_CASE(float, false);
   } else if (act_dtype == BLM_BF16) {

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 _lib = None
 _lock = threading.Lock()
 
@@ -30,7 +30,7 @@ _SIGNATURES = {
     "blm_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "blm_attn_paged": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                       _c_void_p],
+                       _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     "blm_attn_decode": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                         _c_void_p, _c_void_p, _c_void_p, _c_void_p],
@@ -117,6 +117,9 @@ def _stream():
 
 def _call(name, *args):
     lib = library()
+    if len(args) != len(_SIGNATURES[name]):
+        # ctypes would pass the surplus as 32-bit integers and cut pointers (a stream handle) short
+        raise KernelError(f"{name}: {len(args)} arguments given, its signature has {len(_SIGNATURES[name])}")
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelError(lib.blm_last_error().decode())
@@ -229,9 +232,10 @@ def swiglu(gate_up, out):
 
 
 def attn_paged(q, q_row_stride, out, positions, token_seq, block_table, kcache, vcache, page_size,
-               nh, nkv, hd, scale, window=0):
+               nh, nkv, hd, scale, window=0, n_splits=1):
     """Attention of every query token over its sequence's cached keys (generic kernel).
-    q: first nh*hd columns of rows with stride q_row_stride; out: [T, nh*hd]."""
+    q: first nh*hd columns of rows with stride q_row_stride; out: [T, nh*hd].  n_splits > 1 cuts
+    every key range into that many pieces for different wavefronts (few tokens over long ranges)."""
     _gpu(q, out, positions, token_seq, block_table, kcache, vcache)
     T = out.shape[0]
     _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
@@ -241,9 +245,19 @@ def attn_paged(q, q_row_stride, out, positions, token_seq, block_table, kcache, 
         raise KernelError("attn_paged: q rows must be contiguous and at least heads*head_dim long")
     _check_planes("attn_paged", kcache, vcache, nkv, page_size, hd)
     _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
+    n_splits = max(1, int(n_splits))
+    part_o = part_ml = arrivals = None
+    if n_splits > 1:
+        arrivals = arrival_counters(out.device)
+        if T * nh > arrivals.numel():
+            n_splits = 1      # more (token, head) pairs than counters: enough parallel work without cutting
+        else:
+            part_o = torch.empty(T * nh * n_splits * hd, dtype=torch.float32, device=out.device)
+            part_ml = torch.empty(T * nh * n_splits * 2, dtype=torch.float32, device=out.device)
     _call("blm_attn_paged", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
-          page_size, T, nh, nkv, hd, float(scale), int(window), _stream())
+          page_size, T, nh, nkv, hd, float(scale), int(window), n_splits, _ptr(part_o), _ptr(part_ml),
+          _ptr(arrivals if n_splits > 1 else None), _stream())
     return out
 
 

@@ -69,6 +69,12 @@ class Attention(Mixer):
             rt.ops.attn_prefill_mfma(qkv, qkv.shape[1], out, step.positions, step.cu_seqlens, table, view.k, view.v,
                                      view.page_size, step.n_seqs, step.max_new, nh, nkv, hd, self.scale, self.window)
         else:
+            # the generic kernel has one wavefront per (token, head); with few tokens over long key
+            # ranges the ranges are cut so that the whole chip has work
+            n_splits = 1
+            if step.max_new == 1:
+                span = step.max_len_after if not self.window else min(step.max_len_after, self.window)
+                n_splits = max(1, min((span + 255) // 256, (4 * DECODE_TARGET_BLOCKS) // max(1, x.shape[0] * nh)))
             rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
-                              view.page_size, nh, nkv, hd, self.scale, self.window)
+                              view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
         return rt.linear(out, self.w_o, partials=True)   # the block's next norm sums partial products

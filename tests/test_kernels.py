@@ -153,10 +153,13 @@ def _attn_ref(q, keys, values, pos, scale, window, n_rep):
     return torch.einsum("hs,shd->hd", torch.softmax(s, -1), v)
 
 
+@pytest.mark.parametrize("splits", [1, 2, 5])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (6, 1, 24, 0), (5, 5, 64, 0), (8, 2, 128, 0),
                                                (3, 1, 200, 0), (4, 2, 32, 37)])
-def test_attn_paged(ops, dtype, nh, nkv, hd, window):
+def test_attn_paged(ops, dtype, nh, nkv, hd, window, splits):
+    """The generic kernel, whole key ranges and ranges cut into pieces that are merged by the last
+    wavefront to finish (more pieces than some sequences have chunks of keys: empty pieces)."""
     g = torch.Generator().manual_seed(4)
     page, n_pages = 16, 40
     lens = [150, 1, 70]          # cached length of three sequences after this step
@@ -188,9 +191,12 @@ def test_attn_paged(ops, dtype, nh, nkv, hd, window):
     qkv = torch.randn(T, stride, generator=g).to(DT[dtype])
     out = torch.full((T, nh * hd), 7.0, dtype=DT[dtype], device="cuda")
     scale = 1.0 / math.sqrt(hd)
-    ops.attn_paged(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
-                   dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc.to(DT[dtype])),
-                   dev(vc.to(DT[dtype])), page, nh, nkv, hd, scale, window)
+    for rep in range(3 if splits > 1 else 1):     # again and again: the counters must come back to zero
+        out.fill_(7.0)
+        ops.attn_paged(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
+                       dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc.to(DT[dtype])),
+                       dev(vc.to(DT[dtype])), page, nh, nkv, hd, scale, window, splits)
+    assert int(ops.arrival_counters("cuda").abs().sum()) == 0
     got = out.cpu().double().reshape(T, nh, hd)
     assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
     for t in range(T - 1):
