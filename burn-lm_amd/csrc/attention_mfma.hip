@@ -459,7 +459,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
-static bool hd_ok(int hd, int max_hd) { return hd >= 16 && hd <= max_hd && (hd & (hd - 1)) == 0; }
+static bool hd_ok(int hd, int max_hd) { return hd >= 16 && hd % 16 == 0 && (hd <= 128 || hd == 256) && hd <= max_hd; }
 
 extern "C" int blm_attn_prefill_mfma_supported(int act_dtype, int hd, int page_size) {
   return (act_dtype == BLM_BF16 && page_size == AM_PAGE && hd_ok(hd, 256)) ? 1 : 0;
@@ -476,7 +476,7 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
   BLM_REQUIRE(n_seqs > 0 && n_seqs <= 65535 && max_new > 0 && nh > 0 && nkv > 0 && nkv <= 65535 && nh % nkv == 0,
               "attn_prefill_mfma: bad sizes seqs=%d max_new=%d heads=%d kv_heads=%d", n_seqs, max_new, nh, nkv);
   BLM_REQUIRE(blm_attn_prefill_mfma_supported(act_dtype, hd, page_size),
-              "attn_prefill_mfma: needs bfloat16, pages of 64 and a head_dim of 16, 32, 64, 128 or 256 "
+              "attn_prefill_mfma: needs bfloat16, pages of 64 and a head_dim that is a multiple of 16 up to 128, or 256 "
               "(got dtype %d, page %d, head_dim %d)", act_dtype, page_size, hd);
   BLM_REQUIRE(table_width > 0 && window >= 0, "attn_prefill_mfma: bad geometry");
   BLM_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive (got %g)", (double)scale);
@@ -491,7 +491,9 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
                        (bf16*)out, positions, cu_seqlens, block_table, table_width, (const bf16*)kcache,          \
                        (const bf16*)vcache, nh, nkv, scale, window);                                              \
     break
-  switch (hd) { BLM_AP(16); BLM_AP(32); BLM_AP(64); BLM_AP(128); BLM_AP(256); }
+  switch (hd) {
+    BLM_AP(16); BLM_AP(32); BLM_AP(48); BLM_AP(64); BLM_AP(80); BLM_AP(96); BLM_AP(112); BLM_AP(128); BLM_AP(256);
+  }
 #undef BLM_AP
   BLM_LAUNCH_CHECK("attn_prefill_mfma");
   return 0;
@@ -508,7 +510,7 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
   BLM_REQUIRE(T > 0 && T <= 65535 && nh > 0 && nkv > 0 && nh % nkv == 0,
               "attn_decode: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
   BLM_REQUIRE(blm_attn_decode_supported(act_dtype, hd, page_size),
-              "attn_decode: needs bfloat16, pages of 64 and a head_dim of 16, 32, 64 or 128 "
+              "attn_decode: needs bfloat16, pages of 64 and a head_dim that is a multiple of 16 up to 128 "
               "(got dtype %d, page %d, head_dim %d)", act_dtype, page_size, hd);
   BLM_REQUIRE(table_width > 0 && window >= 0 && n_splits >= 1 && n_splits <= 65535,
               "attn_decode: bad geometry width=%d window=%d splits=%d", table_width, window, n_splits);
@@ -524,7 +526,7 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
                        positions, token_seq, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache,    \
                        nh, nkv, scale, window, n_splits, part_o, part_ml, arrivals, (bf16*)out);                    \
     break
-  switch (hd) { BLM_AD(16); BLM_AD(32); BLM_AD(64); BLM_AD(128); }
+  switch (hd) { BLM_AD(16); BLM_AD(32); BLM_AD(48); BLM_AD(64); BLM_AD(80); BLM_AD(96); BLM_AD(112); BLM_AD(128); }
 #undef BLM_AD
   BLM_LAUNCH_CHECK("attn_decode_mfma");
   return 0;

@@ -305,8 +305,8 @@ def test_graph_replays_of_larger_batches(folders, dtype, n, bucket):
 
 
 def test_head_size_that_is_no_power_of_two_and_odd_counts(tmp_path):
-    """head_dim 48 (a step of 16 that the matrix-core attention does not take: the generic kernel
-    runs), 5 heads without grouping, an odd vocabulary: whole, tail and batch against plain."""
+    """head_dim 48 (a step of 16 that is no power of two), 5 heads without grouping, an odd
+    vocabulary: whole, tail and batch against plain."""
     cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=120, intermediate_size=200, num_hidden_layers=2,
                num_attention_heads=5, num_key_value_heads=5, head_dim=48, vocab_size=257, max_position_embeddings=256,
                rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)

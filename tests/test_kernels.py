@@ -260,13 +260,15 @@ def test_attn_decode_merge_by_the_last_split_over_many_calls(ops):
 
 
 @pytest.mark.parametrize("nh,nkv,hd,window,splits", [(4, 2, 16, 0, 3), (6, 1, 32, 0, 1), (5, 5, 64, 0, 4), (8, 2, 128, 0, 16),
-                                                      (32, 1, 64, 0, 2), (20, 1, 32, 0, 5), (4, 2, 32, 100, 2)])
+                                                      (32, 1, 64, 0, 2), (20, 1, 32, 0, 5), (4, 2, 32, 100, 2),
+                                                      (6, 2, 48, 0, 3), (3, 3, 80, 0, 2), (4, 1, 96, 70, 4), (2, 2, 112, 0, 5)])
 def test_attn_decode(ops, nh, nkv, hd, window, splits):
     """The matrix-core decode kernel: sequences of very different lengths in one call (one of a single
     key, one that ends exactly at a page edge), scrambled pages with NaN in every unused place, a far
     key that stands out, more splits than some sequences have pages, more than 16 heads to a group,
     a padding token."""
     assert ops.attn_decode_supported(torch.bfloat16, hd) and not ops.attn_decode_supported(torch.bfloat16, 24)
+    assert not ops.attn_decode_supported(torch.bfloat16, 144) and not ops.attn_decode_supported(torch.bfloat16, 256)
     assert not ops.attn_decode_supported(torch.float32, hd) and not ops.attn_decode_supported(torch.bfloat16, hd, 16)
     g = torch.Generator().manual_seed(14)
     lens = [403, 1, 64, 17, 130, 65]
@@ -295,7 +297,7 @@ def test_attn_decode(ops, nh, nkv, hd, window, splits):
 
 
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (6, 1, 32, 0), (5, 5, 64, 0), (8, 2, 128, 0), (2, 1, 256, 0),
-                                               (4, 2, 64, 90)])
+                                               (4, 2, 64, 90), (6, 2, 48, 0), (3, 3, 80, 0), (4, 1, 96, 50), (2, 2, 112, 0)])
 def test_attn_prefill_mfma(ops, nh, nkv, hd, window):
     """The matrix-core prefill kernel on packed sequences: a whole prompt from position 0 (not a
     multiple of 16 long), a chunk that continues a long past, one token on top of a past that ends at
