@@ -192,6 +192,9 @@ extern "C" int blm_cache_reserve(BlmCache* c, int n, const int* slots, const int
 extern "C" int blm_cache_advance(BlmCache* c, int slot, int n) {
   if (!is_open(*c, slot)) return fail(BLM_E_USAGE, "slot %d is not open", slot);
   if (n < 0 || c->length[slot] + n > c->max_context) return fail(BLM_E_USAGE, "slot %d cannot advance by %d", slot, n);
+  for (const Group& g : c->groups)
+    if (pages_for(*c, c->length[slot] + n) > (int)g.tables[slot].size())
+      return fail(BLM_E_USAGE, "slot %d advances by %d tokens that no page was reserved for", slot, n);
   c->length[slot] += n;
   for (Group& g : c->groups) {
     std::vector<int>& table = g.tables[slot];

@@ -224,3 +224,16 @@ def test_step_assembly_refuses_what_it_cannot_lay_out():
     with pytest.raises(CacheError, match="wider"):
         c.reserve([(a, 40)])
         c.fill_step([(a, [1], [0])], 0, 1, host.data_ptr(), 64)
+
+
+def test_advance_needs_reserved_pages():
+    c = make()
+    a = c.open()
+    with pytest.raises(CacheError, match="no page was reserved"):
+        c.advance(a, 5)
+    c.reserve([(a, 5)])
+    c.advance(a, 5)
+    with pytest.raises(CacheError, match="no page was reserved"):
+        c.advance(a, 16)          # 21 tokens need a second page of 16
+    c.advance(a, 11)              # the reserved page holds 16
+    assert c.length(a) == 16
