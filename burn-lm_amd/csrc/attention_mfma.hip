@@ -59,7 +59,7 @@ __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
 template <int HD, bool FULL, int KSTR, int VSTR, bool V_LATE>
 __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf16* __restrict__ vp,
                                           const uint4* qf, int key0, int qpos, int lo, int max_key, float scale2,
-                                          float& m, float& l, f32x4_t* o) {
+                                          float& m, f32x4_t& l, f32x4_t* o) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
   const int lane = threadIdx.x & (BLM_WAVE - 1);
@@ -109,7 +109,6 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
   const float m_new = fmaxf(m, mx * scale2);
   // m = -inf, m_new finite -> 0;  both -inf (nothing visible yet) -> 1, and every p below is 0
   const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
-  float psum = 0.f;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -118,14 +117,14 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
       if (FULL) p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
       else p = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
       s[t][r] = p;
-      psum += p;
     }
-  l = l * corr + psum;
   if (__any(m != m_new)) {   // once the running maxima have settled, most pages change none of them
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) l[r] *= corr;
   }
   m = m_new;
 
@@ -139,6 +138,10 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
     pf.y = pack_bf16x2(s[2 * h][2], s[2 * h][3]);
     pf.z = pack_bf16x2(s[2 * h + 1][0], s[2 * h + 1][1]);
     pf.w = pack_bf16x2(s[2 * h + 1][2], s[2 * h + 1][3]);
+    // the softmax's denominator as one more output row: a row of ones for V^T sums the rounded
+    // probabilities of every query column over the 32 keys, on the matrix cores instead of 16 adds
+    l = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u)),
+                                                __builtin_bit_cast(bf16x8_t, pf), l, 0, 0, 0);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       uint2 v0 = vf[dt][2 * h], v1 = vf[dt][2 * h + 1];
@@ -234,7 +237,8 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 
   uint4 qf[KS];
   load_q<HD>(q + (size_t)row * q_row_stride + (size_t)head * HD, qf);
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY;
+  f32x4_t lsum = {0.f, 0.f, 0.f, 0.f};   // the denominator of query column c, the same in all four places
   f32x4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -270,9 +274,9 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
     const int key0 = pi * AM_PAGE;                                                                              \
     /* pages wholly inside every query's range need no mask */                                                  \
     if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)                                                    \
-      attn_page<HD, true, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, l, o);  \
+      attn_page<HD, true, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o);  \
     else                                                                                                        \
-      attn_page<HD, false, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, l, o); \
+      attn_page<HD, false, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o); \
   }
   AM_FETCH(blk_first);
   if (NBUF == 2) {
@@ -298,8 +302,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 #undef AM_USE
 #undef AM_FETCH
   if (!active) return;
-  l += __shfl_xor(l, 16, BLM_WAVE);
-  l += __shfl_xor(l, 32, BLM_WAVE);
+  const float l = lsum[0];
   if (c < nq) {
     const float inv = 1.0f / l;
     bf16* orow = out + (size_t)row * nh * HD + (size_t)head * HD;
@@ -342,7 +345,8 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   const int b = token_seq[t];
   const int head = kvh * G + min(g0 + c, G - 1);   // columns past the group's end repeat its last head
 
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY;
+  f32x4_t lsum = {0.f, 0.f, 0.f, 0.f};   // the denominator of query column c, the same in all four places
   f32x4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -362,14 +366,12 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
       const int key0 = pi * AM_PAGE;
       if (key0 + AM_PAGE - 1 <= pos && key0 >= lo)
-        attn_page<HD, true, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+        attn_page<HD, true, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, lsum, o);
       else
-        attn_page<HD, false, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, l, o);
+        attn_page<HD, false, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, lsum, o);
     }
   }
-  l += __shfl_xor(l, 16, BLM_WAVE);
-  l += __shfl_xor(l, 32, BLM_WAVE);
-  if (kg == 0) { sm_m[wave][c] = m; sm_l[wave][c] = l; }
+  if (kg == 0) { sm_m[wave][c] = m; sm_l[wave][c] = lsum[0]; }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
