@@ -15,9 +15,10 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-// QR_KSTEPS: k-steps of 32 per wavefront (16 for K <= 2048, 32 up to 4096); at most 8 wavefronts.
-template <int QR_KSTEPS>
-__global__ void __launch_bounds__(512)
+// QR_KSTEPS: k-steps of 32 per wavefront.  MAXT: most threads of a block (8 or 16 wavefronts).  All
+// loads of a block are in flight at once: its time is one memory latency.
+template <int QR_KSTEPS, int MAXT>
+__global__ void __launch_bounds__(MAXT)
     gemv_qkv_rope_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wp, bf16* __restrict__ qkv_out,
                          const int* __restrict__ positions, const int* __restrict__ token_seq,
                          const int* __restrict__ block_table, int table_width, const float2* __restrict__ cos_sin,
@@ -136,16 +137,20 @@ extern "C" int blm_gemv_qkv_rope(const void* A, const void* Wp, void* qkv_out, c
   BLM_REQUIRE(lda % 8 == 0 && lda >= K && ldq >= nh * hd, "gemv_qkv_rope: bad strides lda=%d ldq=%d", lda, ldq);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0, "gemv_qkv_rope: operands must be 16-byte aligned");
   const int k_steps = (K + 31) / 32;
-  const int ksteps = K <= 2048 ? 16 : 32;
-  const int kw = (k_steps + ksteps - 1) / ksteps;   // at most 4
+  // all of a block's loads are in flight at once: 4 wavefronts per tile with 16 k-steps each up to
+  // K = 2048, with 24 up to 3072 (their registers still fit), and 8 wavefronts with 16 up to 4096
+  const int ksteps = (k_steps > 64 && k_steps <= 96) ? 24 : 16;
+  const int kw = (k_steps + ksteps - 1) / ksteps;   // at most 8
   const int units = (nh + 2 * nkv) * (hd / 32);
   const size_t smem = (size_t)2 * kw * 256 * sizeof(float);
-#define BLM_QR(KS)                                                                                                    \
-  hipLaunchKernelGGL(gemv_qkv_rope_kernel<KS>, dim3(units), dim3(2 * kw * BLM_WAVE), smem, stream, (const bf16*)A,    \
+#define BLM_QR(KS, MAXT)                                                                                              \
+  hipLaunchKernelGGL((gemv_qkv_rope_kernel<KS, MAXT>), dim3(units), dim3(2 * kw * BLM_WAVE), smem, stream, (const bf16*)A, \
                      (const bf16*)Wp, (bf16*)qkv_out, positions, token_seq, block_table, table_width,                 \
                      (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache, page_size, M, K, lda, ldq, k_steps, kw, nh, \
                      nkv, hd, pairing, store)
-  if (ksteps == 16) BLM_QR(16); else BLM_QR(32);
+  if (ksteps == 24) BLM_QR(24, 512);
+  else if (kw <= 4) BLM_QR(16, 512);
+  else BLM_QR(16, 1024);
 #undef BLM_QR
   BLM_LAUNCH_CHECK("gemv_qkv_rope");
   return 0;

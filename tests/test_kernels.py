@@ -582,7 +582,8 @@ def test_sample_large_vocabulary_matches_the_ordered_nucleus(ops, V, ld):
 
 
 @pytest.mark.parametrize("pairing", ["interleaved", "half"])
-@pytest.mark.parametrize("M,K,nh,nkv,hd", [(8, 2048, 4, 2, 64), (5, 264, 3, 1, 32), (16, 3072, 2, 2, 128), (1, 64, 6, 3, 64)])
+@pytest.mark.parametrize("M,K,nh,nkv,hd", [(8, 2048, 4, 2, 64), (5, 264, 3, 1, 32), (16, 3072, 2, 2, 128), (1, 64, 6, 3, 64),
+                                           (4, 4096, 2, 1, 64), (9, 3608, 3, 1, 32), (7, 2056, 2, 2, 32)])
 def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     """The fused decode projection: equals the product, the rotation of its float result and the
     cache write done one after the other (in float64), for both pairings, with a padding row and
