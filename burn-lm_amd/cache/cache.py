@@ -296,10 +296,11 @@ class Cache:
             _raise(code)
         return [list(out[i * width:(i + 1) * width]) for i in range(len(slots))]
 
-    def fill_step(self, entries, pad_to: int, width: int, out_ptr: int, capacity: int):
+    def fill_step(self, entries, pad_seqs: int, pad_tokens: int, width: int, out_ptr: int, capacity: int):
         """Writes the index arrays of a step for entries (slot, tokens, want) into int32 host memory
-        at out_ptr (see blm_step_fill in csrc/host/cache_core.h for the layout) and returns
-        (tokens, wanted rows, most tokens of one sequence, greatest length after the step)."""
+        at out_ptr (see blm_step_fill in csrc/host/cache_core.h for the layout and for the padding
+        to pad_seqs sequences and pad_tokens tokens; 0: none) and returns (tokens, wanted rows, most
+        tokens of one sequence, greatest length after the step)."""
         slots, counts, tokens, want_counts, wants = [], [], [], [], []
         for slot, toks, want in entries:
             slots.append(slot)
@@ -309,7 +310,8 @@ class Cache:
             wants.extend(want)
         meta = (_core.ctypes.c_int * 4)()
         code = self._lib.blm_step_fill(self._h, len(slots), _core.ints(slots), _core.ints(counts), _core.ints(tokens),
-                                       _core.ints(want_counts), _core.ints(wants), pad_to, width, out_ptr, capacity, meta)
+                                       _core.ints(want_counts), _core.ints(wants), pad_seqs, pad_tokens, width, out_ptr,
+                                       capacity, meta)
         if code:
             _raise(code)
         return tuple(meta)

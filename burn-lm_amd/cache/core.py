@@ -8,7 +8,7 @@ from typing import List, Sequence
 
 from ..csrc import build as _build
 
-HOST_ABI = 1
+HOST_ABI = 2
 OK, E_FULL, E_OVERFLOW, E_USAGE = 0, 1, 2, 3
 
 _lib = None
@@ -29,7 +29,7 @@ _SIGNATURES = {
     "blm_cache_n_free_slots": ([_ptr], _int), "blm_cache_free_slots": ([_ptr, _ints], _int),
     "blm_cache_live_slots": ([_ptr, _ints], _int),
     "blm_step_size": ([_int, _int, _int, _int, _int], _ll),
-    "blm_step_fill": ([_ptr, _int, _ints, _ints, _ints, _ints, _ints, _int, _int, _ptr, _ll, _ints], _int),
+    "blm_step_fill": ([_ptr, _int, _ints, _ints, _ints, _ints, _ints, _int, _int, _int, _ptr, _ll, _ints], _int),
 }
 
 

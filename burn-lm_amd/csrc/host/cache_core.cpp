@@ -266,23 +266,26 @@ extern "C" long long blm_step_size(int n_groups, int T, int B, int R, int width)
 }
 
 extern "C" int blm_step_fill(const BlmCache* c, int n, const int* slots, const int* counts, const int* tokens,
-                             const int* want_counts, const int* wants, int pad_to, int width, int* out, long long cap,
-                             int* meta) {
+                             const int* want_counts, const int* wants, int pad_seqs_to, int pad_tokens_to, int width,
+                             int* out, long long cap, int* meta) {
   if (n <= 0) return fail(BLM_E_USAGE, "a step needs at least one sequence");
-  const int B = std::max(n, pad_to);
-  long long T = 0, R = 0;
+  const int B = std::max(n, pad_seqs_to);
+  long long real = 0, R = 0;
   int max_new = 0, max_after = 0;
   for (int i = 0; i < n; ++i) {
     if (!is_open(*c, slots[i])) return fail(BLM_E_USAGE, "slot %d is not open", slots[i]);
     if (counts[i] <= 0 || want_counts[i] < 0) return fail(BLM_E_USAGE, "slot %d: bad token or want count", slots[i]);
-    if (B > n && (counts[i] != 1 || want_counts[i] != 1))
-      return fail(BLM_E_USAGE, "only a step of one wanted token per sequence can be padded");
-    T += counts[i];
+    real += counts[i];
     R += want_counts[i];
     max_new = std::max(max_new, counts[i]);
     max_after = std::max(max_after, c->length[slots[i]] + counts[i]);
   }
-  if (B > n) { T = B; R = B; }
+  const long long T = std::max(real, (long long)pad_tokens_to);
+  if (B > n || T > real) {
+    for (int i = 0; i < n; ++i)
+      if (want_counts[i] != 1) return fail(BLM_E_USAGE, "only a step of one wanted place per sequence can be padded");
+    R = B;
+  }
   if (T > 2147483647LL || R > 2147483647LL) return fail(BLM_E_USAGE, "step too large");
   const int G = (int)c->groups.size();
   if (blm_step_size(G, (int)T, B, (int)R, width) > cap) return fail(BLM_E_USAGE, "the step's buffer is too small");
@@ -313,12 +316,14 @@ extern "C" int blm_step_fill(const BlmCache* c, int n, const int* slots, const i
     cu[i + 1] = t;
     after[i] = past + counts[i];
   }
-  for (int i = n; i < B; ++i) {   // padding rows of a decode step
-    tok[t] = 0; pos[t] = 0; seq[t] = -1; ++t;
-    rows[r++] = i;
+  for (int i = n; i < B; ++i) {   // padding sequences: no tokens, no slot
+    rows[r++] = 0;
     slot_out[i] = -1;
     cu[i + 1] = t;
     after[i] = 0;
+  }
+  for (; t < T; ++t) {   // padding tokens: of no sequence
+    tok[t] = 0; pos[t] = 0; seq[t] = -1;
   }
   for (int g = 0; g < G; ++g) {
     const int rc = page_rows(*c, g, B, slot_out, width, tables + (size_t)g * B * width);

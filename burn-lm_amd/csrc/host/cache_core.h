@@ -10,7 +10,7 @@
 extern "C" {
 #endif
 
-#define BLM_HOST_ABI 1
+#define BLM_HOST_ABI 2
 
 #define BLM_OK 0
 #define BLM_E_FULL 1      // no free slot, or not enough free pages
@@ -61,16 +61,18 @@ int blm_cache_live_slots(const BlmCache*, int* out);     // ascending; returns t
 //   sequence [B + 1], lengths after the step [B], wanted rows [R], then for every group a page
 //   table [B, width]
 // for n sequences that bring counts[i] tokens (tokens: all of them in order) and ask for
-// want_counts[i] places (wants: places within each sequence's own tokens).  B = max(n, pad_to):
-// with pad_to > n every sequence must bring one token and ask for it (a decode step), and the
-// step is filled up with padding rows (token 0, position 0, sequence -1, slot -1) so that its
-// shape is that of a recorded graph; then T = R = B.  Lengths are the cache's, before advance.
+// want_counts[i] places (wants: places within each sequence's own tokens).  Lengths are the
+// cache's, before advance.
+// Padding to the shape of a recorded graph: B = max(n, pad_seqs_to), T = max(tokens, pad_tokens_to).
+// A padded step must ask for exactly one place per sequence (R = B).  Padding sequences bring no
+// token (slot -1, length 0, their wanted row is row 0 and is dropped by the caller); padding tokens
+// stand behind the real ones and belong to no sequence (token 0, position 0, sequence -1).
 // meta: T, R, most tokens of one sequence, greatest length after the step.  The caller sizes
 // `out` with blm_step_size.
 long long blm_step_size(int n_groups, int T, int B, int R, int width);
 int blm_step_fill(const BlmCache*, int n, const int* slots, const int* counts, const int* tokens,
-                  const int* want_counts, const int* wants, int pad_to, int width, int* out, long long cap,
-                  int* meta);
+                  const int* want_counts, const int* wants, int pad_seqs_to, int pad_tokens_to, int width,
+                  int* out, long long cap, int* meta);
 
 #ifdef __cplusplus
 }

@@ -39,7 +39,7 @@ def build_step(entries: Sequence, lengths: Sequence[int], cache, device) -> Step
     width = max(1, (max_after + cache.page_size - 1) // cache.page_size)
     size = cache.step_size(T, B, R, width)
     host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
-    cache.fill_step(entries, 0, width, host.data_ptr(), size)
+    cache.fill_step(entries, 0, 0, width, host.data_ptr(), size)
     dev = host.to(device, non_blocking=True)
     o = 0
 

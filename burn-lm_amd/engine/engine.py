@@ -36,8 +36,8 @@ class Engine:
         model.prepare_positions(max_context)
         self.max_context = max_context
         self.vocab_size = model.vocab_size
-        from .graphs import DecodeGraphs
-        self.graphs = DecodeGraphs(self) if graphs else None
+        from .graphs import StepGraphs
+        self.graphs = StepGraphs(self) if graphs else None
 
     # ---- sequences ---------------------------------------------------------------------------
     def open(self) -> int:
@@ -76,7 +76,7 @@ class Engine:
         lengths = [self.cache.length(s) for s, _, _ in entries]
         self.cache.reserve([(s, len(t)) for s, t, _ in entries])  # raises before any change
         key = self.graphs.key_for(entries, lengths) if self.graphs is not None else None
-        logits = self.graphs.run(key, entries, lengths) if key is not None else None
+        logits = self.graphs.run(key, entries) if key is not None else None
         if logits is None:
             step = self.build_step(entries, lengths)
             logits = self.model.forward(step, self.cache)

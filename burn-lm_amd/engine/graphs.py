@@ -1,14 +1,18 @@
-"""Decode steps replayed as HIP graphs.
+"""Steps replayed as HIP graphs.
 
-A decode step is some hundred small kernels; launched one by one from Python they cost more time
-than they run.  For every shape of decode step (sequences rounded up to a bucket, page-table width
-rounded up to a bucket) the step is run once eagerly, then captured, and from then on replayed: the
-host only refreshes one int32 buffer (tokens, positions, page tables) and launches the graph.
+A step is some hundred kernels; launched one by one from Python they cost more time than they run
+as long as the step is small: every decode step, and prompts up to a few thousand tokens.  For
+every shape of such a step (sequences rounded up to a bucket, tokens rounded up to a bucket,
+page-table width rounded up to a bucket) the step is run once eagerly, then captured, and from then
+on replayed: the host only refreshes one int32 buffer (tokens, positions, page tables) and
+launches the graph.  Two kinds of step are recorded: decode steps (one token per sequence, its
+logits wanted) and prompt steps (any number of tokens per sequence, the last one's logits wanted).
 
-Places of the bucket that no sequence fills are padding: their sequence index is -1, so they write
-no cache and their rows are dropped; the kernels compute every row on its own, so padding changes
-no result.  Only models whose parts all declare ``graph_safe`` are replayed this way, and no memset
-node is recorded (buffers are cleared, where needed, by kernels).
+Places of the bucket that nothing fills are padding: padding tokens belong to no sequence (index
+-1), so they write no cache; padding sequences bring no token; their rows are dropped.  The kernels
+compute every row on its own, so padding changes no result.  Only models whose parts all declare
+``graph_safe`` are replayed this way, and no memset node is recorded (buffers are cleared, where
+needed, by kernels).
 """
 from __future__ import annotations
 
@@ -30,6 +34,20 @@ def batch_bucket(n: int):
     return None
 
 
+# prompt steps: total tokens of the step, and at most this many sequences (a step's attention
+# launches blocks for bucket sequences x bucket tokens; beyond these sizes the launches are no
+# longer what a step's time goes to)
+TOKEN_BUCKETS = (64, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
+PROMPT_MAX_SEQS = 16
+
+
+def token_bucket(n: int):
+    for b in TOKEN_BUCKETS:
+        if n <= b:
+            return b
+    return None
+
+
 def width_bucket(pages: int, max_width: int) -> int:
     w = 8
     while w < pages:
@@ -38,13 +56,18 @@ def width_bucket(pages: int, max_width: int) -> int:
 
 
 class _Captured:
-    def __init__(self, engine, B: int, W: int, pool):
+    """One recorded shape: B sequences, T tokens (T = 0: a decode step, one token per sequence),
+    page tables W wide."""
+
+    def __init__(self, engine, B: int, T: int, W: int, pool):
         cache, dev = engine.cache, engine.rt.device
         G = len(cache.groups)
-        self.B, self.W = B, W
+        self.B, self.T, self.W = B, T, W
+        self.decode = T == 0
+        NT = B if self.decode else T           # tokens of the recorded step
         self.copied = None
-        n = 7 * B + 1 + G * B * W          # the step's index arrays ...
-        self.src_at = n                    # ... and behind them, for run_ahead, where each row's token comes from
+        n = 3 * NT + 4 * B + 1 + G * B * W     # the step's index arrays ...
+        self.src_at = n                        # ... and behind them, for run_ahead, where each row's token comes from
         self.host = torch.zeros(n + B, dtype=torch.int32).pin_memory()
         self.host_np = self.host.numpy()
         self.dev = torch.zeros(n + B, dtype=torch.int32, device=dev)
@@ -56,16 +79,16 @@ class _Captured:
             o += k
             return v
 
-        token_ids, positions, token_seq, seq_slots = take(B), take(B), take(B), take(B)
+        token_ids, positions, token_seq, seq_slots = take(NT), take(NT), take(NT), take(B)
         cu, after, rows = take(B + 1), take(B), take(B)
         tables = {gi: take(B * W).view(B, W) for gi in range(G)}
         self.src_rows = take(B)
         span = min(W * cache.page_size, cache.max_context)
-        self.step = Step(n_tokens=B, n_seqs=B, n_wanted=B, token_ids=token_ids, positions=positions,
+        self.step = Step(n_tokens=NT, n_seqs=B, n_wanted=B, token_ids=token_ids, positions=positions,
                          token_seq=token_seq, seq_slots=seq_slots, cu_seqlens=cu, lens_after=after, want_rows=rows,
-                         block_tables=tables, max_new=1, max_position=span - 1, max_len_after=span, is_decode=True,
-                         host_slots=[], host_new=[])
-        self.fill([], [], cache)       # all padding: valid contents while capturing
+                         block_tables=tables, max_new=1 if self.decode else T, max_position=span - 1,
+                         max_len_after=span, is_decode=self.decode, host_slots=[], host_new=[])
+        self.fill([], cache)       # all padding: valid contents while capturing
         self.dev.copy_(self.host)
         self.graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize()
@@ -81,22 +104,23 @@ class _Captured:
                 gc.enable()
         torch.cuda.synchronize()
 
-    def fill(self, entries, lengths, cache):
-        """Host image of the index buffer for these (slot, [token], [0]) entries, the rest padding;
+    def fill(self, entries, cache):
+        """Host image of the index buffer for these (slot, tokens, [last]) entries, the rest padding;
         written by the native core straight into the pinned buffer."""
         B, W = self.B, self.W
+        NT = B if self.decode else self.T
         if entries:
-            cache.fill_step(entries, B, W, self.host.data_ptr(), self.src_at)
+            cache.fill_step(entries, B, NT, W, self.host.data_ptr(), self.src_at)
             return
         # all padding (used while recording): token 0, position 0, no sequence, no slot, no pages
-        flat = [0] * B + [0] * B + [-1] * B + [-1] * B + list(range(B + 1)) + [0] * B + list(range(B))
+        flat = [0] * NT + [0] * NT + [-1] * NT + [-1] * B + [0] * (B + 1) + [0] * B + [0] * B
         flat += [-1] * (len(cache.groups) * B * W)
         self.host[: self.src_at].copy_(torch.tensor(flat, dtype=torch.int32))
 
-    def run(self, entries, lengths, cache):
+    def run(self, entries, cache):
         if self.copied is not None:
             self.copied.synchronize()      # the last copy out of the host image must be over before it changes
-        self.fill(entries, lengths, cache)
+        self.fill(entries, cache)
         self.dev.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
@@ -104,12 +128,12 @@ class _Captured:
         return self.logits[: len(entries)].clone()   # the graph's own output buffer is overwritten by the next replay
 
     def run_ahead(self, slots, rows, tokens_dev, cache):
-        """Like run(), but row i's token is tokens_dev[rows[i]], taken on the device: the host
-        need not have seen the tokens of the step before.  The logits come back without a copy."""
+        """Like run() for a decode step, but row i's token is tokens_dev[rows[i]], taken on the device:
+        the host need not have seen the tokens of the step before.  The logits come back without a copy."""
         if self.copied is not None:
             self.copied.synchronize()
         n = len(slots)
-        self.fill([(s, [0], [0]) for s in slots], None, cache)
+        self.fill([(s, [0], [0]) for s in slots], cache)
         self.host_np[self.src_at: self.src_at + n] = rows
         self.dev.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()
@@ -119,39 +143,46 @@ class _Captured:
         return self.logits[:n]      # the graph's own buffer: good until the next replay of this shape
 
 
-class DecodeGraphs:
+class StepGraphs:
     def __init__(self, engine):
         # a weak reference: the engine owns this object, and a cycle would leave the graphs to the
         # cyclic collector, which may run at any time (see the note on capture above)
         self._engine = weakref.ref(engine)
-        self.captured: Dict[Tuple[int, int], _Captured] = {}
-        self.seen = set()
+        self.captured: Dict[Tuple[int, int, int], _Captured] = {}
         self.pool = None
         self.enabled = all(p.graph_safe for p in engine.model.all_parts())
         self.replays = 0
 
     def key_for(self, entries, lengths):
-        """Bucket key of a decode step, or None if the step cannot be replayed from a graph."""
-        if not self.enabled or any(len(t) != 1 or w != [0] for _, t, w in entries):
+        """Bucket key (sequences, tokens or 0 for a decode step, table width) of a step, or None if
+        the step cannot be replayed from a graph."""
+        if not self.enabled or any(w != [len(t) - 1] for _, t, w in entries):
             return None
+        cache = self._engine().cache
+        tokens = sum(len(t) for _, t, _ in entries)
         B = batch_bucket(len(entries))
         if B is None:
             return None
-        cache = self._engine().cache
-        pages = (max(lengths) + 1 + cache.page_size - 1) // cache.page_size
-        return B, width_bucket(pages, cache.table_width)
+        if tokens == len(entries):
+            T = 0
+        else:
+            T = token_bucket(tokens)
+            if T is None or B > PROMPT_MAX_SEQS:
+                return None
+        pages = (max(past + len(t) for past, (_, t, _) in zip(lengths, entries)) + cache.page_size - 1) // cache.page_size
+        return B, T, width_bucket(pages, cache.table_width)
 
-    def run(self, key, entries, lengths):
+    def run(self, key, entries):
         """Replays the step if its shape has been captured; returns None if it must run eagerly
         (the first time a shape is met; it is captured right after that run)."""
         c = self.captured.get(key)
         if c is None:
             return None
         self.replays += 1
-        return c.run(entries, lengths, self._engine().cache)
+        return c.run(entries, self._engine().cache)
 
     def run_ahead(self, key, slots, rows, tokens_dev):
-        """Replays a recorded shape with the tokens taken on the device; None if it is not recorded."""
+        """Replays a recorded decode shape with the tokens taken on the device; None if it is not recorded."""
         c = self.captured.get(key)
         if c is None:
             return None
@@ -165,4 +196,4 @@ class DecodeGraphs:
             return
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
-        self.captured[key] = _Captured(self._engine(), key[0], key[1], self.pool)
+        self.captured[key] = _Captured(self._engine(), key[0], key[1], key[2], self.pool)

@@ -167,13 +167,14 @@ def test_random_traffic_keeps_the_books():
     assert c.pages_in_use() == 0 and c.free_slots == 5
 
 
-def _fill(c, entries, pad_to, width):
-    T = max(sum(len(t) for _, t, _ in entries), pad_to)
-    B = max(len(entries), pad_to)
-    R = max(sum(len(w) for _, _, w in entries), pad_to)
+def _fill(c, entries, pad_seqs, width, pad_tokens=None):
+    pad_tokens = pad_seqs if pad_tokens is None else pad_tokens
+    T = max(sum(len(t) for _, t, _ in entries), pad_tokens)
+    B = max(len(entries), pad_seqs)
+    R = max(sum(len(w) for _, _, w in entries), pad_seqs)
     size = c.step_size(T, B, R, width)
     host = torch.full((size,), 12345, dtype=torch.int32)
-    meta = c.fill_step(entries, pad_to, width, host.data_ptr(), size)
+    meta = c.fill_step(entries, pad_seqs, pad_tokens, width, host.data_ptr(), size)
     return host.tolist(), meta
 
 
@@ -202,10 +203,33 @@ def test_step_assembly_pads_a_decode_step_to_a_recorded_shape():
     c.reserve([(a, 1), (b, 1)])
     flat, meta = _fill(c, [(a, [40], [0]), (b, [41], [0])], 4, 8)
     assert meta == (4, 4, 1, 18)
-    want = [40, 41, 0, 0] + [17, 3, 0, 0] + [0, 1, -1, -1] + [a, b, -1, -1] + [0, 1, 2, 3, 4] + [18, 4, 0, 0] + [0, 1, 2, 3]
+    # padding sequences bring no token (their wanted row is row 0, dropped by the caller); padding
+    # tokens stand behind the real ones and belong to no sequence
+    want = [40, 41, 0, 0] + [17, 3, 0, 0] + [0, 1, -1, -1] + [a, b, -1, -1] + [0, 1, 2, 2, 2] + [18, 4, 0, 0] + [0, 1, 0, 0]
     for row in c.page_table(0, [a, b, -1, -1], 8):
         want += row
     assert flat == want and want[-8:] == [-1] * 8
+
+
+def test_step_assembly_pads_a_prompt_step_to_a_recorded_shape():
+    """Two prompts of 3 and 2 tokens, the second on top of 17 cached ones, in a shape of 4 sequences
+    and 8 tokens: the last token of each is wanted."""
+    c = make(max_seqs=4)
+    a, b = c.open(), c.open()
+    c.reserve([(b, 17)]); c.advance(b, 17)
+    c.reserve([(a, 3), (b, 2)])
+    flat, meta = _fill(c, [(a, [7, 8, 9], [2]), (b, [5, 6], [1])], 4, 8, pad_tokens=8)
+    assert meta == (8, 4, 3, 19)
+    want = ([7, 8, 9, 5, 6, 0, 0, 0] + [0, 1, 2, 17, 18, 0, 0, 0] + [0, 0, 0, 1, 1, -1, -1, -1] + [a, b, -1, -1]
+            + [0, 3, 5, 5, 5] + [3, 19, 0, 0] + [2, 4, 0, 0])
+    for row in c.page_table(0, [a, b, -1, -1], 8):
+        want += row
+    assert flat == want
+    # tokens alone can be padded too, and a shape smaller than the step pads nothing
+    flat, meta = _fill(c, [(a, [7, 8, 9], [2])], 0, 8, pad_tokens=4)
+    assert meta == (4, 1, 3, 3) and flat[:12] == [7, 8, 9, 0, 0, 1, 2, 0, 0, 0, 0, -1]
+    flat, meta = _fill(c, [(a, [7, 8, 9], [2])], 1, 8, pad_tokens=2)
+    assert meta == (3, 1, 3, 3)
 
 
 def test_step_assembly_refuses_what_it_cannot_lay_out():
@@ -214,16 +238,18 @@ def test_step_assembly_refuses_what_it_cannot_lay_out():
     c.reserve([(a, 4)])
     host = torch.zeros(64, dtype=torch.int32)
     with pytest.raises(CacheError, match="padded"):
-        c.fill_step([(a, [1, 2], [0])], 4, 2, host.data_ptr(), 64)
+        c.fill_step([(a, [1, 2], [0, 1])], 4, 0, 2, host.data_ptr(), 64)
+    with pytest.raises(CacheError, match="padded"):
+        c.fill_step([(a, [1, 2], [])], 0, 8, 2, host.data_ptr(), 64)
     with pytest.raises(CacheError, match="too small"):
-        c.fill_step([(a, [1, 2, 3, 4], [0])], 0, 2, host.data_ptr(), 5)
+        c.fill_step([(a, [1, 2, 3, 4], [0])], 0, 0, 2, host.data_ptr(), 5)
     with pytest.raises(CacheError, match="outside"):
-        c.fill_step([(a, [1, 2], [2])], 0, 2, host.data_ptr(), 64)
+        c.fill_step([(a, [1, 2], [2])], 0, 0, 2, host.data_ptr(), 64)
     with pytest.raises(CacheError, match="not open"):
-        c.fill_step([(3, [1], [0])], 0, 2, host.data_ptr(), 64)
+        c.fill_step([(3, [1], [0])], 0, 0, 2, host.data_ptr(), 64)
     with pytest.raises(CacheError, match="wider"):
         c.reserve([(a, 40)])
-        c.fill_step([(a, [1], [0])], 0, 1, host.data_ptr(), 64)
+        c.fill_step([(a, [1], [0])], 0, 0, 1, host.data_ptr(), 64)
 
 
 def test_advance_needs_reserved_pages():

@@ -234,6 +234,47 @@ def test_graph_replays_equal_eager_steps(folders, dtype):
     assert max(g.length(sg[i]) for i in live) > 512, "the page table grew past the first width bucket"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_prompt_steps_replayed_from_graphs(folders, name, dtype):
+    """Batches of unequal prompts one after another, slots used again: the first batch of a shape
+    runs eagerly and is recorded, the later ones are replayed with padding sequences and padding
+    tokens, with eager work and synchronisations between the replays.  Every prompt's last logits
+    equal the plain implementation's, a prompt's second chunk on top of a replayed first one too,
+    and so do the tokens decoded after a replayed prompt (they read the cache it wrote)."""
+    cfg, seed = TINIES[name]
+    plain = P.load_model_folder(folders[name])
+    eng = load(folders[name], dtype, max_tokens=4096)
+    V = cfg["vocab_size"]
+    batches = [[40, 7, 90], [64, 1, 20, 33], [100, 3], [5, 5, 5, 120], [130], [61, 2, 70, 1], [150, 30], [128]]
+    seen_replay = 0
+    for bi, lens in enumerate(batches):
+        prompts = [random_tokens(1000 + 10 * bi + i, V, n + 3) for i, n in enumerate(lens)]
+        want = [P.transformer_forward([p], plain)[0] for p in prompts]
+        slots = [eng.open() for _ in lens]
+        before = eng.graphs.replays
+        got = eng.step([(s, p[:n], [n - 1]) for s, p, n in zip(slots, prompts, lens)]).double().cpu().numpy()
+        seen_replay += eng.graphs.replays - before
+        for i, n in enumerate(lens):
+            assert rel_err(got[i], want[i][n - 1]) <= TOL[dtype], f"batch {bi} prompt {i} ({n} tokens)"
+        if bi % 3 == 1:     # eager work between replays: a step that asks for every row cannot be replayed
+            x = eng.open(); eng.step([(x, prompts[0][:9], list(range(9)))]); eng.close(x)
+            torch.cuda.synchronize()
+        # a second chunk of two tokens on top of the first, then one decoded token
+        got = eng.step([(s, p[n:n + 2], [1]) for s, p, n in zip(slots, prompts, lens)]).double().cpu().numpy()
+        for i, n in enumerate(lens):
+            assert rel_err(got[i], want[i][n + 1]) <= TOL[dtype], f"batch {bi} prompt {i}: second chunk"
+        got = eng.step([(s, [p[n + 2]], [0]) for s, p, n in zip(slots, prompts, lens)]).double().cpu().numpy()
+        for i, n in enumerate(lens):
+            assert rel_err(got[i], want[i][n + 2]) <= TOL[dtype], f"batch {bi} prompt {i}: decoded token"
+        for s in slots:
+            eng.close(s)
+    assert eng.cache.pages_in_use() == 0
+    prompt_shapes = [k for k in eng.graphs.captured if k[1] > 0]
+    # whole prompts replayed (batches 3 and 5 have the shape of batch 0), and the second chunks
+    assert seen_replay >= 2 and len(prompt_shapes) >= 4 and eng.graphs.replays >= 8, (seen_replay, sorted(eng.graphs.captured))
+
+
 def test_a_part_that_is_not_graph_safe_turns_replay_off(folders):
     from burn_lm_amd.parts.attention import Attention
     eng = load(folders["A"], "float32")
