@@ -177,7 +177,7 @@ __device__ __forceinline__ void load_q(const bf16* qrow, uint4* qf) {
 // padded by 16 bytes so that the fragment reads do not collide.
 // ---------------------------------------------------------------------------------------
 template <int HD>
-__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 4 : (HD <= 128 ? 2 : 1))))
+__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 4 : (HD <= 128 ? 2 : 1), HD <= 64 ? 8 : (HD <= 128 ? 2 : 1))))
     attn_prefill_mfma_kernel(const bf16* __restrict__ q, int q_row_stride, bf16* __restrict__ out,
                              const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
                              const int* __restrict__ block_table, int table_width,
