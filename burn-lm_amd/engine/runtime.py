@@ -103,12 +103,15 @@ class Runtime:
                 return ops.gemv_mfma(x, packed, out, K)
         if out is None:
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
-        if packed is not None and aligned and out_dtype == torch.float32 and M <= MFMA_SKINNY_MAX_ROWS:
-            # float32 results (logits) for rows whose width the wide form does not take: 16 rows at a
-            # time; the weights stream once per 16 rows, which still beats the plain tiled kernel by far
-            for r in range(0, M, 16):
-                ops.gemv_mfma(x[r:r + 16], packed, out[r:r + 16], K)
-            return out
+        if packed is not None and aligned and out_dtype == torch.float32:
+            # float32 results (logits) for more rows than one skinny product takes at this width: the
+            # most rows it does take at a time (64, 32 or 16); the weights stream once per chunk, which
+            # still beats the plain tiled kernel by far
+            chunk = next((c for c in (64, 32, 16) if ops.gemv_mfma_supported(c, N, K)), 0)
+            if chunk:
+                for r in range(0, M, chunk):
+                    ops.gemv_mfma(x[r:r + chunk], packed, out[r:r + chunk], K)
+                return out
         if M <= SKINNY_MAX_ROWS and aligned:
             return ops.gemv_skinny(x, w, out)
         if out_dtype == torch.bfloat16:
