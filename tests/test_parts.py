@@ -151,7 +151,7 @@ def test_embedding_and_head_parts(rt):
     assert h.dtype == torch.float32 and torch.equal(h.cpu(), t["e"][[300, 0, 17]].float())
     head = registry.part("head", "linear")(dict(vocab=301, width=72), dict(weight="h"))
     head.bind(on_gpu(t), rt)
-    for rows in (2, 30):
+    for rows in (2, 30, 150):   # one skinny product, one with several row tiles, chunks of 64 rows
         x = torch.randn(rows, 72, generator=torch.Generator().manual_seed(7)).to(rt.dtype)
         y = head.forward(x.to("cuda"))
         assert y.dtype == torch.float32 and y.shape == (rows, 301)
