@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X, with roofline fractions.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers L]
+    python bench.py --preset llama3.2-3b --unequal 16 [--generate 256]     (an unequal batch, end to end)
 
 A "step" is one decode step of the whole batch: the engine's step function on one token per
 sequence, the sampling kernel, and the tokens' trip to the host, as the generation loop does it.
@@ -108,6 +109,43 @@ def time_prefill(engine, T, reps=3):
     return best
 
 
+def run_unequal(args):
+    """An unequal batch through the generation loop: --unequal N prompts of 64..2048 seeded random
+    tokens in one prefill step, then --generate greedy tokens each.  One JSON line of its own."""
+    import numpy as np
+    import torch
+    from burn_lm_amd.config.presets import preset
+    from burn_lm_amd.engine.generate import generate
+    from burn_lm_amd.engine.loading import random_engine
+    from burn_lm_amd.sampling.sampler import Sampler
+
+    rng = np.random.default_rng(0)
+    lens = [int(x) for x in rng.integers(64, 2049, args.unequal)]
+    context = (max(lens) + args.generate + 63) // 64 * 64
+    engine = random_engine(preset(args.preset), seed=0, dtype=args.dtype, max_tokens=args.unequal * context,
+                           max_seqs=args.unequal, max_context=context)
+    prompts = [[int(t) for t in rng.integers(0, engine.vocab_size, n)] for n in lens]
+    best = None
+    for _ in range(3):      # the first run records the graphs of its shapes
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _, stats = generate(engine, prompts, Sampler(temperature=0.0), args.generate, batch_size=args.unequal)
+        torch.cuda.synchronize()
+        whole = time.perf_counter() - t0
+        if best is None or whole < best[0]:
+            best = (whole, stats)
+    whole, stats = best
+    print(json.dumps({
+        "metric": "generation_seconds", "value": round(whole, 4), "unit": "s", "n_gpus": 1, "higher_is_better": False,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (seeded random weights and token ids)",
+        "config": {"model": args.preset, "sequences": args.unequal, "prompt_tokens": sum(lens), "shortest": min(lens),
+                   "longest": max(lens), "generated_each": args.generate, "sampling": "greedy"},
+        "prefill": {"value": round(stats.prompt_tokens / stats.prompt_seconds, 1), "tokens": stats.prompt_tokens,
+                    "ms": round(stats.prompt_seconds * 1e3, 2)},
+        "decode": {"value": round(stats.decode_tokens / stats.decode_seconds, 1), "tokens": stats.decode_tokens,
+                   "ms": round(stats.decode_seconds * 1e3, 2)}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -120,10 +158,16 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 decode points")
+    ap.add_argument("--unequal", type=int, default=0, metavar="N",
+                    help="instead of the decode measurement: N prompts of 64..2048 tokens through the generation loop")
+    ap.add_argument("--generate", type=int, default=256, help="tokens generated per prompt with --unequal")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this library has no multi-GPU path (run with --gpus 1)")
         sys.exit(2)
+
+    if args.unequal:
+        return run_unequal(args)
 
     import torch
     from burn_lm_amd.config.presets import preset
