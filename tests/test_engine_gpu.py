@@ -558,3 +558,60 @@ def test_random_schedules_of_steps(folders, name, dtype, seed):
     for s in list(live):
         eng.close(s)
     assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 5
+
+
+@pytest.mark.parametrize("name,dtype,seed", [("A", "bfloat16", 0), ("B", "float32", 1)])
+def test_random_schedules_through_recorded_graphs(folders, name, dtype, seed):
+    """Like the random schedules above, but every step asks for the last logits of each of its
+    sequences, so decode steps and prompt steps (whole prompts, pieces, mixed with single tokens)
+    run from recorded graphs as soon as their shape has been seen: slots and pages are used
+    again, shapes alternate, and every logit is compared with the plain implementation's."""
+    from burn_lm_amd.cache.cache import CacheFull
+    cfg, _ = TINIES[name]
+    plain = P.load_model_folder(folders[name])
+    rng = np.random.default_rng(1000 + seed)
+    eng = load(folders[name], dtype, max_tokens=1024, max_seqs=6, max_context=min(cfg["max_position_embeddings"], 256))
+    live, checked = {}, 0
+    for it in range(160):
+        if len(live) < 6 and (not live or rng.random() < 0.5):
+            try:
+                s = eng.open()
+            except CacheFull:
+                s = None
+            if s is not None:
+                toks = random_tokens(int(rng.integers(1 << 30)), cfg["vocab_size"], int(rng.integers(1, 200)))
+                live[s] = [toks, 0, P.transformer_forward([toks], plain)[0]]
+        picks = [s for s in live if rng.random() < 0.7]
+        rng.shuffle(picks)
+        single = rng.random() < 0.5
+        entries, expect = [], []
+        for s in picks:
+            toks, fed, want = live[s]
+            if fed == len(toks):
+                continue
+            n = 1 if single else int(min(len(toks) - fed, rng.choice([1, 2, 17, 64, 65, 130])))
+            entries.append((s, toks[fed:fed + n], [n - 1]))
+            expect.append(want[fed + n - 1])
+        if entries:
+            try:
+                got = eng.step(entries).double().cpu().numpy()
+            except CacheFull:
+                victim = max(live, key=lambda s: live[s][1])
+                eng.close(victim)
+                del live[victim]
+                continue
+            for s, t, _ in entries:
+                live[s][1] += len(t)
+            for g_row, w_row in zip(got, expect):
+                assert rel_err(g_row, w_row) <= TOL[dtype], f"iteration {it}"
+                checked += 1
+        for s in list(live):
+            if live[s][1] == len(live[s][0]) or rng.random() < 0.05:
+                eng.close(s)
+                del live[s]
+    for s in list(live):
+        eng.close(s)
+    assert eng.cache.pages_in_use() == 0
+    shapes = eng.graphs.captured
+    assert checked > 200 and eng.graphs.replays > 60 and any(k[1] > 0 for k in shapes) and any(k[1] == 0 for k in shapes)
+
