@@ -23,6 +23,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 __device__ __forceinline__ uint4 ld16(const bf16* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint4 ld16_stream(const bf16* p) { return load16_stream(p); }   // the weights: read once
 
 // KSTEPS: k-steps of 32 per wavefront.  MAXT: most threads of a block (sets the register budget).
 // KEEP_A: the activations' fragments stay in registers across the block's column tiles.
@@ -72,7 +73,7 @@ __global__ void __launch_bounds__(MAXT)
 #pragma unroll
       for (int s = 0; s < CH; ++s) {
         const int st = step0 + c + s;
-        w[s] = ld16(wt + (size_t)(st < k_steps ? st : k_steps - 1) * 512);
+        w[s] = ld16_stream(wt + (size_t)(st < k_steps ? st : k_steps - 1) * 512);
       }
       if (!KEEP_A) {
 #pragma unroll
@@ -162,7 +163,7 @@ __global__ void __launch_bounds__(512)
   if (PREFETCH) {
     const bf16* wt = wbase + (size_t)min(tile_begin, n_tiles - 1) * k_steps * 512;
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) w[s] = ld16(wt + woff[s]);
+    for (int s = 0; s < KSTEPS; ++s) w[s] = ld16_stream(wt + woff[s]);
   }
   uint4 a[MT][KSTEPS];
 #pragma unroll
@@ -182,11 +183,11 @@ __global__ void __launch_bounds__(512)
       const int next = tile + 1 < tile_end ? tile + 1 : tile;   // the last round re-reads its own (from the cache)
       const bf16* wt = wbase + (size_t)next * k_steps * 512;
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) wn[s] = ld16(wt + woff[s]);
+      for (int s = 0; s < KSTEPS; ++s) wn[s] = ld16_stream(wt + woff[s]);
     } else {
       const bf16* wt = wbase + (size_t)tile * k_steps * 512;
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) w[s] = ld16(wt + woff[s]);
+      for (int s = 0; s < KSTEPS; ++s) w[s] = ld16_stream(wt + woff[s]);
     }
     __builtin_amdgcn_sched_barrier(0);   // every load is issued before this tile's first MFMA
     f32x4_t acc[MT];

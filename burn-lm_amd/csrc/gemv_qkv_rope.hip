@@ -44,7 +44,7 @@ __global__ void __launch_bounds__(MAXT)
 #pragma unroll
   for (int s = 0; s < QR_KSTEPS; ++s) {
     const int st = step0 + s;
-    w[s] = *reinterpret_cast<const uint4*>(wt + (size_t)(st < k_steps ? st : k_steps - 1) * 512);
+    w[s] = load16_stream(wt + (size_t)(st < k_steps ? st : k_steps - 1) * 512);   // the weights: read once
   }
   const bf16* ap = A + (size_t)(row < M ? row : M - 1) * lda;
   uint4 a[QR_KSTEPS];
