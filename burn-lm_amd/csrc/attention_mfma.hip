@@ -333,9 +333,24 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
                             float* part_ml, int* arrivals, bf16* out) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
+  // Every wavefront brings its pages through a staging area of its own in shared memory: whole
+  // pages come in with 16-byte loads that cover complete cache lines and are used once (taking the
+  // MFMA fragments straight from global memory touches 16 bytes of 16 lines per instruction, which
+  // costs 7 % of a batch-64 step); the fragments are then read from the staged page, whose rows are
+  // padded as in the prefill kernel.  Nobody else touches a wavefront's area, so no barrier is
+  // needed, and the next page travels in registers while the current one is used.  The areas serve
+  // once more at the end, for the wavefronts' partial outputs.
+  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 4;
+  constexpr int CHUNKS = AM_PAGE * HD / 8;              // 16-byte pieces of a page (keys and values alike)
+  constexpr int PER_LANE = CHUNKS / BLM_WAVE;           // HD is a multiple of 16, so this is exact
+  constexpr int STAGE_ELEMS = AM_PAGE * KSTR + HD * VSTR;
+  constexpr int AREA_BYTES = STAGE_ELEMS * 2 > 16 * HD * 4 ? STAGE_ELEMS * 2 : 16 * HD * 4;
+  static_assert(CHUNKS % BLM_WAVE == 0 && (AM_PAGE * KSTR * 2) % 16 == 0 && AREA_BYTES % 16 == 0, "page staging layout");
   __shared__ float sm_m[AM_WAVES][16], sm_l[AM_WAVES][16];
-  __shared__ float sm_o[AM_WAVES][16][HD];
+  __shared__ __align__(16) unsigned char sm_area[AM_WAVES][AREA_BYTES];
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  bf16* const k_lds = reinterpret_cast<bf16*>(sm_area[wave]);
+  bf16* const v_lds = k_lds + AM_PAGE * KSTR;
   const int c = lane & 15, kg = lane >> 4;
   const int split = blockIdx.x;
   const int G = nh / nkv;
@@ -362,22 +377,49 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     uint4 qf[KS];
     load_q<HD>(q + (size_t)t * q_row_stride + (size_t)head * HD, qf);
     const float scale2 = scale * 1.4426950408889634f;
-    for (int pi = p_begin + wave; pi < p_end; pi += AM_WAVES) {
-      const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;
+    u32x4_t kreg[PER_LANE], vreg[PER_LANE];
+#define AD_FETCH(pi)                                                                          \
+  {                                                                                           \
+    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;                          \
+    _Pragma("unroll") for (int i = 0; i < PER_LANE; ++i) {                                    \
+      const int j = i * BLM_WAVE + lane;                                                      \
+      kreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kcache + base + (size_t)j * 8));   \
+      vreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vcache + base + (size_t)j * 8));   \
+    }                                                                                         \
+  }
+#define AD_STAGE()                                                                                            \
+  _Pragma("unroll") for (int i = 0; i < PER_LANE; ++i) {                                                        \
+    const int j = i * BLM_WAVE + lane;                                                                          \
+    const int kr = j / (HD / 8), kc = j - kr * (HD / 8);           /* key row, 16-byte column */                \
+    *reinterpret_cast<u32x4_t*>(k_lds + kr * KSTR + kc * 8) = kreg[i];                                          \
+    const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8); /* value row (a dim), 16-byte column */      \
+    u32x2_t* vd = reinterpret_cast<u32x2_t*>(v_lds + vr * VSTR + vc * 8);   /* rows are 8-byte aligned */       \
+    vd[0] = u32x2_t{vreg[i].x, vreg[i].y};                                                                      \
+    vd[1] = u32x2_t{vreg[i].z, vreg[i].w};                                                                      \
+  }
+    int pi = p_begin + wave;
+    if (pi < p_end) AD_FETCH(pi);
+    for (; pi < p_end; pi += AM_WAVES) {
+      AD_STAGE()
+      if (pi + AM_WAVES < p_end) AD_FETCH(pi + AM_WAVES);   // travels while this page is used
       const int key0 = pi * AM_PAGE;
       if (key0 + AM_PAGE - 1 <= pos && key0 >= lo)
-        attn_page<HD, true, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, lsum, o);
+        attn_page<HD, true, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, pos, lo, pos, scale2, m, lsum, o);
       else
-        attn_page<HD, false, HD, AM_PAGE, false>(kcache + base, vcache + base, qf, key0, pos, lo, pos, scale2, m, lsum, o);
+        attn_page<HD, false, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, pos, lo, pos, scale2, m, lsum, o);
     }
+#undef AD_FETCH
+#undef AD_STAGE
   }
+  // the staging area is free now: this wavefront's partial output goes there
+  float (*const sm_o)[HD] = reinterpret_cast<float (*)[HD]>(sm_area[wave]);
   if (kg == 0) { sm_m[wave][c] = m; sm_l[wave][c] = lsum[0]; }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int d = dt * 16 + kg * 4 + r;
-      if (HD % 16 == 0 || d < HD) sm_o[wave][c][d] = o[dt][r];
+      if (HD % 16 == 0 || d < HD) sm_o[c][d] = o[dt][r];
     }
   __syncthreads();
   for (int idx = threadIdx.x; idx < 16 * HD; idx += blockDim.x) {
@@ -391,7 +433,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     for (int k = 0; k < AM_WAVES; ++k) {
       const float f = (sm_m[k][cc] == M) ? 1.f : __builtin_amdgcn_exp2f(sm_m[k][cc] - M);   // maxima are in base 2
       L += sm_l[k][cc] * f;
-      O += sm_o[k][cc][d] * f;
+      O += reinterpret_cast<const float*>(sm_area[k])[cc * HD + d] * f;
     }
     if (n_splits == 1 || b < 0) {   // nothing to merge (a padding token gives zeros)
       out[((size_t)t * nh + kvh * G + g0 + cc) * HD + d] = from_float<bf16>(b < 0 ? 0.f : O / L);
