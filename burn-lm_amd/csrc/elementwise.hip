@@ -114,11 +114,18 @@ __global__ void __launch_bounds__(512)
     if (d < D) {
       load4<float>(hr + d, v[it]);
       if (dr) {
-        for (int p = 0; p < n_planes; ++p) {
-          float t[4];
-          load4<TD>(dr + p * plane_stride + d, t);
+        // four planes at a time: their loads are issued together (a loop that loads and adds plane
+        // by plane waits for memory once per plane), the adds keep the planes' order
+        for (int p0 = 0; p0 < n_planes; p0 += 4) {
+          float t[4][4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[it][e] += t[e];
+          for (int q = 0; q < 4; ++q) load4<TD>(dr + (size_t)min(p0 + q, n_planes - 1) * plane_stride + d, t[q]);
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (p0 + q < n_planes) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[it][e] += t[q][e];
+            }
         }
         if (write_h) store4<float>(hr + d, v[it]);
       }
