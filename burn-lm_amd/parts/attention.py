@@ -17,6 +17,22 @@ from .base import KVNeed, Mixer, TensorSpec
 
 # blocks the decode attention aims for when it cuts the key ranges into splits
 DECODE_TARGET_BLOCKS = int(os.environ.get("BLM_DECODE_BLOCKS", "512"))
+DECODE_MIN_BLOCKS = 128
+
+
+def decode_splits(pages: int, blocks: int, head_dim: int) -> int:
+    """Into how many pieces the decode attention cuts a sequence's pages.  Every piece is a block of
+    four wavefronts that take pages in turn, and the pieces' results are merged by the last block to
+    finish, so a piece should hold two pages per wavefront (eight), or one (four) while that leaves
+    fewer than DECODE_MIN_BLOCKS blocks; and there is no point in more blocks than the chip takes at
+    once (pages of wide heads hold more bytes: half as many blocks reach the same memory rate).
+    Measured at context 4096, head_dim 64, ms per step: batch 1: 16 pieces 0.870, 8: 0.880, 64: 1.002;
+    batch 2: 8 pieces 0.909, 16: 0.928; batch 4: 8 pieces 0.961, 16: 0.988; batch 8: 8 pieces best."""
+    target = DECODE_TARGET_BLOCKS if head_dim <= 64 else max(1, DECODE_TARGET_BLOCKS // 2)
+    n = min(max(1, pages // 8), (target + blocks - 1) // blocks)
+    if blocks * n < DECODE_MIN_BLOCKS:
+        n = max(n, min(max(1, pages // 4), (DECODE_MIN_BLOCKS + blocks - 1) // blocks))
+    return max(1, n)
 
 
 class Attention(Mixer):
@@ -62,10 +78,7 @@ class Attention(Mixer):
             span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
             pages = (span + view.page_size - 1) // view.page_size
             blocks = x.shape[0] * nkv * ((nh // nkv + 15) // 16)
-            # pages of wide heads hold more bytes: half as many blocks reach the same memory rate
-            # (measured at head_dim 128: 256 blocks 1.2 % faster per step than 512)
-            target = DECODE_TARGET_BLOCKS if hd <= 64 else max(1, DECODE_TARGET_BLOCKS // 2)
-            n_splits = max(1, min(pages, (target + blocks - 1) // blocks))
+            n_splits = decode_splits(pages, blocks, hd)
             rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                                view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
         elif aligned and rt.ops.attn_prefill_mfma_supported(rt.dtype, hd, view.page_size):

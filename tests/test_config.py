@@ -136,3 +136,22 @@ def test_tokenizers_for_the_command_line(tmp_path):
     assert f.encode("hello world") == [0, 1] and f.encode("hello", bos=True, eos=True) == [3, 0, 4]
     assert f.stop_ids() == [4, 5]            # <|eom_id|> is not in this file
     assert f.decode([3, 0, 1, 5]) == "hello world"
+
+
+def test_decode_attention_split_rule():
+    """How many pieces a sequence's pages are cut into for the decode attention: never more pieces
+    than pages, pieces of at least eight pages (four while the chip would be mostly idle), no more
+    blocks than the target."""
+    from burn_lm_amd.parts.attention import DECODE_MIN_BLOCKS, DECODE_TARGET_BLOCKS, decode_splits
+    assert DECODE_TARGET_BLOCKS == 512 and DECODE_MIN_BLOCKS == 128
+    # context 4096 (64 pages), 8 key-value heads: batch 1, 2, 4, 8, 16, 64
+    assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 64)] == [16, 8, 8, 8, 4, 1]
+    assert decode_splits(64, 8, 128) == 16 and decode_splits(64, 64, 128) == 4      # wide heads: half the blocks
+    assert decode_splits(1, 8, 64) == 1 and decode_splits(3, 8, 64) == 1 and decode_splits(8, 8, 64) == 2
+    assert decode_splits(2048, 8, 64) == 64                                         # a long context at batch 1
+    for pages in (1, 2, 5, 8, 9, 31, 64, 100, 1000):
+        for blocks in (1, 3, 8, 64, 500, 5000):
+            for hd in (64, 128):
+                n = decode_splits(pages, blocks, hd)
+                assert 1 <= n <= pages
+                assert n == 1 or pages // n >= 4
