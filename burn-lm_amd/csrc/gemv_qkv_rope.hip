@@ -6,7 +6,8 @@
 //
 // A block owns one rotation unit: the two 16-column tiles that hold partner lanes of one head.
 // With pairing 1 (lane i with i + head_dim/2) these are tiles j and j + head_dim/32 of the head;
-// with pairing 0 (lanes 2i, 2i+1) the partners sit in one tile and the unit is two adjacent tiles.
+// with pairing 0 (lanes 2i, 2i+1) the partners sit in one tile: see gemv_qkv_rope_tile_kernel, which
+// the entry point uses then (this kernel takes both pairings).
 // Value heads are not rotated and use the same unit shape.  Wavefronts 0..KW-1 work on the first
 // tile, KW..2KW-1 on the second, each on 512 of K; the partial tiles are summed through LDS and
 // the epilogue rotates and scatters them.
@@ -118,8 +119,91 @@ __global__ void __launch_bounds__(MAXT)
   }
 }
 
-extern "C" int blm_gemv_qkv_rope_supported(int M, int K, int hd) {
-  return (M >= 1 && M <= 16 && K >= 8 && K % 8 == 0 && K <= 4096 && hd >= 32 && hd % 32 == 0) ? 1 : 0;
+// Pairing 0 (partners are neighbours 2i, 2i+1): both partners sit in the same 16-column tile, so a
+// block owns ONE tile and its wavefronts split K.  That is twice as many blocks as with two-tile
+// units, which matters because the whole product is a few blocks per compute unit at most (3072
+// columns are 192 tiles).  Value heads are not rotated.  red: [wavefronts][256].
+template <int QR_KSTEPS>
+__global__ void __launch_bounds__(512)
+    gemv_qkv_rope_tile_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wp, bf16* __restrict__ qkv_out,
+                              const int* __restrict__ positions, const int* __restrict__ token_seq,
+                              const int* __restrict__ block_table, int table_width,
+                              const float2* __restrict__ cos_sin, bf16* __restrict__ kcache,
+                              bf16* __restrict__ vcache, int page_size, int M, int K, int lda, int ldq, int k_steps,
+                              int nh, int nkv, int hd, int store) {
+  extern __shared__ float red[];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int n_waves = blockDim.x / BLM_WAVE;
+  const int row = lane & 15, kg = lane >> 4;
+  const int tiles_per_head = hd / 16;
+  const int tile = blockIdx.x;
+  const int head = tile / tiles_per_head, col0 = (tile - head * tiles_per_head) * 16;
+  if (!store && head >= nh) return;   // keys and values belong to another layer's cache: only q is needed
+  const int step0 = wave * QR_KSTEPS;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+
+  const bf16* wt = Wp + ((size_t)tile * k_steps * 64 + lane) * 8;
+  uint4 w[QR_KSTEPS];
+#pragma unroll
+  for (int s = 0; s < QR_KSTEPS; ++s) {
+    const int st = step0 + s;
+    w[s] = load16_stream(wt + (size_t)(st < k_steps ? st : k_steps - 1) * 512);   // the weights: read once
+  }
+  const bf16* ap = A + (size_t)(row < M ? row : M - 1) * lda;
+  uint4 a[QR_KSTEPS];
+#pragma unroll
+  for (int s = 0; s < QR_KSTEPS; ++s) {
+    const int k = (step0 + s) * 32 + kg * 8;
+    const uint4 v = *reinterpret_cast<const uint4*>(ap + (k < K ? k : K - 8));
+    a[s] = (row < M && k < K) ? v : zero;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < QR_KSTEPS; ++s)
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
+                                                  __builtin_bit_cast(bf16x8_t, w[s]), acc, 0, 0, 0);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) red[wave * 256 + r * 64 + lane] = acc[r];
+  __syncthreads();
+
+  // epilogue: one thread per (token row m, column c of the tile)
+  for (int idx = threadIdx.x; idx < 256; idx += blockDim.x) {
+    const int r = idx >> 6, l2 = idx & 63, c = l2 & 15;
+    const int m = (l2 >> 4) * 4 + r;
+    if (m >= M) continue;
+    float x = 0.f, partner = 0.f;   // column c and its neighbour c ^ 1
+    for (int k2 = 0; k2 < n_waves; ++k2) {
+      x += red[k2 * 256 + idx];
+      partner += red[k2 * 256 + (idx ^ 1)];
+    }
+    const int b = token_seq[m];
+    const int pos = positions[m];
+    const int d = col0 + c;
+    float y = x;     // value heads are stored as they are
+    if (head < nh + nkv) {
+      const float2 cs = cos_sin[(size_t)pos * (hd / 2) + (d >> 1)];
+      y = (c & 1) == 0 ? x * cs.x - partner * cs.y : partner * cs.y + x * cs.x;
+    }
+    const bf16 o = from_float<bf16>(y);
+    if (head < nh) {
+      qkv_out[(size_t)m * ldq + (size_t)head * hd + d] = o;
+    } else if (b >= 0) {
+      const int page = block_table[(size_t)b * table_width + pos / page_size];
+      const int slot = pos % page_size;
+      if (page < 0) continue;
+      if (head < nh + nkv) kcache[(((size_t)page * nkv + (head - nh)) * page_size + slot) * hd + d] = o;
+      else vcache[((size_t)page * nkv + (head - nh - nkv)) * hd * page_size + (size_t)d * page_size + slot] = o;
+    }
+  }
+}
+
+// pairing 0 takes every head size that is a multiple of 16; pairing 1 (partners half a head apart,
+// two tiles per block) needs a multiple of 32
+extern "C" int blm_gemv_qkv_rope_supported(int M, int K, int hd, int pairing) {
+  const int step = pairing == 0 ? 16 : 32;
+  return (M >= 1 && M <= 16 && K >= 8 && K % 8 == 0 && K <= 4096 && hd >= step && hd % step == 0 &&
+          (pairing == 0 || pairing == 1)) ? 1 : 0;
 }
 
 // Wp: pack_weight of W_qkv [(nh + 2 nkv) * hd, K].  qkv_out: [M, ldq] bf16; only its first nh*hd
@@ -130,13 +214,28 @@ extern "C" int blm_gemv_qkv_rope(const void* A, const void* Wp, void* qkv_out, c
                                  const float* cos_sin, void* kcache, void* vcache, int page_size, int M, int K,
                                  int lda, int ldq, int nh, int nkv, int hd, int pairing, int store,
                                  hipStream_t stream) {
-  BLM_REQUIRE(blm_gemv_qkv_rope_supported(M, K, hd), "gemv_qkv_rope: M=%d K=%d head_dim=%d not supported "
-              "(M <= 16, K a multiple of 8 and at most 4096, head_dim a multiple of 32)", M, K, hd);
-  BLM_REQUIRE(nh > 0 && nkv > 0 && page_size > 0 && table_width > 0 && (pairing == 0 || pairing == 1),
-              "gemv_qkv_rope: bad geometry");
+  BLM_REQUIRE(blm_gemv_qkv_rope_supported(M, K, hd, pairing), "gemv_qkv_rope: M=%d K=%d head_dim=%d pairing=%d not "
+              "supported (M <= 16, K a multiple of 8 and at most 4096, head_dim a multiple of 16 for adjacent "
+              "pairs and of 32 for pairs half a head apart)", M, K, hd, pairing);
+  BLM_REQUIRE(nh > 0 && nkv > 0 && page_size > 0 && table_width > 0, "gemv_qkv_rope: bad geometry");
   BLM_REQUIRE(lda % 8 == 0 && lda >= K && ldq >= nh * hd, "gemv_qkv_rope: bad strides lda=%d ldq=%d", lda, ldq);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0, "gemv_qkv_rope: operands must be 16-byte aligned");
   const int k_steps = (K + 31) / 32;
+  const int tiles = (nh + 2 * nkv) * (hd / 16);
+  // Adjacent pairs: one tile per block while that is one round of blocks on the chip's 256 compute
+  // units (or the head size leaves no choice, or K is so wide that two-tile blocks would need 16
+  // wavefronts and spill); beyond that, blocks of two tiles (measured at 320 tiles, K = 3072: one
+  // tile per block 2.7 % of a step slower).
+  if (pairing == 0 && (tiles <= 256 || hd % 32 != 0 || k_steps > 96)) {
+    // 16 k-steps per wavefront: up to 8 wavefronts
+    const int waves = (k_steps + 15) / 16;
+    hipLaunchKernelGGL(gemv_qkv_rope_tile_kernel<16>, dim3(tiles), dim3(waves * BLM_WAVE), (size_t)waves * 256 * sizeof(float),
+                       stream, (const bf16*)A, (const bf16*)Wp, (bf16*)qkv_out, positions, token_seq, block_table,
+                       table_width, (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache, page_size, M, K, lda, ldq,
+                       k_steps, nh, nkv, hd, store);
+    BLM_LAUNCH_CHECK("gemv_qkv_rope_tile");
+    return 0;
+  }
   // all of a block's loads are in flight at once: 4 wavefronts per tile with 16 k-steps each up to
   // K = 2048, with 24 up to 3072 (their registers still fit), and 8 wavefronts with 16 up to 4096
   const int ksteps = (k_steps > 64 && k_steps <= 96) ? 24 : 16;

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 _lib = None
 _lock = threading.Lock()
 
@@ -47,7 +47,7 @@ _SIGNATURES = {
                       _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_gemv_mfma_group_limit": [_c_int],
-    "blm_gemv_qkv_rope_supported": [_c_int, _c_int, _c_int],
+    "blm_gemv_qkv_rope_supported": [_c_int, _c_int, _c_int, _c_int],
     "blm_gemv_qkv_rope": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
@@ -413,8 +413,9 @@ def gemv_mfma(a, packed, out, K, gated=False):
     return out
 
 
-def gemv_qkv_rope_supported(M, K, hd):
-    return bool(library().blm_gemv_qkv_rope_supported(int(M), int(K), int(hd)))
+def gemv_qkv_rope_supported(M, K, hd, pairing):
+    """pairing 0 (adjacent lanes): head_dim a multiple of 16; pairing 1 (half a head apart): of 32."""
+    return bool(library().blm_gemv_qkv_rope_supported(int(M), int(K), int(hd), int(pairing)))
 
 
 def gemv_qkv_rope(x, packed, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,

@@ -37,12 +37,14 @@ class Model:
         self.rt = None
 
     def all_parts(self):
+        """In the order they are bound: the position encodings first, because a mixer consults its
+        encoding while it binds its own projections."""
+        yield from self.positions.values()
         yield self.embedding
         for b in self.blocks:
             yield from b.parts()
         yield self.final_norm
         yield self.head
-        yield from self.positions.values()
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         specs: Dict[str, TensorSpec] = {}

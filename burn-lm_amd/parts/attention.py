@@ -59,8 +59,8 @@ class Attention(Mixer):
         self.heads, self.kv_heads, self.head_dim = p["heads"], p["kv_heads"], p["head_dim"]
         self.scale = float(p["scale"])
         self.window = int(p.get("window", 0))
-        self.position = p["position"]
         ws = [tensors[self.names[r]] for r in ("q", "k", "v")]
+        ws[0], ws[1], self.position = p["position"].for_projection(ws[0], ws[1], self.heads, self.kv_heads)
         if len({w.dtype for w in ws}) != 1:
             ws = [w.float() for w in ws]
         self.w_qkv = rt.weight(torch.cat(ws, dim=0))

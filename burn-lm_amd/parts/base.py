@@ -17,7 +17,8 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
   ``Mixer.forward(x, step, view) -> delta``; ``view`` is what the cache holds for this place
   in the layer order (``KVView``, ``StateView`` or ``None``).
 * ``FeedForward.forward(x, step) -> delta``.
-* ``PositionEncoding.prepare(n_positions, rt)`` and, for encodings that act on queries and keys,
+* ``PositionEncoding.prepare(n_positions, rt)``, ``for_projection(w_q, w_k, heads, kv_heads)`` (the
+  encoding may re-order the projections' rows when they are bound) and, for encodings that act on queries and keys,
   ``encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store)``; the attention mixer calls
   ``project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)``, whose default is the
   projection followed by ``encode_and_store`` and which an encoding may fuse.
@@ -100,6 +101,12 @@ class FeedForward(Part):
 class PositionEncoding(Part):
     def prepare(self, n_positions: int, rt) -> None:
         pass
+
+    def for_projection(self, w_q, w_k, heads: int, kv_heads: int):
+        """Called by a mixer when it binds its query and key projections ([heads * head_dim, width]
+        rows): returns (w_q, w_k, encoding) to use from then on.  An encoding may hand back
+        re-ordered rows and a variant of itself that computes the same function on them."""
+        return w_q, w_k, self
 
     def project_encode_store(self, x, w_qkv, step, view, heads, kv_heads, head_dim):
         """x @ w_qkv^T, then encode q and k by position and store k, v (unless view.store is

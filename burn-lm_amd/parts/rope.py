@@ -48,13 +48,39 @@ class RotaryEncoding(PositionEncoding):
             raise ValueError(f"rotary pairing {self.params['pairing']!r} unknown; one of {list(PAIRING)}")
         self.pairing = PAIRING[self.params["pairing"]]
         self.freqs = rope_frequencies(self.head_dim, self.params["theta"], self.params.get("scaling"))
-        self.table = None
+        self._shared = {"table": None, "n_positions": 0}    # one table for this encoding and its adjacent-pair twin
+        self._twin = None
+
+    table = property(lambda self: self._shared["table"])
+    n_positions = property(lambda self: self._shared["n_positions"])
 
     def prepare(self, n_positions, rt):
         ang = np.arange(n_positions, dtype=np.float64)[:, None] * self.freqs[None, :]
         cs = np.stack([np.cos(ang), np.sin(ang)], axis=-1).astype(np.float32)
-        self.table = torch.from_numpy(cs).to(rt.device)
-        self.n_positions = n_positions
+        self._shared["table"] = torch.from_numpy(cs).to(rt.device)
+        self._shared["n_positions"] = n_positions
+
+    def for_projection(self, w_q, w_k, heads, kv_heads):
+        """Pairs half a head apart are the same function as adjacent pairs on rows that are permuted
+        within every head (row ``r * head_dim/2 + i`` goes to ``2i + r``), which is the re-layout the
+        reference applies to such checkpoints (nn/llama/import.rs:99-126).  The kernels prefer
+        adjacent pairs (both partners in one 16-column tile), so the projection's rows are permuted
+        when they are bound and a twin of this encoding with adjacent pairs, sharing its table, does
+        the rotating.  Keys are cached in the permuted lane order; the scores do not change, since
+        queries are permuted alike."""
+        if self.pairing == PAIRING["interleaved"]:
+            return w_q, w_k, self
+        if self._twin is None:
+            twin = RotaryEncoding(dict(self.params, pairing="interleaved"), self.names)
+            twin.bind({}, self.rt)
+            twin._shared = self._shared
+            self._twin = twin
+        hd = self.head_dim
+
+        def permute(w, n):
+            return w.reshape(n, 2, hd // 2, w.shape[1]).transpose(1, 2).reshape(n * hd, w.shape[1]).contiguous()
+
+        return permute(w_q, heads), permute(w_k, kv_heads), self._twin
 
     def encode_and_store(self, qkv, step, view, heads, kv_heads, head_dim, store=True):
         if step.max_position >= self.n_positions:
@@ -70,7 +96,7 @@ class RotaryEncoding(PositionEncoding):
         packed = getattr(w_qkv, "packed", None)
         M, K = x.shape
         if (packed is not None and not getattr(w_qkv, "gated", False) and x.dtype == torch.bfloat16
-                and rt.ops.gemv_qkv_rope_supported(M, K, head_dim) and x.stride(0) % 8 == 0
+                and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing) and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0 and view.k.dtype == torch.bfloat16):
             if step.max_position >= self.n_positions:
                 raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
