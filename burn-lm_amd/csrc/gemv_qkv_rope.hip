@@ -198,12 +198,105 @@ __global__ void __launch_bounds__(512)
   }
 }
 
-// pairing 0 takes every head size that is a multiple of 16; pairing 1 (partners half a head apart,
-// two tiles per block) needs a multiple of 32
+// 17 to 64 rows, adjacent pairs: as gemv_qkv_rope_tile_kernel, with MT row tiles of 16 against every
+// weight fragment (the activations of all row tiles stay in registers, as in gemv_mfma_rows_kernel:
+// MT * QR_KSTEPS fragments, at most 32).  One tile per block; red: [wavefronts][MT][256].
+template <int MT, int QR_KSTEPS>
+__global__ void __launch_bounds__(512)
+    gemv_qkv_rope_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wp, bf16* __restrict__ qkv_out,
+                              const int* __restrict__ positions, const int* __restrict__ token_seq,
+                              const int* __restrict__ block_table, int table_width,
+                              const float2* __restrict__ cos_sin, bf16* __restrict__ kcache,
+                              bf16* __restrict__ vcache, int page_size, int M, int K, int lda, int ldq, int k_steps,
+                              int nh, int nkv, int hd, int store) {
+  extern __shared__ float red[];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int n_waves = blockDim.x / BLM_WAVE;
+  const int row = lane & 15, kg = lane >> 4;
+  const int tiles_per_head = hd / 16;
+  const int tile = blockIdx.x;
+  const int head = tile / tiles_per_head, col0 = (tile - head * tiles_per_head) * 16;
+  if (!store && head >= nh) return;   // keys and values belong to another layer's cache: only q is needed
+  const int step0 = wave * QR_KSTEPS;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+
+  const bf16* wt = Wp + ((size_t)tile * k_steps * 64 + lane) * 8;
+  uint4 w[QR_KSTEPS];
+#pragma unroll
+  for (int s = 0; s < QR_KSTEPS; ++s) {
+    const int st = step0 + s;
+    w[s] = load16_stream(wt + (size_t)(st < k_steps ? st : k_steps - 1) * 512);   // the weights: read once
+  }
+  uint4 a[MT][QR_KSTEPS];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + row;
+    const bf16* ap = A + (size_t)(m < M ? m : M - 1) * lda;   // rows >= M read a real row and are zeroed
+#pragma unroll
+    for (int s = 0; s < QR_KSTEPS; ++s) {
+      const int k = (step0 + s) * 32 + kg * 8;
+      const uint4 v = *reinterpret_cast<const uint4*>(ap + (k < K ? k : K - 8));
+      a[mt][s] = (m < M && k < K) ? v : zero;
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < QR_KSTEPS; ++s)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[mt][s]),
+                                                        __builtin_bit_cast(bf16x8_t, w[s]), acc[mt], 0, 0, 0);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[(wave * MT + mt) * 256 + r * 64 + lane] = acc[mt][r];
+  __syncthreads();
+
+  // epilogue: one thread per (token row m, column c of the tile)
+  for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
+    const int mt = idx >> 8, i = idx & 255;
+    const int r = i >> 6, l2 = i & 63, c = l2 & 15;
+    const int m = mt * 16 + (l2 >> 4) * 4 + r;
+    if (m >= M) continue;
+    float x = 0.f, partner = 0.f;   // column c and its neighbour c ^ 1
+    for (int k2 = 0; k2 < n_waves; ++k2) {
+      x += red[(k2 * MT + mt) * 256 + i];
+      partner += red[(k2 * MT + mt) * 256 + (i ^ 1)];
+    }
+    const int b = token_seq[m];
+    const int pos = positions[m];
+    const int d = col0 + c;
+    float y = x;     // value heads are stored as they are
+    if (head < nh + nkv) {
+      const float2 cs = cos_sin[(size_t)pos * (hd / 2) + (d >> 1)];
+      y = (c & 1) == 0 ? x * cs.x - partner * cs.y : partner * cs.y + x * cs.x;
+    }
+    const bf16 o = from_float<bf16>(y);
+    if (head < nh) {
+      qkv_out[(size_t)m * ldq + (size_t)head * hd + d] = o;
+    } else if (b >= 0) {
+      const int page = block_table[(size_t)b * table_width + pos / page_size];
+      const int slot = pos % page_size;
+      if (page < 0) continue;
+      if (head < nh + nkv) kcache[(((size_t)page * nkv + (head - nh)) * page_size + slot) * hd + d] = o;
+      else vcache[((size_t)page * nkv + (head - nh - nkv)) * hd * page_size + (size_t)d * page_size + slot] = o;
+    }
+  }
+}
+
+// Up to 16 rows: pairing 0 takes every head size that is a multiple of 16; pairing 1 (partners half a
+// head apart, two tiles per block) needs a multiple of 32; K up to 4096.  17 to 64 rows: adjacent
+// pairs only; K up to 4096 for at most 32 rows and up to 2048 beyond (the activations' registers).
 extern "C" int blm_gemv_qkv_rope_supported(int M, int K, int hd, int pairing) {
   const int step = pairing == 0 ? 16 : 32;
-  return (M >= 1 && M <= 16 && K >= 8 && K % 8 == 0 && K <= 4096 && hd >= step && hd % step == 0 &&
-          (pairing == 0 || pairing == 1)) ? 1 : 0;
+  if (!(M >= 1 && M <= 64 && K >= 8 && K % 8 == 0 && hd >= step && hd % step == 0 && (pairing == 0 || pairing == 1)))
+    return 0;
+  if (M <= 16) return K <= 4096 ? 1 : 0;
+  if (pairing != 0) return 0;
+  return K <= (M <= 32 ? 4096 : 2048) ? 1 : 0;
 }
 
 // Wp: pack_weight of W_qkv [(nh + 2 nkv) * hd, K].  qkv_out: [M, ldq] bf16; only its first nh*hd
@@ -215,13 +308,32 @@ extern "C" int blm_gemv_qkv_rope(const void* A, const void* Wp, void* qkv_out, c
                                  int lda, int ldq, int nh, int nkv, int hd, int pairing, int store,
                                  hipStream_t stream) {
   BLM_REQUIRE(blm_gemv_qkv_rope_supported(M, K, hd, pairing), "gemv_qkv_rope: M=%d K=%d head_dim=%d pairing=%d not "
-              "supported (M <= 16, K a multiple of 8 and at most 4096, head_dim a multiple of 16 for adjacent "
-              "pairs and of 32 for pairs half a head apart)", M, K, hd, pairing);
+              "supported (K a multiple of 8 and at most 4096, head_dim a multiple of 16 for adjacent pairs and of "
+              "32 for pairs half a head apart; 17 to 64 rows: adjacent pairs, K at most 2048 above 32 rows)",
+              M, K, hd, pairing);
   BLM_REQUIRE(nh > 0 && nkv > 0 && page_size > 0 && table_width > 0, "gemv_qkv_rope: bad geometry");
   BLM_REQUIRE(lda % 8 == 0 && lda >= K && ldq >= nh * hd, "gemv_qkv_rope: bad strides lda=%d ldq=%d", lda, ldq);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0, "gemv_qkv_rope: operands must be 16-byte aligned");
   const int k_steps = (K + 31) / 32;
   const int tiles = (nh + 2 * nkv) * (hd / 16);
+  if (M > 16) {
+    const int mt = (M + 15) / 16;
+    const int ks = k_steps > 64 ? 16 : 8;            // more than 2048 of K: two row tiles at most
+    const int waves = (k_steps + ks - 1) / ks;       // at most 8
+    const size_t smem = (size_t)waves * mt * 256 * sizeof(float);
+#define BLM_QRR(MT, KS)                                                                                            \
+  hipLaunchKernelGGL((gemv_qkv_rope_rows_kernel<MT, KS>), dim3(tiles), dim3(waves * BLM_WAVE), smem, stream,       \
+                     (const bf16*)A, (const bf16*)Wp, (bf16*)qkv_out, positions, token_seq, block_table,           \
+                     table_width, (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache, page_size, M, K, lda, ldq, \
+                     k_steps, nh, nkv, hd, store)
+    if (ks == 16) BLM_QRR(2, 16);
+    else if (mt == 2) BLM_QRR(2, 8);
+    else if (mt == 3) BLM_QRR(3, 8);
+    else BLM_QRR(4, 8);
+#undef BLM_QRR
+    BLM_LAUNCH_CHECK("gemv_qkv_rope_rows");
+    return 0;
+  }
   // Adjacent pairs: one tile per block while that is one round of blocks on the chip's 256 compute
   // units (or the head size leaves no choice, or K is so wide that two-tile blocks would need 16
   // wavefronts and spill); beyond that, blocks of two tiles (measured at 320 tiles, K = 3072: one

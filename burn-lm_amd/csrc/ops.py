@@ -414,13 +414,15 @@ def gemv_mfma(a, packed, out, K, gated=False):
 
 
 def gemv_qkv_rope_supported(M, K, hd, pairing):
-    """pairing 0 (adjacent lanes): head_dim a multiple of 16; pairing 1 (half a head apart): of 32."""
+    """Up to 16 rows: pairing 0 (adjacent lanes) with head_dim a multiple of 16, pairing 1 (half a head
+    apart) with a multiple of 32, K up to 4096.  17 to 64 rows: pairing 0; K up to 4096 for at most 32
+    rows, up to 2048 beyond."""
     return bool(library().blm_gemv_qkv_rope_supported(int(M), int(K), int(hd), int(pairing)))
 
 
 def gemv_qkv_rope(x, packed, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,
                   nh, nkv, hd, pairing, write_kv=True):
-    """Decode: x [M<=16, K] @ W_qkv^T on the matrix cores, rotary encoding of q and k on the float
+    """Decode: x [M<=64, K] @ W_qkv^T on the matrix cores, rotary encoding of q and k on the float
     results, q into qkv_out[:, :nh*hd], k and v into their cache pages, all in one kernel.
     packed: pack_weight of W_qkv [(nh + 2 nkv) * hd, K]."""
     _gpu(x, packed, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache)

@@ -584,7 +584,9 @@ def test_sample_large_vocabulary_matches_the_ordered_nucleus(ops, V, ld):
 @pytest.mark.parametrize("pairing", ["interleaved", "half"])
 @pytest.mark.parametrize("M,K,nh,nkv,hd", [(8, 2048, 4, 2, 64), (5, 264, 3, 1, 32), (16, 3072, 2, 2, 128), (1, 64, 6, 3, 64),
                                            (4, 4096, 2, 1, 64), (9, 3608, 3, 1, 32), (7, 2056, 2, 2, 32),
-                                           (6, 520, 3, 1, 48), (16, 2048, 2, 1, 80), (8, 264, 30, 2, 128)])
+                                           (6, 520, 3, 1, 48), (16, 2048, 2, 1, 80), (8, 264, 30, 2, 128),
+                                           (33, 2048, 4, 2, 64), (64, 520, 3, 1, 48), (20, 4096, 2, 1, 64), (17, 264, 30, 2, 128),
+                                           (48, 2056, 2, 1, 32)])
 def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     """The fused decode projection: equals the product, the rotation of its float result and the
     cache write done one after the other (in float64), for both pairings, with a padding row and
@@ -592,11 +594,13 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     from burn_lm_amd.parts.rope import PAIRING, rope_frequencies
     # adjacent pairs sit in one 16-column tile: any head size in steps of 16; pairs half a head apart
     # need two whole tiles per half: steps of 32
-    assert ops.gemv_qkv_rope_supported(M, K, hd, PAIRING[pairing]) == (pairing == "interleaved" or hd % 32 == 0)
-    if not ops.gemv_qkv_rope_supported(M, K, hd, PAIRING[pairing]):
+    # and from 17 rows on only adjacent pairs, with K up to 4096 for 32 rows and up to 2048 beyond
+    takes = (pairing == "interleaved" or hd % 32 == 0) if M <= 16 else (pairing == "interleaved" and K <= (4096 if M <= 32 else 2048))
+    assert ops.gemv_qkv_rope_supported(M, K, hd, PAIRING[pairing]) == takes
+    if not takes:
         return
     g = torch.Generator().manual_seed(19)
-    page, n_pages = 64, 16
+    page, n_pages = 64, (16 if M <= 16 else 64)       # four pages for every sequence
     N = (nh + 2 * nkv) * hd
     x = torch.randn(M, K, generator=g).bfloat16()
     W = (torch.randn(N, K, generator=g) / K ** 0.5).bfloat16()
