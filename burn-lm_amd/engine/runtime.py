@@ -8,9 +8,16 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
   streams the weight once (where the width fits its registers: see ops.gemv_mfma_group_limit).
 * bfloat16 weights, many rows (prefill): the library product (hipBLASLt through torch), as the
   reference's engine leaves its matrix products to its tensor library
-  (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).
+  (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).  With BURN_LM_AMD_FUSED_GATE_UP=1 the
+  gate/up product of a gated feed-forward runs instead on the hand-written matrix-core kernel that
+  applies the gating in its epilogue (ops.gemm_mfma): it never writes the [rows, 2 I] intermediate
+  nor reads it back, but its lower rate eats that gain (measured over whole prefills: 3-5 % faster
+  at 256-1,024 rows of the 1B shape, even at 2,048, 5-10 % slower at the 8B shape), so it is off
+  unless asked for.
 """
 from __future__ import annotations
+
+import os
 
 import torch
 
@@ -18,6 +25,9 @@ from ..csrc import ops
 
 SKINNY_MAX_ROWS = 8
 MFMA_SKINNY_MAX_ROWS = 64
+# Rows for which the fused gate/up product is used when it is switched on (below, the library is
+# ahead by far; above, its better rate on long runs of tiles has made up for the extra pass).
+FUSED_GATE_UP_ROWS = (192, 4096)
 
 
 class LinearWeight:
@@ -42,6 +52,8 @@ class Runtime:
         self.ops = ops
         ops.library()  # fail now, loudly, if the kernel library cannot be had
         ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
+        ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
+        self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if os.environ.get("BURN_LM_AMD_FUSED_GATE_UP") == "1" else (0, -1)
 
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
@@ -131,7 +143,14 @@ class Runtime:
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
             return ops.gemv_mfma(x, w.packed, out, K, gated=True)
-        gu = self.linear(x, w.w if isinstance(w, LinearWeight) else w)
+        plain = w.w if isinstance(w, LinearWeight) else w
+        if (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]
+                and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+                and plain.is_contiguous()):
+            # the largest tile that still gives every compute unit a block (a 256x256 tile holds 128 gated pairs)
+            tile = (256, 256) if -(-M // 256) * -(-inner // 128) >= 256 else (128, 128)
+            return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True, tile=tile)
+        gu = self.linear(x, plain)
         act = torch.empty(M, inner, dtype=gu.dtype, device=x.device)
         ops.swiglu(gu, act)
         return act

@@ -495,6 +495,66 @@ def test_gemv_mfma_refuses_what_it_cannot_do(ops):
         ops.gemv_mfma(dev(torch.zeros(4, 64).bfloat16()), wp, torch.zeros(4, 40, dtype=torch.bfloat16, device="cuda"), 64)
 
 
+@pytest.mark.parametrize("tile", [(128, 128), (256, 128), (256, 256)])
+@pytest.mark.parametrize("M,N,K,groups,out_dtype", [(200, 136, 72, 1, "float32"), (300, 264, 200, 1, "bfloat16"),
+                                                    (513, 520, 1096, 2, "float32"), (65, 31, 8, 1, "bfloat16"),
+                                                    (129, 1000, 2048, 1, "bfloat16"), (260, 100, 4104, 4, "float32")])
+def test_gemm_mfma(ops, tile, M, N, K, groups, out_dtype):
+    """Matrix-core product for many rows: every tile shape; tails in M, N and K (a last stage that is
+    no whole one, fewer stages than the ring holds), K cut into groups whose planes the reader sums,
+    an output with a row stride and rows of a wider buffer."""
+    g = torch.Generator().manual_seed(21)
+    wide = torch.randn(M, K + 16, generator=g).bfloat16()
+    W = torch.randn(N, K, generator=g).bfloat16()
+    W[N // 2, K - 8:] = 40.0      # one term dominates a column: a wrong operand layout cannot hide in the noise
+    A = wide[:, 8:K + 8]
+    want = A.double() @ W.double().T
+    if groups > 1:
+        out = torch.full((groups, M, N), 7.0, dtype=torch.float32, device="cuda")
+        ops.gemm_mfma(dev(wide)[:, 8:K + 8], dev(W), out, tile=tile)
+        got = out.double().sum(0).cpu()
+    else:
+        big = torch.zeros(M, N + 8, dtype=DT[out_dtype], device="cuda")
+        ops.gemm_mfma(dev(wide)[:, 8:K + 8], dev(W), big[:, :N], tile=tile)
+        assert bool((big[:, N:] == 0).all())
+        got = big[:, :N].double().cpu()
+    err = ((got - want).abs() / (want.abs() + want.abs().mean())).max()
+    assert float(err) <= (2e-5 if out_dtype == "float32" else 8e-3), f"error {float(err):.3g}"
+
+
+@pytest.mark.parametrize("tile", [(128, 128), (256, 128), (256, 256)])
+@pytest.mark.parametrize("M,I,K", [(70, 176, 64), (300, 264, 200), (257, 1000, 2048), (128, 8, 520)])
+def test_gemm_mfma_gated(ops, tile, M, I, K):
+    """The SwiGLU gating in the epilogue: a block takes gate columns and the matching up columns of
+    the matrix as the checkpoint stores it ([gate rows; up rows])."""
+    g = torch.Generator().manual_seed(22)
+    A = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(2 * I, K, generator=g) * (2.0 / K ** 0.5)).bfloat16()
+    out = torch.full((M, I), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_mfma(dev(A), dev(W), out, gated=True, tile=tile)
+    gate, up = A.double() @ W[:I].double().T, A.double() @ W[I:].double().T
+    want = torch.nn.functional.silu(gate) * up
+    close(out, want, EPS["bfloat16"] * 1.5)
+    assert float((torch.nn.functional.silu(up) * gate - want).abs().max() / want.abs().max()) > 0.1
+
+
+def test_gemm_mfma_refuses_what_it_cannot_do(ops):
+    from burn_lm_amd.csrc.ops import KernelError
+    a, w = dev(torch.zeros(80, 64).bfloat16()), dev(torch.zeros(48, 64).bfloat16())
+    with pytest.raises(KernelError, match="tile"):
+        ops.gemm_mfma(a, w, torch.zeros(80, 48, dtype=torch.bfloat16, device="cuda"), tile=(64, 64))
+    with pytest.raises(KernelError, match="do not fit"):
+        ops.gemm_mfma(a, w, torch.zeros(80, 40, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(KernelError, match="bfloat16"):
+        ops.gemm_mfma(a.float(), w, torch.zeros(80, 48, dtype=torch.float32, device="cuda"))
+    with pytest.raises(KernelError, match="float32"):
+        ops.gemm_mfma(a, w, torch.zeros(2, 80, 48, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(KernelError, match="K a multiple of 8"):
+        ops.gemm_mfma(a[:, :60], w[:, :60], torch.zeros(80, 48, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(KernelError, match="one K group"):
+        ops.gemm_mfma(a, w, torch.zeros(2, 80, 24, dtype=torch.float32, device="cuda"), gated=True)
+
+
 def test_argmax_first_maximum_wins(ops):
     g = torch.Generator().manual_seed(7)
     x = torch.randn(6, 1000, generator=g)

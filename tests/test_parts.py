@@ -139,6 +139,15 @@ def test_swiglu_part(rt):
     # swapping gate and up must show: silu is on the gate
     wrong = P.swiglu_feed_forward(x.double().numpy(), tn["u"], tn["g"], tn["d"])
     assert np.abs(wrong - want).max() / np.abs(want).max() > 0.1
+    if rt.dtype == torch.bfloat16:
+        # many rows with the gating fused into the matrix-core product (off unless asked for)
+        rt.fused_gate_up_rows = (65, 4096)
+        try:
+            x = (torch.randn(300, 72, generator=torch.Generator().manual_seed(6))).to(rt.dtype)
+            want = P.swiglu_feed_forward(x.double().numpy(), tn["g"], tn["u"], tn["d"])
+            assert rel(ffn.forward(x.to("cuda"), None), want) <= TOL[rt.dtype]
+        finally:
+            rt.fused_gate_up_rows = (0, -1)
 
 
 def test_embedding_and_head_parts(rt):
