@@ -1,13 +1,13 @@
 // Matrix product for many rows (prefill) on the matrix cores: C[M, N] = A[M, K] * W[N, K]^T, bf16
 // operands, float accumulation, bf16 or float output.
 //
-// A block of four wavefronts owns a BM x BN tile of C and walks K in stages of BK.  Both operands
+// A block of four or eight wavefronts owns a BM x BN tile of C and walks K in stages of BK.  Both operands
 // are rows of consecutive k (the weight matrix is used as the checkpoint stores it), so their
 // tiles are staged the same way: 16 bytes per lane from global memory straight into a ring of NS
 // shared-memory buffers (no registers in between), NS - 1 stages ahead of the multiplications: a
-// load takes longer than a stage's multiplications, and one wavefront per SIMD has nothing else to
-// hide it behind.  The pieces of a staged row are permuted so that a fragment read meets every
-// bank once.  A wavefront owns a quarter of the tile as 32x32 accumulators of the 32x32x16
+// load takes longer than a stage's multiplications, and one or two wavefronts per SIMD have little
+// else to hide it behind.  The pieces of a staged row are permuted so that a fragment read meets every
+// bank once.  A wavefront owns its part of the tile as 32x32 accumulators of the 32x32x16
 // instruction; per k-step of 16 it reads one fragment per 32 rows and per 32 columns and
 // multiplies every pair.
 //
@@ -23,7 +23,6 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
-constexpr int GM_THREADS = 256;
 
 // 16 zero bytes for the pieces that lie beyond the end of K
 __device__ __align__(16) const uint32_t gm_zero_piece[4] = {0u, 0u, 0u, 0u};
@@ -46,18 +45,25 @@ __device__ __forceinline__ float gm_silu(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
-template <int BM, int BN, int BK, int NS, int MODE, typename TC>
-__global__ void __launch_bounds__(GM_THREADS)
+// columns per pass of the epilogue: as many of a wavefront's `on` as the staging of all `waves` leaves room for
+constexpr int gm_pass_columns(int on, int waves, size_t bytes) {
+  int cw = on;
+  while (cw >= 32 && (size_t)waves * 32 * (cw + 4) * sizeof(float) > bytes) cw /= 2;
+  return cw;
+}
+
+template <int BM, int BN, int BK, int NS, int WGM, int WGN, int MODE, typename TC>
+__global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
     gemm_mfma_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
                      int lda, int ldw, int ldc, int m_tiles, int n_tiles, int k_per_group) {
-  constexpr int WGM = 2, WGN = 2;                 // wavefronts along M and N
+  constexpr int NW = WGM * WGN;                   // wavefronts, WGM along M and WGN along N
   constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
   static_assert(WM % 32 == 0 && WN % 32 == 0 && (MODE == 0 || TN % 2 == 0), "wavefront tile");
   static_assert(BK == 32 || BK == 64, "stage depth");
   constexpr int P = BK / 8;                       // 16-byte pieces per staged row
   constexpr int RPL = 64 / P;                     // rows that one load instruction of a wavefront fills
   constexpr int RPB = 256 / (BK * 2);             // staged rows per 256 bytes (one pass over the banks)
-  constexpr int A_LD = BM / RPL / 4, B_LD = BN / RPL / 4;   // loads per wavefront and stage
+  constexpr int A_LD = BM / RPL / NW, B_LD = BN / RPL / NW;   // loads per wavefront and stage
   constexpr int LOADS = A_LD + B_LD;
   static_assert(A_LD >= 1 && B_LD >= 1 && (NS - 1) * LOADS <= 63 && NS >= 2, "staging");
   constexpr int QN = BK / 16;                     // k-steps of the matrix instruction per stage
@@ -259,69 +265,75 @@ __global__ void __launch_bounds__(GM_THREADS)
   for (; s < n_steady; ++s, buf = buf + 1 == NS ? 0 : buf + 1) iteration(s, buf, std::true_type{});
   for (; s < n_stages; ++s, buf = buf + 1 == NS ? 0 : buf + 1) iteration(s, buf, std::false_type{});
 
-  // Results leave through shared memory, 32 rows at a time per wavefront, so that every store
-  // writes 16 bytes per lane and whole lines per row.
+  // Results leave through shared memory, 32 rows and CW columns at a time per wavefront, so that
+  // every store writes 16 bytes per lane and runs of whole lines per row.
   __syncthreads();
   constexpr int ON = MODE == 1 ? WN / 2 : WN;           // output columns of a wavefront
-  constexpr int OSTR = ON + 4;                          // floats per staged row
+  constexpr int CW = gm_pass_columns(ON, NW, (size_t)NS * (BM + BN) * BK * sizeof(bf16));
+  static_assert(CW >= 32, "output staging fits");
+  constexpr int OSTR = CW + 4;                          // floats per staged row
   float* stage_out = reinterpret_cast<float*>(gm_smem) + wave * 32 * OSTR;
-  static_assert(4 * 32 * OSTR * sizeof(float) <= (size_t)NS * (BM + BN) * BK * sizeof(bf16), "output staging fits");
   constexpr int PER = sizeof(TC) == 2 ? 8 : 4;          // elements per 16-byte store
   const int out_n0 = n0 + wn * ON;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int j = 0; j < (MODE == 1 ? TN / 2 : TN); ++j)
+    for (int c0 = 0; c0 < ON; c0 += CW) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float4 v;
-        if (MODE == 1) {
-          float4 gt = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-          float4 up = make_float4(acc[i][j + TN / 2][4 * g], acc[i][j + TN / 2][4 * g + 1], acc[i][j + TN / 2][4 * g + 2],
-                                  acc[i][j + TN / 2][4 * g + 3]);
-          v = make_float4(gm_silu(gt.x) * up.x, gm_silu(gt.y) * up.y, gm_silu(gt.z) * up.z, gm_silu(gt.w) * up.w);
-        } else {
-          v = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-        }
-        *reinterpret_cast<float4*>(stage_out + l32 * OSTR + j * 32 + 8 * g + 4 * lh) = v;
-      }
-    // the wavefront reads back what it wrote itself: no barrier, the compiler orders the accesses
-    const int m_base = m0 + wm * WM + i * 32;
-    constexpr int LANES_PER_ROW = ON / PER;
+      for (int jj = 0; jj < CW / 32; ++jj) {
+        const int j = c0 / 32 + jj;
 #pragma unroll
-    for (int x = 0; x < 32 * LANES_PER_ROW / BLM_WAVE; ++x) {
-      const int idx = x * BLM_WAVE + lane;
-      const int r = idx / LANES_PER_ROW, c = (idx % LANES_PER_ROW) * PER;
-      const int m = m_base + r, n = out_n0 + c;
-      const float* src = stage_out + r * OSTR + c;
-      if (m < M && n < N) {
-        TC* dst = C + (size_t)m * ldc + n;
-        const bool vec = n + PER <= N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
-        const float4 lo = *reinterpret_cast<const float4*>(src);
-        if (sizeof(TC) == 2) {
-          const float4 hi = *reinterpret_cast<const float4*>(src + 4);
-          if (vec) {
-            *reinterpret_cast<uint4*>(dst) = make_uint4(f32x2_to_bf16x2_bits(lo.x, lo.y), f32x2_to_bf16x2_bits(lo.z, lo.w),
-                                                        f32x2_to_bf16x2_bits(hi.x, hi.y), f32x2_to_bf16x2_bits(hi.z, hi.w));
+        for (int g = 0; g < 4; ++g) {
+          float4 v;
+          if (MODE == 1) {
+            float4 gt = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+            float4 up = make_float4(acc[i][j + TN / 2][4 * g], acc[i][j + TN / 2][4 * g + 1],
+                                    acc[i][j + TN / 2][4 * g + 2], acc[i][j + TN / 2][4 * g + 3]);
+            v = make_float4(gm_silu(gt.x) * up.x, gm_silu(gt.y) * up.y, gm_silu(gt.z) * up.z, gm_silu(gt.w) * up.w);
           } else {
-            // a row end that is no multiple of 8, or a row that starts off a 16-byte boundary
-            dst[0] = from_float<TC>(lo.x);
-            if (n + 1 < N) dst[1] = from_float<TC>(lo.y);
-            if (n + 2 < N) dst[2] = from_float<TC>(lo.z);
-            if (n + 3 < N) dst[3] = from_float<TC>(lo.w);
-            if (n + 4 < N) dst[4] = from_float<TC>(hi.x);
-            if (n + 5 < N) dst[5] = from_float<TC>(hi.y);
-            if (n + 6 < N) dst[6] = from_float<TC>(hi.z);
-            if (n + 7 < N) dst[7] = from_float<TC>(hi.w);
+            v = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
           }
-        } else {
-          if (vec) {
-            *reinterpret_cast<float4*>(dst) = lo;
+          *reinterpret_cast<float4*>(stage_out + l32 * OSTR + jj * 32 + 8 * g + 4 * lh) = v;
+        }
+      }
+      // the wavefront reads back what it wrote itself: no barrier, the compiler orders the accesses
+      const int m_base = m0 + wm * WM + i * 32;
+      constexpr int LANES_PER_ROW = CW / PER;
+#pragma unroll
+      for (int x = 0; x < 32 * LANES_PER_ROW / BLM_WAVE; ++x) {
+        const int idx = x * BLM_WAVE + lane;
+        const int r = idx / LANES_PER_ROW, c = (idx % LANES_PER_ROW) * PER;
+        const int m = m_base + r, n = out_n0 + c0 + c;
+        const float* src = stage_out + r * OSTR + c;
+        if (m < M && n < N) {
+          TC* dst = C + (size_t)m * ldc + n;
+          const bool vec = n + PER <= N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+          const float4 lo = *reinterpret_cast<const float4*>(src);
+          if (sizeof(TC) == 2) {
+            const float4 hi = *reinterpret_cast<const float4*>(src + 4);
+            if (vec) {
+              *reinterpret_cast<uint4*>(dst) = make_uint4(f32x2_to_bf16x2_bits(lo.x, lo.y), f32x2_to_bf16x2_bits(lo.z, lo.w),
+                                                          f32x2_to_bf16x2_bits(hi.x, hi.y), f32x2_to_bf16x2_bits(hi.z, hi.w));
+            } else {
+              // a row end that is no multiple of 8, or a row that starts off a 16-byte boundary
+              dst[0] = from_float<TC>(lo.x);
+              if (n + 1 < N) dst[1] = from_float<TC>(lo.y);
+              if (n + 2 < N) dst[2] = from_float<TC>(lo.z);
+              if (n + 3 < N) dst[3] = from_float<TC>(lo.w);
+              if (n + 4 < N) dst[4] = from_float<TC>(hi.x);
+              if (n + 5 < N) dst[5] = from_float<TC>(hi.y);
+              if (n + 6 < N) dst[6] = from_float<TC>(hi.z);
+              if (n + 7 < N) dst[7] = from_float<TC>(hi.w);
+            }
           } else {
-            dst[0] = from_float<TC>(lo.x);
-            if (n + 1 < N) dst[1] = from_float<TC>(lo.y);
-            if (n + 2 < N) dst[2] = from_float<TC>(lo.z);
-            if (n + 3 < N) dst[3] = from_float<TC>(lo.w);
+            if (vec) {
+              *reinterpret_cast<float4*>(dst) = lo;
+            } else {
+              dst[0] = from_float<TC>(lo.x);
+              if (n + 1 < N) dst[1] = from_float<TC>(lo.y);
+              if (n + 2 < N) dst[2] = from_float<TC>(lo.z);
+              if (n + 3 < N) dst[3] = from_float<TC>(lo.w);
+            }
           }
         }
       }
@@ -329,46 +341,49 @@ __global__ void __launch_bounds__(GM_THREADS)
   }
 }
 
-template <int BM, int BN, int BK, int NS, int MODE, typename TC>
+template <int BM, int BN, int BK, int NS, int WGM, int WGN, int MODE, typename TC>
 static int prepare_gemm() {
   constexpr size_t smem = (size_t)NS * (BM + BN) * BK * sizeof(bf16);
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_kernel<BM, BN, BK, NS, MODE, TC>),
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_kernel<BM, BN, BK, NS, WGM, WGN, MODE, TC>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
     return blm_fail("gemm_mfma: %zu bytes of shared memory refused", smem);
   return 0;
 }
 
-template <int BM, int BN, int BK, int NS, int MODE, typename TC>
+template <int BM, int BN, int BK, int NS, int WGM, int WGN, int MODE, typename TC>
 static int launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                        int k_groups, hipStream_t stream) {
   constexpr size_t smem = (size_t)NS * (BM + BN) * BK * sizeof(bf16);
   const int m_tiles = (M + BM - 1) / BM;
   const int n_tiles = (N + (MODE == 1 ? BN / 2 : BN) - 1) / (MODE == 1 ? BN / 2 : BN);
   const int k_per_group = ((K + k_groups - 1) / k_groups + BK - 1) / BK * BK;
-  dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)k_groups), block(GM_THREADS);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, BK, NS, MODE, TC>), grid, block, smem, stream, (const bf16*)A,
+  dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)k_groups), block(WGM * WGN * BLM_WAVE);
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, BK, NS, WGM, WGN, MODE, TC>), grid, block, smem, stream, (const bf16*)A,
                      (const bf16*)W, (TC*)C, M, N, K, lda, ldw, ldc, m_tiles, n_tiles, k_per_group);
   BLM_LAUNCH_CHECK("gemm_mfma");
   return 0;
 }
 
-#define BLM_GEMM_TILES(X) X(128, 128, 64, 2) X(256, 128, 64, 3) X(256, 256, 64, 2)
+#define BLM_GEMM_TILES(X) X(128, 128, 64, 2, 2, 2) X(256, 128, 64, 3, 4, 2) X(256, 256, 64, 2, 2, 4)
 
 // Lets every variant use more than 64 KiB of shared memory; to be called once per device before the
 // first product (not from inside a stream capture).
 extern "C" int blm_gemm_mfma_init() {
-#define BLM_PREP(BM, BN, BK, NS)                                                                     \
-  if (prepare_gemm<BM, BN, BK, NS, 0, bf16>() || prepare_gemm<BM, BN, BK, NS, 0, float>() ||         \
-      prepare_gemm<BM, BN, BK, NS, 1, bf16>() || prepare_gemm<BM, BN, BK, NS, 1, float>())           \
+#define BLM_PREP(BM, BN, BK, NS, WGM, WGN)                                                                     \
+  if (prepare_gemm<BM, BN, BK, NS, WGM, WGN, 0, bf16>() || prepare_gemm<BM, BN, BK, NS, WGM, WGN, 0, float>() ||       \
+      prepare_gemm<BM, BN, BK, NS, WGM, WGN, 1, bf16>() || prepare_gemm<BM, BN, BK, NS, WGM, WGN, 1, float>())         \
     return 1;
   BLM_GEMM_TILES(BLM_PREP)
 #undef BLM_PREP
   return 0;
 }
 
-// tile: rows x columns of C per block: 0 = 128x128, 1 = 256x128, 2 = 256x256 (measured at 2,048 rows:
-// the largest tile that still gives every compute unit a block is the fastest; K in stages of 64,
-// two of them in shared memory, three for 256x128; stages of 32 and deeper rings were not faster)
+// tile: rows x columns of C per block: 0 = 128x128 (four wavefronts, several blocks per compute unit),
+// 1 = 256x128 and 2 = 256x256 (eight wavefronts: two per SIMD, so that one issues matrix instructions
+// while the other issues loads or waits; 10 % faster than four wavefronts with twice the tile each,
+// sixteen are no faster).  K in stages of 64, two of them in shared memory, three for 256x128;
+// stages of 32 in deeper rings were not faster.  Measured at 256 to 4,096 rows: the largest tile
+// that still gives every compute unit a block is the fastest.
 // mode 0: C[M, N] = A W^T, W [N, K].  mode 1: W [2N, K] = [gate rows; up rows], C[M, N] = silu(gate) * up.
 extern "C" int blm_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda,
                              int ldw, int ldc, int mode, int k_groups, int tile, hipStream_t stream) {
@@ -384,19 +399,20 @@ extern "C" int blm_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   // per-lane byte offsets into a tile's rows are 32-bit
   BLM_REQUIRE((size_t)256 * lda * 2 < ((size_t)1 << 32) && (size_t)(mode == 1 ? 2 : 1) * N * ldw * 2 < ((size_t)1 << 32),
               "gemm_mfma: matrices of 4 GiB and more are not supported (lda=%d, N=%d, ldw=%d)", lda, N, ldw);
-#define BLM_GEMM(BM, BN, BK, NS)                                                                                     \
+#define BLM_GEMM(BM, BN, BK, NS, WGM, WGN)                                                                           \
   do {                                                                                                               \
     if (mode == 1)                                                                                                   \
       return c_dtype == BLM_BF16                                                                                     \
-                 ? launch_gemm<BM, BN, BK, NS, 1, bf16>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream)           \
-                 : launch_gemm<BM, BN, BK, NS, 1, float>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream);         \
-    return c_dtype == BLM_BF16 ? launch_gemm<BM, BN, BK, NS, 0, bf16>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream) \
-                               : launch_gemm<BM, BN, BK, NS, 0, float>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream); \
+                 ? launch_gemm<BM, BN, BK, NS, WGM, WGN, 1, bf16>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream) \
+                 : launch_gemm<BM, BN, BK, NS, WGM, WGN, 1, float>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream); \
+    return c_dtype == BLM_BF16                                                                                       \
+               ? launch_gemm<BM, BN, BK, NS, WGM, WGN, 0, bf16>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream)   \
+               : launch_gemm<BM, BN, BK, NS, WGM, WGN, 0, float>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream); \
   } while (0)
   switch (tile) {
-    case 0: BLM_GEMM(128, 128, 64, 2);
-    case 1: BLM_GEMM(256, 128, 64, 3);
-    case 2: BLM_GEMM(256, 256, 64, 2);
+    case 0: BLM_GEMM(128, 128, 64, 2, 2, 2);
+    case 1: BLM_GEMM(256, 128, 64, 3, 4, 2);
+    case 2: BLM_GEMM(256, 256, 64, 2, 2, 4);
   }
 #undef BLM_GEMM
   return blm_fail("gemm_mfma: tile %d out of range 0..2", tile);

@@ -11,9 +11,8 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
   (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).  With BURN_LM_AMD_FUSED_GATE_UP=1 the
   gate/up product of a gated feed-forward runs instead on the hand-written matrix-core kernel that
   applies the gating in its epilogue (ops.gemm_mfma): it never writes the [rows, 2 I] intermediate
-  nor reads it back, but its lower rate eats that gain (measured over whole prefills: 3-5 % faster
-  at 256-1,024 rows of the 1B shape, even at 2,048, 5-10 % slower at the 8B shape), so it is off
-  unless asked for.
+  nor reads it back, but its lower rate eats that gain at wider shapes (measured over whole
+  prefills: 1-6 % faster at the 1B shape, even at 3B, 2-7 % slower at 8B), so it is off unless asked for.
 """
 from __future__ import annotations
 
@@ -147,8 +146,10 @@ class Runtime:
         if (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]
                 and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
                 and plain.is_contiguous()):
-            # the largest tile that still gives every compute unit a block (a 256x256 tile holds 128 gated pairs)
-            tile = (256, 256) if -(-M // 256) * -(-inner // 128) >= 256 else (128, 128)
+            # the largest tile that still gives every compute unit a block (a tile of n columns holds n / 2 gated pairs)
+            m256 = -(-M // 256)
+            tile = ((256, 256) if m256 * -(-inner // 128) >= 256 else
+                    (256, 128) if m256 * -(-inner // 64) >= 256 else (128, 128))
             return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True, tile=tile)
         gu = self.linear(x, plain)
         act = torch.empty(M, inner, dtype=gu.dtype, device=x.device)
