@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 _lib = None
 _lock = threading.Lock()
 
@@ -55,7 +55,8 @@ _SIGNATURES = {
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
-    "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
+    "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p, _c_void_p,
+                   _c_void_p],
 }
 
 
@@ -75,6 +76,8 @@ def library():
                     fn = getattr(lib, name)
                     fn.argtypes = sig
                     fn.restype = _c_int
+                lib.blm_sample_scratch_bytes.argtypes = [_c_int, _c_int]
+                lib.blm_sample_scratch_bytes.restype = ctypes.c_longlong
                 _lib = lib
     return _lib
 
@@ -511,8 +514,11 @@ def argmax(logits, out=None):
 
 
 def sample(logits, uniforms, temperature, top_p=1.0, out=None):
-    """Pick from softmax(logits / temperature) cut to the top-p nucleus at the given uniforms."""
-    _gpu(logits, uniforms, out)
+    """Pick from softmax(logits / temperature) cut to the top-p nucleus at the given uniforms (on the
+    GPU, or in pinned host memory, which the kernel reads in place)."""
+    _gpu(logits, out)
+    if not (uniforms.is_cuda or uniforms.is_pinned()):
+        raise KernelError("sample: uniforms must be on the GPU or in pinned host memory")
     R, V = logits.shape
     if logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise KernelError("sample: logits must be float32 with unit stride along the vocabulary")
@@ -521,6 +527,11 @@ def sample(logits, uniforms, temperature, top_p=1.0, out=None):
     if out is None:
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
     _i32("out", out, R)
+    counters = arrival_counters(logits.device)
+    if R > counters.numel():
+        raise KernelError(f"sample: {R} rows are more than the {counters.numel()} counters")
+    lib = library()
+    scratch = torch.empty((int(lib.blm_sample_scratch_bytes(R, V)) + 7) // 8, dtype=torch.int64, device=logits.device)
     _call("blm_sample", logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), R, V, logits.stride(0),
-          float(temperature), float(top_p), _stream())
+          float(temperature), float(top_p), scratch.data_ptr(), counters.data_ptr(), _stream())
     return out

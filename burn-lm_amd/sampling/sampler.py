@@ -14,6 +14,7 @@ from typing import List, Sequence
 import torch
 
 _MASK = (1 << 64) - 1
+UNIFORM_RING = 8
 
 
 def _splitmix64(x: int) -> int:
@@ -61,6 +62,23 @@ class Sampler:
         # seed 0 means a fresh random seed (crates/burn-lm-llama/src/server/llama3.rs:454-457)
         self.seed = int(seed) if seed else int.from_bytes(os.urandom(8), "little")
         self._ops = ops
+        self._ring, self._next = [], 0
+
+    def _pinned_uniforms(self, values):
+        """The uniforms of one step in pinned host memory that the kernel reads in place (a copy to the
+        GPU would go through the copy engine and cost the step some 20 us of switching between
+        queues).  A ring of buffers; one is written again only after the kernel that read it has run."""
+        n = len(values)
+        if len(self._ring) < UNIFORM_RING:
+            self._ring.append([torch.empty(max(n, 64), dtype=torch.float32).pin_memory(), None])
+        slot = self._ring[self._next % len(self._ring)] if len(self._ring) == UNIFORM_RING else self._ring[-1]
+        self._next += 1
+        if slot[1] is not None:
+            slot[1].synchronize()
+        if slot[0].numel() < n:
+            slot[0] = torch.empty(n, dtype=torch.float32).pin_memory()
+        slot[0].numpy()[:n] = values
+        return slot
 
     @property
     def greedy(self):
@@ -79,9 +97,10 @@ class Sampler:
         if self.greedy:
             out = ops.argmax(logits)
         else:
-            # through pinned memory, so that the copy does not wait for the work already queued
-            u = torch.tensor(self.uniforms(requests, indices), dtype=torch.float32).pin_memory()
-            out = ops.sample(logits, u.to(logits.device, non_blocking=True), self.temperature, self.top_p)
+            slot = self._pinned_uniforms(self.uniforms(requests, indices))
+            out = ops.sample(logits, slot[0][:logits.shape[0]], self.temperature, self.top_p)
+            slot[1] = torch.cuda.Event()
+            slot[1].record()
         return Picked(out)
 
     def pick(self, logits: torch.Tensor, requests: Sequence[int], indices: Sequence[int]) -> List[int]:
