@@ -4,7 +4,7 @@ with no command it opens the shell; ``models`` lists what can be run; ``run <mod
 session with the slash commands ``/help /stats /clear /exit``; ``-d/--dtype`` picks the element
 type (a run-time choice here, a recompilation there).  ``random <preset>`` stands where
 ``download`` does in the reference: it puts a model folder with seeded random weights into the
-models directory.  A model is named by a folder path or by a folder name inside the models
+models directory; ``delete <model>|all`` removes folders from it.  A model is named by a folder path or by a folder name inside the models
 directory (``$BURN_LM_AMD_MODELS``, default ``~/.cache/burn-lm_amd/models``).
 """
 from __future__ import annotations
@@ -56,6 +56,8 @@ def build_parser():
     g.add_argument("--seed", type=int, default=0)
     g.add_argument("--name", default=None, help="folder name inside the models directory (default: the preset's)")
     g.add_argument("--layers", type=int, default=None, help="override the number of layers")
+    dl = sub.add_parser("delete", help="Delete models from the models directory")
+    dl.add_argument("model", help="a folder name inside the models directory, or 'all'")
     sub.add_parser("shell", help="Start a burn-lm-amd shell session")
     return p
 
@@ -86,6 +88,25 @@ def cmd_random(args):
     print(f"writing random weights (seed {args.seed}) for {args.preset} into {folder} ...")
     write_model_folder(folder, cfg, seed=args.seed)
     print("done")
+
+
+def cmd_delete(args):
+    """``delete <model>|all`` (crates/burn-lm-cli/src/commands/delete.rs:4-23): removes model folders,
+    and only those of the models directory, one after the other."""
+    import shutil
+    d = models_dir()
+    present = sorted(n for n in (os.listdir(d) if os.path.isdir(d) else [])
+                     if os.path.exists(os.path.join(d, n, "config.json")))
+    names = present if args.model == "all" else [args.model]
+    for n in names:
+        if n not in present or os.sep in n or n in (".", ".."):
+            raise SystemExit(f"model {n!r} is not in the models directory {d} (it holds: {', '.join(present) or 'nothing'})")
+    for n in names:
+        print(f"deleting model '{n}'...")
+        shutil.rmtree(os.path.join(d, n))
+        print("model deleted!")
+    if not names:
+        print("no model to delete")
 
 
 def cmd_run(args):
@@ -192,6 +213,8 @@ def dispatch(args):
         cmd_chat(args)
     elif args.command == "random":
         cmd_random(args)
+    elif args.command == "delete":
+        cmd_delete(args)
 
 
 def main(argv=None):

@@ -155,3 +155,30 @@ def test_decode_attention_split_rule():
                 n = decode_splits(pages, blocks, hd)
                 assert 1 <= n <= pages
                 assert n == 1 or pages // n >= 4
+
+
+def test_command_line_random_models_delete(tmp_path, monkeypatch, capsys):
+    """`random` writes a model folder into the models directory, `models` lists it, `delete` removes
+    it and nothing outside the models directory."""
+    import pytest
+    from burn_lm_amd.cli.main import main
+    monkeypatch.setenv("BURN_LM_AMD_MODELS", str(tmp_path / "models"))
+    outside = tmp_path / "elsewhere"
+    outside.mkdir()
+    (outside / "config.json").write_text("{}")
+    main(["random", "llama3.2-1b-test", "--name", "mine"])
+    assert (tmp_path / "models" / "mine" / "model.safetensors").exists()
+    capsys.readouterr()
+    main(["models"])
+    listing = capsys.readouterr().out
+    assert "| mine" in listing and "run mine" in listing and "random llama3.2-1b-test" in listing
+    with pytest.raises(SystemExit, match="not in the models directory"):
+        main(["delete", "../elsewhere"])
+    with pytest.raises(SystemExit, match="not in the models directory"):
+        main(["delete", "absent"])
+    main(["delete", "mine"])
+    assert not (tmp_path / "models" / "mine").exists() and (outside / "config.json").exists()
+    main(["random", "llama3.2-1b-test"])
+    main(["random", "llama3.2-1b-test", "--name", "second", "--seed", "3"])
+    main(["delete", "all"])
+    assert sorted(p.name for p in (tmp_path / "models").iterdir()) == []
