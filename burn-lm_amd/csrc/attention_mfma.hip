@@ -320,6 +320,8 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 }
 
 // ---------------------------------------------------------------------------------------
+#define AD_MERGE 32   // splits whose partial results are asked for together when they are merged
+
 // decode: grid (splits, kv heads * head tiles, tokens); partial results per split
 //   part_o [T, nh, splits, HD] float, part_ml [T, nh, splits, 2] float,
 // merged by whichever split of a (token, head tile) finishes last
@@ -469,12 +471,13 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     const size_t head_at = (size_t)t * nh + kvh * G + g0 + cc;
     const size_t base = head_at * n_splits;
     const float* ml = part_ml + base * 2;
-    // eight splits per memory round trip, merged online
+    // AD_MERGE splits per memory round trip, merged online (with eight per trip, 64 splits cost 12 us
+    // of round trips in a row)
     float M = -INFINITY, L = 0.f, O = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += 8) {
-      float vm[8], vl[8], po[8];
+    for (int s0 = 0; s0 < n_splits; s0 += AD_MERGE) {
+      float vm[AD_MERGE], vl[AD_MERGE], po[AD_MERGE];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < AD_MERGE; ++i) {
         const int sp = min(s0 + i, n_splits - 1);
         vm[i] = coherent_load(ml + 2 * sp);
         vl[i] = coherent_load(ml + 2 * sp + 1);
@@ -482,12 +485,12 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       }
       float Mc = M;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) Mc = fmaxf(Mc, vm[i]);
+      for (int i = 0; i < AD_MERGE; ++i) Mc = fmaxf(Mc, vm[i]);
       const float keep = (M == Mc) ? 1.f : __builtin_amdgcn_exp2f(M - Mc);   // maxima are in base 2
       L *= keep;
       O *= keep;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < AD_MERGE; ++i) {
         if (s0 + i < n_splits) {
           const float f = (vm[i] == Mc) ? 1.f : __builtin_amdgcn_exp2f(vm[i] - Mc);
           L += vl[i] * f;
