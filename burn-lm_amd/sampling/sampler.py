@@ -65,16 +65,18 @@ class Sampler:
         self._ring, self._next = [], 0
 
     def _pinned_uniforms(self, values):
-        """The uniforms of one step in pinned host memory that the kernel reads in place (a copy to the
-        GPU would go through the copy engine and cost the step some 20 us of switching between
-        queues).  A ring of buffers; one is written again only after the kernel that read it has run."""
+        """The uniforms of one step in pinned host memory that the kernel reads in place: no copy is
+        queued and no pinned buffer is allocated per step.  A ring of buffers; one is written again
+        only after the kernel that read it has run."""
         n = len(values)
         if len(self._ring) < UNIFORM_RING:
             self._ring.append([torch.empty(max(n, 64), dtype=torch.float32).pin_memory(), None])
-        slot = self._ring[self._next % len(self._ring)] if len(self._ring) == UNIFORM_RING else self._ring[-1]
-        self._next += 1
+            slot = self._ring[-1]
+        else:
+            slot = self._ring[self._next % UNIFORM_RING]
+            self._next += 1
         if slot[1] is not None:
-            slot[1].synchronize()
+            slot[1].synchronize()     # the kernel that read this buffer last has run (long since, as a rule)
         if slot[0].numel() < n:
             slot[0] = torch.empty(n, dtype=torch.float32).pin_memory()
         slot[0].numpy()[:n] = values
