@@ -145,7 +145,8 @@ def test_decode_attention_split_rule():
     from burn_lm_amd.parts.attention import DECODE_MIN_BLOCKS, DECODE_TARGET_BLOCKS, decode_splits
     assert DECODE_TARGET_BLOCKS == 512 and DECODE_MIN_BLOCKS == 128
     # context 4096 (64 pages), 8 key-value heads: batch 1, 2, 4, 8, 16, 64
-    assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 64)] == [16, 8, 8, 8, 4, 1]
+    assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 32, 64)] == [16, 8, 8, 8, 4, 1, 1]
+    assert decode_splits(256, 32 * 8, 64) == 1                                      # every compute unit has a block: no cutting
     assert decode_splits(64, 8, 128) == 16 and decode_splits(64, 64, 128) == 4      # wide heads: half the blocks
     assert decode_splits(1, 8, 64) == 1 and decode_splits(3, 8, 64) == 1 and decode_splits(8, 8, 64) == 2
     assert decode_splits(2048, 8, 64) == 32 and decode_splits(512, 8, 64) == 32     # a long context at batch 1: the cap
