@@ -158,6 +158,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 decode points")
+    ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of picking greedily (0: greedy)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="nucleus mass when sampling")
     ap.add_argument("--unequal", type=int, default=0, metavar="N",
                     help="instead of the decode measurement: N prompts of 64..2048 tokens through the generation loop")
     ap.add_argument("--generate", type=int, default=256, help="tokens generated per prompt with --unequal")
@@ -183,7 +185,7 @@ def main():
                            max_seqs=biggest, max_context=args.context)
     cfg = engine.config
     itemsize = 2 if args.dtype == "bfloat16" else 4
-    sampler = Sampler(temperature=0.0)
+    sampler = Sampler(temperature=args.temperature, top_p=args.top_p, seed=1)
 
     sec = time_decode(engine, sampler, args.batch, args.context, args.steps, args.warmup)
     value = args.batch / sec
@@ -212,7 +214,8 @@ def main():
                    "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size,
                    "tied_head": cfg.tie_word_embeddings, "page_size": engine.cache.page_size,
-                   "sampling": "greedy", "parallelism": "single GPU"},
+                   "sampling": "greedy" if args.temperature == 0 else f"temperature {args.temperature:g} top-p {args.top_p:g}",
+                   "parallelism": "single GPU"},
         "prefill": {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3), "frac": round(pf / psec / peak, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
