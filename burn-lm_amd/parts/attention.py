@@ -11,12 +11,11 @@ from __future__ import annotations
 
 import torch
 
-import os
 
 from .base import KVNeed, Mixer, TensorSpec
 
 # blocks the decode attention aims for when it cuts the key ranges into splits
-DECODE_TARGET_BLOCKS = int(os.environ.get("BLM_DECODE_BLOCKS", "512"))
+DECODE_TARGET_BLOCKS = 512
 DECODE_MIN_BLOCKS = 128
 DECODE_MAX_PIECES = 32
 DECODE_WHOLE_BLOCKS = 256
