@@ -401,7 +401,7 @@ def test_pack_weight_layout(ops):
                                    (8, 257, 2048), (3, 40, 8192), (16, 100, 8200), (5, 31, 14336), (9, 77, 4104),
                                    (2, 9000, 264), (8, 8200, 1024), (6, 100, 4096), (4, 52, 600),
                                    (17, 130, 264), (32, 48, 2048), (29, 5000, 2040), (33, 77, 2048), (32, 200, 4096), (20, 1000, 3072), (48, 257, 520),
-                                   (47, 16, 64), (49, 300, 1032), (64, 4200, 2048), (61, 40, 136)])
+                                   (47, 16, 64), (49, 300, 1032), (64, 4200, 2048), (61, 40, 136), (35, 20000, 520), (64, 12300, 2048)])
 def test_gemv_mfma(ops, out_dtype, M, N, K):
     """Matrix-core skinny product: every way K is cut among wavefronts, tails in N, K and M; above 16
     rows the form with two, three and four row tiles."""
