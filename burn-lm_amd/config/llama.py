@@ -106,8 +106,9 @@ class LlamaConfig:
             if not isinstance(rs, dict):
                 raise ConfigError("config.json: 'rope_scaling' must be null or an object")
             kind = rs.get("rope_type", rs.get("type"))
-            if kind != "llama3":
-                raise ConfigError(f"config.json: rope_scaling.rope_type {kind!r} is not supported (only 'llama3')")
+            if kind not in ("llama3", "default"):
+                raise ConfigError(f"config.json: rope_scaling.rope_type {kind!r} is not supported "
+                                  f"(only 'llama3', or 'default' for none)")
             dflt = RopeScaling()
             w = "config.json rope_scaling"
             scaling = RopeScaling(
@@ -117,6 +118,8 @@ class LlamaConfig:
                 original_max_position_embeddings=(_typed(rs, "original_max_position_embeddings", int, w)
                                                   if "original_max_position_embeddings" in rs
                                                   else dflt.original_max_position_embeddings))
+            if kind == "default":   # the plain frequencies, spelled out
+                scaling = None
         # the architecture has no bias and one activation (crates/burn-lm-llama/src/nn/attention/
         # mha.rs:193-204, nn/fftn.rs:27-32): say so instead of silently ignoring the keys
         for key in ("attention_bias", "mlp_bias"):

@@ -29,6 +29,9 @@ def test_defaults_are_the_references():
     assert c.tie_word_embeddings is False and c.rope_scaling is None
     c = LlamaConfig.from_dict({**TINY_A, "rope_scaling": {"rope_type": "llama3"}})
     assert c.rope_scaling == RopeScaling(8.0, 1.0, 4.0, 8192)
+    # the older key name, and the spelled-out absence of scaling
+    assert LlamaConfig.from_dict({**TINY_A, "rope_scaling": {"type": "llama3", "factor": 2}}).rope_scaling.factor == 2.0
+    assert LlamaConfig.from_dict({**TINY_A, "rope_scaling": {"rope_type": "default"}}).rope_scaling is None
 
 
 @pytest.mark.parametrize("key", ["hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
