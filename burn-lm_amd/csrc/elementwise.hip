@@ -116,7 +116,12 @@ __global__ void __launch_bounds__(512)
       if (dr) {
         // four planes at a time: their loads are issued together (a loop that loads and adds plane
         // by plane waits for memory once per plane), the adds keep the planes' order
-        for (int p0 = 0; p0 < n_planes; p0 += 4) {
+        if (n_planes == 1) {   // the usual case with many rows: one load, not four of the same plane
+          float t[4];
+          load4<TD>(dr + d, t);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[it][e] += t[e];
+        } else for (int p0 = 0; p0 < n_planes; p0 += 4) {
           float t[4][4];
 #pragma unroll
           for (int q = 0; q < 4; ++q) load4<TD>(dr + (size_t)min(p0 + q, n_planes - 1) * plane_stride + d, t[q]);
