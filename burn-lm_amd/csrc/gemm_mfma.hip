@@ -364,7 +364,7 @@ static int launch_gemm(const void* A, const void* W, void* C, int M, int N, int 
   return 0;
 }
 
-#define BLM_GEMM_TILES(X) X(128, 128, 64, 2, 2, 2) X(256, 128, 64, 3, 4, 2) X(256, 256, 64, 2, 4, 2)
+#define BLM_GEMM_TILES(X) X(128, 128, 64, 2, 2, 2) X(256, 128, 64, 3, 4, 2) X(256, 256, 64, 2, 4, 2) X(128, 128, 64, 4, 2, 2) X(128, 64, 64, 6, 4, 1)
 
 // Lets every variant use more than 64 KiB of shared memory; to be called once per device before the
 // first product (not from inside a stream capture).
@@ -382,6 +382,10 @@ extern "C" int blm_gemm_mfma_init() {
 // 1 = 256x128 and 2 = 256x256 (eight wavefronts: two per SIMD, so that one issues matrix instructions
 // while the other issues loads or waits; 10 % faster than four wavefronts with twice the tile each,
 // sixteen are no faster; each of the eight owns 64 rows x 128 columns, 2 % faster than 128 x 64).
+// 3 = 128x128 with a ring of four stages and 4 = 128x64 with six (four wavefronts, one block per
+// compute unit): for products of so few tiles that all run at once, where a block waits for memory
+// and not for the matrix cores; a single 128x128 tile walks K = 2048 in 21 us with two stages and
+// in 19 us with four, a 128x64 tile in 15 us with six.
 // K in stages of 64, two of them in shared memory, three for 256x128;
 // stages of 32 in deeper rings were not faster.  Measured at 256 to 4,096 rows: the largest tile
 // that still gives every compute unit a block is the fastest.
@@ -414,7 +418,9 @@ extern "C" int blm_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
     case 0: BLM_GEMM(128, 128, 64, 2, 2, 2);
     case 1: BLM_GEMM(256, 128, 64, 3, 4, 2);
     case 2: BLM_GEMM(256, 256, 64, 2, 4, 2);
+    case 3: BLM_GEMM(128, 128, 64, 4, 2, 2);
+    case 4: BLM_GEMM(128, 64, 64, 6, 4, 1);
   }
 #undef BLM_GEMM
-  return blm_fail("gemm_mfma: tile %d out of range 0..2", tile);
+  return blm_fail("gemm_mfma: tile %d out of range 0..4", tile);
 }

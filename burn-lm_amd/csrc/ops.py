@@ -419,7 +419,7 @@ def gemv_mfma(a, packed, out, K, gated=False):
     return out
 
 
-GEMM_TILES = {(128, 128): 0, (256, 128): 1, (256, 256): 2}
+GEMM_TILES = {(128, 128): 0, (256, 128): 1, (256, 256): 2, (128, 128, 4): 3, (128, 64, 6): 4}
 _gemm_ready = set()
 
 
@@ -439,7 +439,8 @@ def gemm_mfma(a, w, out, gated=False, tile=(128, 128)):
     checkpoint stores it.  out: bfloat16 or float32 [M, N], or float32 [groups, M, N] partial
     products over that many groups of K (the reader sums them).  gated=True: w is [gate rows; up
     rows] ([2I, K]) and out is [M, I] = silu(a gate^T) * (a up^T).  tile: rows x columns of out (of
-    gate and up columns together when gated) per block, one of GEMM_TILES."""
+    gate and up columns together when gated) per block, one of GEMM_TILES; a third number is the depth of
+    the ring of K stages (deep rings for products of few tiles, which wait for memory, not for the matrix cores)."""
     _gpu(a, w, out)
     gemm_mfma_init(a.device)
     groups = 1

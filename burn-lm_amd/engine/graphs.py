@@ -36,8 +36,9 @@ def batch_bucket(n: int):
 
 # prompt steps: total tokens of the step, and at most this many sequences (a step's attention
 # launches blocks for bucket sequences x bucket tokens; beyond these sizes the launches are no
-# longer what a step's time goes to)
-TOKEN_BUCKETS = (64, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
+# longer what a step's time goes to).  No bucket of 192: the library's products are slower at 192
+# rows than at 256 (a 160-token prompt at the Llama-3.2-3B shape: 4.9 ms padded to 192, 4.3 to 256).
+TOKEN_BUCKETS = (64, 128, 256, 384, 512, 768, 1024, 1536, 2048)
 PROMPT_MAX_SEQS = 16
 
 

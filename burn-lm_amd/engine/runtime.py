@@ -8,11 +8,13 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
   streams the weight once (where the width fits its registers: see ops.gemv_mfma_group_limit).
 * bfloat16 weights, many rows (prefill): the library product (hipBLASLt through torch), as the
   reference's engine leaves its matrix products to its tensor library
-  (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).  With BURN_LM_AMD_FUSED_GATE_UP=1 the
-  gate/up product of a gated feed-forward runs instead on the hand-written matrix-core kernel that
-  applies the gating in its epilogue (ops.gemm_mfma): it never writes the [rows, 2 I] intermediate
-  nor reads it back, but its lower rate eats that gain at wider shapes (measured over whole
-  prefills: 1-6 % faster at the 1B shape, even at 3B, 2-7 % slower at 8B), so it is off unless asked for.
+  (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).  The gate/up product of a gated
+  feed-forward runs instead on the hand-written matrix-core kernel that applies the gating in its
+  epilogue (ops.gemm_mfma) where that is faster: for short prompts whose tiles all run at once
+  (see gated_linear).  With BURN_LM_AMD_FUSED_GATE_UP=1 it is also used for long prompts: it never
+  writes the [rows, 2 I] intermediate nor reads it back, but its lower rate eats that gain at
+  wider shapes (measured over whole prefills: 1-6 % faster at the 1B shape, even at 3B, 2-7 %
+  slower at 8B), so there it is off unless asked for.
 """
 from __future__ import annotations
 
@@ -52,6 +54,7 @@ class Runtime:
         ops.library()  # fail now, loudly, if the kernel library cannot be had
         ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
         ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
+        self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if os.environ.get("BURN_LM_AMD_FUSED_GATE_UP") == "1" else (0, -1)
 
     def empty(self, *shape, dtype=None):
@@ -143,9 +146,21 @@ class Runtime:
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
             return ops.gemv_mfma(x, w.packed, out, K, gated=True)
         plain = w.w if isinstance(w, LinearWeight) else w
-        if (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]
-                and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-                and plain.is_contiguous()):
+        fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
+                   and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
+        if fusable:
+            # Short prompts: when all tiles of the product run at once (one block per compute unit,
+            # most of the units busy), the fused kernel with a deep ring of stages streams the
+            # weights faster than the library product and the gating pass after it (measured at
+            # 65 to 320 rows: 5-25 % at widths of 1536 to 3072, 4 % at 4096; with a second round
+            # of tiles the library is ahead).  The narrower tile first: it spreads over more units.
+            m128 = -(-M // 128)
+            for tile, pairs in (((128, 64, 6), 32), ((128, 128, 4), 64)):
+                blocks = m128 * -(-inner // pairs)
+                if self.compute_units // 4 <= blocks <= self.compute_units:
+                    return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
+                                         gated=True, tile=tile)
+        if fusable and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]:
             # the largest tile that still gives every compute unit a block (a tile of n columns holds n / 2 gated pairs)
             m256 = -(-M // 256)
             tile = ((256, 256) if m256 * -(-inner // 128) >= 256 else

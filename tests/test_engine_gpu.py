@@ -313,6 +313,36 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
             assert rel_err(got[i], want[i][cut[i] + k]) <= TOL["bfloat16"], f"request {i}, decode step {k}"
 
 
+def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
+    """Prompts of 65 rows and more whose gate/up tiles all run at once go through the matrix-core
+    kernel with the gating in its epilogue (both of its deep-ring tiles), longer ones through the
+    library product: all against the plain implementation."""
+    from burn_lm_amd.csrc import ops
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=4096, num_hidden_layers=1,
+               num_attention_heads=16, num_key_value_heads=4, head_dim=128, vocab_size=300, max_position_embeddings=1024,
+               rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False)
+    folder = make_folder(tmp_path / "wide", cfg, seed=6, std=0.03)
+    plain = P.load_model_folder(folder)
+    tiles = []
+    real = ops.gemm_mfma
+    monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: (tiles.append(k.get("tile")), real(*a, **k))[1])
+    eng = load(folder, "bfloat16", max_tokens=2048, graphs=False)
+    # 70 rows: 128 blocks of the 128x64 tile; 100 + 150 rows: 256 of them; 300 + 90: 512, so the 128x128
+    # tile with 256; 700 rows: the library
+    for lengths, tile in (([70], (128, 64, 6)), ([100, 150], (128, 64, 6)), ([300, 90], (128, 128, 4)), ([700], None)):
+        reqs = [random_tokens(300 + i + sum(lengths), 300, n) for i, n in enumerate(lengths)]
+        want = [P.transformer_forward([r], plain)[0] for r in reqs]
+        slots = [eng.open() for _ in reqs]
+        del tiles[:]
+        got = eng.step([(s, r, [0, len(r) // 2, len(r) - 1]) for s, r in zip(slots, reqs)]).double().cpu().numpy()
+        assert tiles == ([tile] if tile else []), (lengths, tiles)
+        for i, r in enumerate(reqs):
+            for j, pos in enumerate([0, len(r) // 2, len(r) - 1]):
+                assert rel_err(got[3 * i + j], want[i][pos]) <= TOL["bfloat16"], (lengths, i, pos)
+        for s in slots:
+            eng.close(s)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("n,bucket", [(20, 24), (70, 96)])
 def test_graph_replays_of_larger_batches(folders, dtype, n, bucket):

@@ -495,7 +495,7 @@ def test_gemv_mfma_refuses_what_it_cannot_do(ops):
         ops.gemv_mfma(dev(torch.zeros(4, 64).bfloat16()), wp, torch.zeros(4, 40, dtype=torch.bfloat16, device="cuda"), 64)
 
 
-@pytest.mark.parametrize("tile", [(128, 128), (256, 128), (256, 256)])
+@pytest.mark.parametrize("tile", [(128, 128), (256, 128), (256, 256), (128, 128, 4), (128, 64, 6)])
 @pytest.mark.parametrize("M,N,K,groups,out_dtype", [(200, 136, 72, 1, "float32"), (300, 264, 200, 1, "bfloat16"),
                                                     (513, 520, 1096, 2, "float32"), (65, 31, 8, 1, "bfloat16"),
                                                     (129, 1000, 2048, 1, "bfloat16"), (260, 100, 4104, 4, "float32")])
@@ -522,7 +522,7 @@ def test_gemm_mfma(ops, tile, M, N, K, groups, out_dtype):
     assert float(err) <= (2e-5 if out_dtype == "float32" else 8e-3), f"error {float(err):.3g}"
 
 
-@pytest.mark.parametrize("tile", [(128, 128), (256, 128), (256, 256)])
+@pytest.mark.parametrize("tile", [(128, 128), (256, 128), (256, 256), (128, 128, 4), (128, 64, 6)])
 @pytest.mark.parametrize("M,I,K", [(70, 176, 64), (300, 264, 200), (257, 1000, 2048), (128, 8, 520)])
 def test_gemm_mfma_gated(ops, tile, M, I, K):
     """The SwiGLU gating in the epilogue: a block takes gate columns and the matching up columns of
