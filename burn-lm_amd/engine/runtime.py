@@ -11,10 +11,11 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
   (crates/burn-lm-llama/src/nn/attention/mha.rs:124-126).  The gate/up product of a gated
   feed-forward runs instead on the hand-written matrix-core kernel that applies the gating in its
   epilogue (ops.gemm_mfma) where that is faster: for short prompts whose tiles all run at once
-  (see gated_linear).  With BURN_LM_AMD_FUSED_GATE_UP=1 it is also used for long prompts: it never
-  writes the [rows, 2 I] intermediate nor reads it back, but its lower rate eats that gain at
-  wider shapes (measured over whole prefills: 1-6 % faster at the 1B shape, even at 3B, 2-7 %
-  slower at 8B), so there it is off unless asked for.
+  and for long prompts of narrow models whose tiles come in whole rounds (see gated_linear).  With
+  BURN_LM_AMD_FUSED_GATE_UP=1 it is used for every prompt of 192 rows and more: it never writes the
+  [rows, 2 I] intermediate nor reads it back, but its lower rate eats that gain at wider shapes
+  (measured over whole prefills: -6 to +4 % at the 1B shape, -6 to +2 % at 3B, 2-7 % slower at
+  8B), so beyond the measured cases it is off unless asked for; =0 leaves every product to the library.
 """
 from __future__ import annotations
 
@@ -55,7 +56,9 @@ class Runtime:
         ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
         ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
-        self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if os.environ.get("BURN_LM_AMD_FUSED_GATE_UP") == "1" else (0, -1)
+        asked = os.environ.get("BURN_LM_AMD_FUSED_GATE_UP")   # "1": wherever it can run, "0": nowhere, unset: where it is ahead
+        self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if asked == "1" else (0, -1)
+        self.fused_gate_up_measured = asked != "0"
 
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
@@ -148,7 +151,7 @@ class Runtime:
         plain = w.w if isinstance(w, LinearWeight) else w
         fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
-        if fusable:
+        if fusable and self.fused_gate_up_measured:
             # Short prompts: when all tiles of the product run at once (one block per compute unit,
             # most of the units busy), the fused kernel with a deep ring of stages streams the
             # weights faster than the library product and the gating pass after it (measured at
@@ -160,6 +163,13 @@ class Runtime:
                 if self.compute_units // 4 <= blocks <= self.compute_units:
                     return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
                                          gated=True, tile=tile)
+            # Long prompts: with whole rounds of 256x256 tiles (as many blocks as compute units, or a
+            # multiple) and a narrow model the fused kernel is ahead of the library over the whole
+            # prefill (width 2048: 2-4 % at 1,024 and 2,048 rows, 0.5 % at 3,072 and 4,096; behind by
+            # 2-6 % with a partial last round, and at width 3072 behind from 1,536 rows on).
+            if K <= 2048 and M >= 256 and (-(-M // 256) * -(-inner // 128)) % self.compute_units == 0:
+                return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
+                                     gated=True, tile=(256, 256))
         if fusable and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]:
             # the largest tile that still gives every compute unit a block (a tile of n columns holds n / 2 gated pairs)
             m256 = -(-M // 256)

@@ -319,17 +319,18 @@ def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
     library product: all against the plain implementation."""
     from burn_lm_amd.csrc import ops
     cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=4096, num_hidden_layers=1,
-               num_attention_heads=16, num_key_value_heads=4, head_dim=128, vocab_size=300, max_position_embeddings=1024,
+               num_attention_heads=16, num_key_value_heads=4, head_dim=128, vocab_size=300, max_position_embeddings=2048,
                rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False)
     folder = make_folder(tmp_path / "wide", cfg, seed=6, std=0.03)
     plain = P.load_model_folder(folder)
     tiles = []
     real = ops.gemm_mfma
     monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: (tiles.append(k.get("tile")), real(*a, **k))[1])
-    eng = load(folder, "bfloat16", max_tokens=2048, graphs=False)
+    eng = load(folder, "bfloat16", max_tokens=4096, graphs=False)
     # 70 rows: 128 blocks of the 128x64 tile; 100 + 150 rows: 256 of them; 300 + 90: 512, so the 128x128
-    # tile with 256; 700 rows: the library
-    for lengths, tile in (([70], (128, 64, 6)), ([100, 150], (128, 64, 6)), ([300, 90], (128, 128, 4)), ([700], None)):
+    # tile with 256; 700 rows: the library (96 tiles of 256x256 are no whole round); 2,000 rows: 256 such tiles
+    for lengths, tile in (([70], (128, 64, 6)), ([100, 150], (128, 64, 6)), ([300, 90], (128, 128, 4)), ([700], None),
+                          ([1500, 500], (256, 256))):
         reqs = [random_tokens(300 + i + sum(lengths), 300, n) for i, n in enumerate(lengths)]
         want = [P.transformer_forward([r], plain)[0] for r in reqs]
         slots = [eng.open() for _ in reqs]
