@@ -526,7 +526,8 @@ def test_a_prompt_fed_in_uneven_chunks_beside_a_decoding_neighbour(folders, dtyp
     assert at == 300
 
 
-@pytest.mark.parametrize("name,dtype,seed", [("A", "float32", 0), ("B", "float32", 1), ("A", "bfloat16", 2), ("B", "bfloat16", 3)])
+@pytest.mark.parametrize("name,dtype,seed", [("A", "float32", 0), ("B", "float32", 1), ("A", "bfloat16", 2), ("B", "bfloat16", 3),
+                                             ("C", "float32", 4), ("C", "bfloat16", 5)])
 def test_random_schedules_of_steps(folders, name, dtype, seed):
     """Sequences are opened, fed in random chunks (whole prompts, pieces, single tokens, several
     sequences per step in random order), and closed at random, on a cache small enough that slots and
@@ -591,7 +592,7 @@ def test_random_schedules_of_steps(folders, name, dtype, seed):
     assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 5
 
 
-@pytest.mark.parametrize("name,dtype,seed", [("A", "bfloat16", 0), ("B", "float32", 1)])
+@pytest.mark.parametrize("name,dtype,seed", [("A", "bfloat16", 0), ("B", "float32", 1), ("C", "bfloat16", 2)])
 def test_random_schedules_through_recorded_graphs(folders, name, dtype, seed):
     """Like the random schedules above, but every step asks for the last logits of each of its
     sequences, so decode steps and prompt steps (whole prompts, pieces, mixed with single tokens)

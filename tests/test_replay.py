@@ -1,7 +1,7 @@
 """Trace replay through bin/trace_run, as a user runs it, against the plain implementation:
 each request whole; with its last 32 tokens one by one; and in batches of unequal lengths whose
 shorter requests end earlier, one batch after another on a cache so small that pages and slots
-are used again.  In 32-bit and in bfloat16, on two tiny configurations."""
+are used again.  In 32-bit and in bfloat16, on two tiny configurations and a middle-sized one."""
 import pytest
 
 import plain_llama as P
@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 LENGTHS = [1, 2, 33, 64, 65, 100, 7, 150]
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C"])
 def case(request, tmp_path_factory):
     cfg, seed = TINIES[request.param]
     folder = make_folder(tmp_path_factory.mktemp("model" + request.param), cfg, seed)
