@@ -647,3 +647,45 @@ def test_random_schedules_through_recorded_graphs(folders, name, dtype, seed):
     shapes = eng.graphs.captured
     assert checked > 200 and eng.graphs.replays > 60 and any(k[1] > 0 for k in shapes) and any(k[1] == 0 for k in shapes)
 
+
+
+def test_the_benchmark_layer_shape_against_the_plain_implementation(tmp_path):
+    """Two layers of the Llama-3.2-1B shape (width 2048, 32 heads in 8 groups, feed-forward 8192,
+    vocabulary 128,256, tied head, the published frequency scaling): the sizes at which the
+    products' policies choose differently than at the small configurations (K-groups, the fused
+    gate/up product in whole rounds of tiles, the head over the whole vocabulary).  Prompts of
+    2,048, 700 and 76 tokens alone and in one batch, then twelve tokens one by one, in both dtypes."""
+    from burn_lm_amd.config.presets import preset
+    cfg = dict(preset("llama3.2-1b"))
+    cfg["num_hidden_layers"] = 2
+    folder = make_folder(tmp_path / "shape", cfg, seed=3, std=0.02)
+    plain = P.load_model_folder(folder)
+    n_dec = 12
+    reqs = [random_tokens(40 + i, cfg["vocab_size"], n + n_dec) for i, n in enumerate([2048, 700, 76])]
+
+    def plain_rows(toks, rows):   # the plain blocks, with the head on the wanted rows only
+        h = plain["tok_embeddings"][np.asarray([toks])]
+        for lw in plain["layers"]:
+            h = P.block(h, lw, plain["cfg"], plain["freqs"], 0)
+        return P.rms_norm(h, plain["norm"], plain["cfg"]["eps"])[0][rows] @ plain["output"].T
+
+    want = []
+    for r in reqs:
+        cut = len(r) - n_dec
+        want.append(plain_rows(r, [0, cut // 2, cut - 1] + list(range(cut, len(r)))))
+    for dtype, tol in (("float32", 1e-5), ("bfloat16", TOL["bfloat16"])):
+        eng = load(folder, dtype, max_tokens=4096, max_seqs=4)
+        for group in ([0], [1], [2], [0, 1, 2]):
+            slots = {i: eng.open() for i in group}
+            cut = {i: len(reqs[i]) - n_dec for i in group}
+            got = eng.step([(slots[i], reqs[i][:cut[i]], [0, cut[i] // 2, cut[i] - 1]) for i in group]).double().cpu().numpy()
+            for k, i in enumerate(group):
+                for j in range(3):
+                    assert rel_err(got[3 * k + j], want[i][j]) <= tol, f"{dtype} {group}: request {i}, prompt row {j}"
+            for s in range(n_dec):
+                got = eng.step([(slots[i], [reqs[i][cut[i] + s]], [0]) for i in group]).double().cpu().numpy()
+                for k, i in enumerate(group):
+                    assert rel_err(got[k], want[i][3 + s]) <= tol, f"{dtype} {group}: request {i}, decode step {s}"
+            for i in group:
+                eng.close(slots[i])
+        del eng
