@@ -316,7 +316,8 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
 def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
     """Prompts of 65 rows and more whose gate/up tiles all run at once go through the matrix-core
     kernel with the gating in its epilogue (both of its deep-ring tiles), longer ones through the
-    library product: all against the plain implementation."""
+    library product; the narrow products of short prompts come as partial planes over groups of K:
+    all against the plain implementation."""
     from burn_lm_amd.csrc import ops
     cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=4096, num_hidden_layers=1,
                num_attention_heads=16, num_key_value_heads=4, head_dim=128, vocab_size=300, max_position_embeddings=2048,
@@ -325,7 +326,9 @@ def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
     plain = P.load_model_folder(folder)
     tiles = []
     real = ops.gemm_mfma
-    monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: (tiles.append(k.get("tile")), real(*a, **k))[1])
+    planes = []
+    monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: ((tiles if k.get("gated") else planes).append(k.get("tile")),
+                                                           real(*a, **k))[1])
     eng = load(folder, "bfloat16", max_tokens=4096, graphs=False)
     # 70 rows: 128 blocks of the 128x64 tile; 100 + 150 rows: 256 of them; 300 + 90: 512, so the 128x128
     # tile with 256; 700 rows: the library (96 tiles of 256x256 are no whole round); 2,000 rows: 256 such tiles
@@ -334,9 +337,12 @@ def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
         reqs = [random_tokens(300 + i + sum(lengths), 300, n) for i, n in enumerate(lengths)]
         want = [P.transformer_forward([r], plain)[0] for r in reqs]
         slots = [eng.open() for _ in reqs]
-        del tiles[:]
+        del tiles[:], planes[:]
         got = eng.step([(s, r, [0, len(r) // 2, len(r) - 1]) for s, r in zip(slots, reqs)]).double().cpu().numpy()
         assert tiles == ([tile] if tile else []), (lengths, tiles)
+        # the output and down projections come as partial planes where a few groups of K fill the chip
+        n_planes = sum(1 for N, K in ((2048, 2048), (2048, 4096)) if eng.rt.mid_k_groups(sum(lengths), N, K))
+        assert len(planes) == n_planes and (n_planes >= 1) == (sum(lengths) <= 512), (lengths, planes)
         for i, r in enumerate(reqs):
             for j, pos in enumerate([0, len(r) // 2, len(r) - 1]):
                 assert rel_err(got[3 * i + j], want[i][pos]) <= TOL["bfloat16"], (lengths, i, pos)
