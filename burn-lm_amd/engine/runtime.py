@@ -97,14 +97,14 @@ class Runtime:
     def mid_k_groups(self, M, N, K):
         """Short prompts, narrow output, long K (the down projection): the product as partial planes
         of 128x64 tiles over groups of K (the block's next norm sums the planes), when eight, four
-        or two groups of at least 1024 give every compute unit at most one block and half of them
+        or two groups of at least 768 give every compute unit at most one block and half of them
         one; 0 otherwise (the library's product).  Measured over whole prompts of 65 to 128 tokens:
-        6 % faster at the Llama-3.2-1B shape, 14 % at 3B, 21 % at 8B (the library's product of few
+        6 % faster at the Llama-3.2-1B shape, 19 % at 3B, 21 % at 8B (the library's product of few
         rows and a long K streams the weights at a quarter of the memory rate); 2-5 % up to 512
         tokens, where two groups still fit; equal beyond."""
         tiles = -(-M // 128) * -(-N // 64)
         for g in (8, 4, 2):
-            if K // g >= 1024 and self.compute_units // 2 <= tiles * g <= self.compute_units:
+            if K // g >= 768 and self.compute_units // 2 <= tiles * g <= self.compute_units:
                 return g
         return 0
 
