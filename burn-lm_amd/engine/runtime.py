@@ -62,6 +62,8 @@ class Runtime:
         self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if asked == "1" else (0, -1)
         self.fused_gate_up_measured = asked != "0"
         self.mid_partials = os.environ.get("BURN_LM_AMD_MID_PARTIALS") != "0"   # "0": the library's products instead
+        self.skinny_gated_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_GATED_ROWS", MFMA_SKINNY_MAX_ROWS))
+        self.skinny_planes_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_PLANES_ROWS", MFMA_SKINNY_MAX_ROWS))
 
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
@@ -127,6 +129,12 @@ class Runtime:
                 return ops.gemv_skinny(x, w, out)
             return ops.gemm_tiled(x, w, out)
         aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+        if (partials and out is None and self.mid_partials and M > self.skinny_planes_rows and aligned
+                and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()):
+            groups = self.mid_k_groups(M, N, K)
+            if groups:
+                return ops.gemm_mfma(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device),
+                                     tile=(128, 64, 6))
         if packed is not None and M <= MFMA_SKINNY_MAX_ROWS and aligned:
             if partials and out is None:
                 groups = self.k_groups(N, K, M)
@@ -136,12 +144,6 @@ class Runtime:
                 if out is None:
                     out = torch.empty(M, N, dtype=out_dtype, device=x.device)
                 return ops.gemv_mfma(x, packed, out, K)
-        if (partials and out is None and self.mid_partials and M > MFMA_SKINNY_MAX_ROWS and aligned
-                and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()):
-            groups = self.mid_k_groups(M, N, K)
-            if groups:
-                return ops.gemm_mfma(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device),
-                                     tile=(128, 64, 6))
         if out is None:
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         if packed is not None and aligned and out_dtype == torch.float32:
@@ -167,7 +169,7 @@ class Runtime:
         M, K = x.shape
         inner = w.shape[0] // 2
         if (isinstance(w, LinearWeight) and w.packed is not None and w.gated and x.dtype == torch.bfloat16
-                and M <= MFMA_SKINNY_MAX_ROWS and ops.gemv_mfma_supported(M, w.shape[0], K)
+                and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
             return ops.gemv_mfma(x, w.packed, out, K, gated=True)
