@@ -62,6 +62,9 @@ class Runtime:
         self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if asked == "1" else (0, -1)
         self.fused_gate_up_measured = asked != "0"
         self.mid_partials = os.environ.get("BURN_LM_AMD_MID_PARTIALS") != "0"   # "0": the library's products instead
+        # most rows for which the skinny kernels take the gated product and the partial planes; above,
+        # the matrix-core kernels of short prompts do where their tiles fit (settings for measurements:
+        # from 33 rows on those are 1-2 % ahead at some shapes and as much behind at others)
         self.skinny_gated_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_GATED_ROWS", MFMA_SKINNY_MAX_ROWS))
         self.skinny_planes_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_PLANES_ROWS", MFMA_SKINNY_MAX_ROWS))
 
