@@ -695,3 +695,18 @@ def test_the_benchmark_layer_shape_against_the_plain_implementation(tmp_path):
             for i in group:
                 eng.close(slots[i])
         del eng
+
+
+def test_wanted_places_come_back_in_the_order_given(folders):
+    """Logits come in the order of the entries and, within an entry, of its list of wanted places as
+    given: unsorted, and with a place named twice."""
+    cfg, seed = TINIES["A"]
+    plain = P.load_model_folder(folders["A"])
+    a, b = random_tokens(810, cfg["vocab_size"], 9), random_tokens(811, cfg["vocab_size"], 5)
+    wa, wb = P.transformer_forward([a], plain)[0], P.transformer_forward([b], plain)[0]
+    eng = load(folders["A"], "float32")
+    sa, sb = eng.open(), eng.open()
+    got = eng.step([(sa, a, [7, 0, 7, 3]), (sb, b, [4, 1])]).double().cpu().numpy()
+    assert got.shape[0] == 6
+    for row, want in zip(got, [wa[7], wa[0], wa[7], wa[3], wb[4], wb[1]]):
+        assert rel_err(row, want) <= TOL["float32"]
