@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 _lib = None
 _lock = threading.Lock()
 
@@ -55,6 +55,8 @@ _SIGNATURES = {
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
+    "blm_static_scratch_init": [],
+    "blm_argmax_static": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p, _c_void_p,
                    _c_void_p],
 }
@@ -432,6 +434,20 @@ def gemm_mfma_init(device=None):
         with torch.cuda.device(index):
             _call("blm_gemm_mfma_init")
         _gemm_ready.add(index)
+
+
+_static_ready = set()
+
+
+def static_scratch_init(device=None):
+    """Once per device, outside any stream capture: the library looks up where its own scratch array
+    lies on that device (blm_argmax_static, the entry point for callers that cannot allocate)."""
+    index = torch.device(device or "cuda").index
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _static_ready:
+        with torch.cuda.device(index):
+            _call("blm_static_scratch_init")
+        _static_ready.add(index)
 
 
 def gemm_mfma(a, w, out, gated=False, tile=(128, 128)):

@@ -20,7 +20,10 @@
 // histogram bins added to the row's with device-wide atomics, chunk masses) in device-coherent
 // memory, count themselves in, and the block that arrives last finishes the pass for the row (the
 // row's maximum, the bin of this level, the pick).  No block ever waits for another.
+#include <mutex>
+
 #include "common.h"
+#include "no_alloc.h"
 
 
 // Two stages so that a row of a large vocabulary is searched by many blocks: stage one leaves the
@@ -78,6 +81,53 @@ __global__ void argmax_final_kernel(const float* __restrict__ slice_val, const i
 extern "C" int blm_argmax(const float* logits, int* out, int R, int V, int ld, float* slice_val, int* slice_idx,
                           hipStream_t stream) {
   BLM_REQUIRE(R > 0 && R <= 65535 && V > 0 && ld >= V, "argmax: bad sizes R=%d V=%d ld=%d", R, V, ld);
+  hipLaunchKernelGGL(argmax_slice_kernel, dim3(ARGMAX_SLICES, R), dim3(256), 0, stream, logits, slice_val, slice_idx, V, ld);
+  BLM_LAUNCH_CHECK("argmax_slice");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(BLM_WAVE), 0, stream, slice_val, slice_idx, out);
+  BLM_LAUNCH_CHECK("argmax_final");
+  return 0;
+}
+
+// ---- the same without workspace arguments: see no_alloc.h ------------------------------------
+// The array's name is only a stand-in in host code: its address on each device comes from
+// hipGetSymbolAddress, asked once per device with that device current, and is what the kernels get.
+#define ARGMAX_STATIC_DEVICES 64
+static __device__ __align__(256) unsigned char argmax_static_scratch[BLM_ARGMAX_STATIC_MAX_ROWS * ARGMAX_SLICES * 8];
+static void* g_argmax_static_ptr[ARGMAX_STATIC_DEVICES];
+static std::mutex g_argmax_static_mutex;
+
+static int argmax_static_address(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  BLM_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  BLM_REQUIRE(dev >= 0 && dev < ARGMAX_STATIC_DEVICES, "argmax_static: device %d is beyond the %d this library keeps an address for",
+              dev, ARGMAX_STATIC_DEVICES);
+  std::lock_guard<std::mutex> hold(g_argmax_static_mutex);
+  if (g_argmax_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_static_scratch));
+    BLM_REQUIRE(e == hipSuccess && p != nullptr, "argmax_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                hipGetErrorString(e));
+    g_argmax_static_ptr[dev] = p;
+  }
+  *ptr = g_argmax_static_ptr[dev];
+  return 0;
+}
+
+extern "C" int blm_static_scratch_init() {
+  void* p = nullptr;
+  return argmax_static_address(&p);
+}
+
+extern "C" int blm_argmax_static(const float* logits, int* out, int R, int V, int ld, hipStream_t stream) {
+  BLM_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: logits and out must be given");
+  BLM_REQUIRE(R > 0 && V > 0 && ld >= V, "argmax_static: bad sizes R=%d V=%d ld=%d", R, V, ld);
+  BLM_REQUIRE(R <= BLM_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows, the library's own scratch array holds %d (use blm_argmax with workspaces)",
+              R, BLM_ARGMAX_STATIC_MAX_ROWS);
+  void* base = nullptr;
+  if (argmax_static_address(&base)) return 1;
+  float* slice_val = reinterpret_cast<float*>(base);
+  int* slice_idx = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(base) + (size_t)BLM_ARGMAX_STATIC_MAX_ROWS * ARGMAX_SLICES * 4);
   hipLaunchKernelGGL(argmax_slice_kernel, dim3(ARGMAX_SLICES, R), dim3(256), 0, stream, logits, slice_val, slice_idx, V, ld);
   BLM_LAUNCH_CHECK("argmax_slice");
   hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(BLM_WAVE), 0, stream, slice_val, slice_idx, out);
