@@ -4,9 +4,10 @@
 (crates/burn-lm-llama/src/tokenizer/byte.rs:3-49: bos 0, eos 1, stop ids [2]); it needs a
 vocabulary of at least 256.  Where the reference prints the id list on decode (byte.rs:34-36),
 this one gives the bytes back as text.  A ``tokenizer.json`` in the model folder is used instead
-when the ``tokenizers`` package can read it; its stop ids are those of the special tokens the
-reference's Llama-3 tokenizer stops at (crates/burn-lm-llama/src/tokenizer/tiktoken.rs:12-15,
-126-132), as far as the file defines them."""
+when the ``tokenizers`` package can read it; which of its special tokens begin and end a text and
+which stop a generation is the architecture's knowledge (``registry.Architecture.special_tokens``;
+the reference's Llama-3 tokenizer: crates/burn-lm-llama/src/tokenizer/tiktoken.rs:12-15, 126-132),
+used as far as the file defines them."""
 from __future__ import annotations
 
 import os
@@ -28,13 +29,13 @@ class ByteTokenizer:
 
 
 class FileTokenizer:
-    BOS, EOS = "<|begin_of_text|>", "<|end_of_text|>"
-    STOPS = ("<|end_of_text|>", "<|eom_id|>", "<|eot_id|>")
-
-    def __init__(self, path):
+    def __init__(self, path, special_tokens=None):
         from tokenizers import Tokenizer
         self._tok = Tokenizer.from_file(path)
-        self.bos_id, self.eos_id = self._tok.token_to_id(self.BOS), self._tok.token_to_id(self.EOS)
+        sp = special_tokens or {}
+        self._stops = tuple(sp.get("stops", ()))
+        self.bos_id = self._tok.token_to_id(sp["bos"]) if sp.get("bos") else None
+        self.eos_id = self._tok.token_to_id(sp["eos"]) if sp.get("eos") else None
 
     def encode(self, text, bos=False, eos=False):
         ids = self._tok.encode(text, add_special_tokens=False).ids
@@ -48,15 +49,16 @@ class FileTokenizer:
         return self._tok.decode(list(tokens), skip_special_tokens=True)
 
     def stop_ids(self):
-        ids = [self._tok.token_to_id(t) for t in self.STOPS]
+        ids = [self._tok.token_to_id(t) for t in self._stops]
         return [i for i in ids if i is not None]
 
 
-def for_folder(folder: str, vocab_size: int):
+def for_folder(folder: str, vocab_size: int, special_tokens=None):
+    """special_tokens: the architecture's names of the tokens that begin, end and stop a text."""
     path = os.path.join(folder, "tokenizer.json")
     if os.path.exists(path):
         try:
-            return FileTokenizer(path)
+            return FileTokenizer(path, special_tokens)
         except Exception as e:  # unreadable file: say so and fall back to bytes
             print(f"warning: {path} could not be read ({e}); using the byte tokenizer")
     if vocab_size < 256:

@@ -14,10 +14,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Optional, Tuple
 
-
-class ConfigError(ValueError):
-    """config.json is missing a key, holds a value of the wrong kind, or asks for something
-    the architecture does not have."""
+from ..errors import ConfigError  # noqa: F401  (also imported from here by older callers)
 
 
 @dataclass(frozen=True)

@@ -563,6 +563,8 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
               "attn_decode: bad geometry width=%d window=%d splits=%d", table_width, window, n_splits);
   BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attn_decode: q rows must be 16-byte aligned");
   BLM_REQUIRE(scale > 0.f, "attn_decode: the score scale must be positive (got %g)", (double)scale);
+  BLM_REQUIRE(n_splits == 1 || (part_o != nullptr && part_ml != nullptr && arrivals != nullptr),
+              "attn_decode: %d splits need the workspaces for partial results and the arrival counters", n_splits);
   const int G = nh / nkv;
   const int gtiles = (G + 15) / 16;
   BLM_REQUIRE((long long)nkv * gtiles <= 65535, "attn_decode: too many heads");

@@ -318,17 +318,27 @@ def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache,
         raise KernelError("attn_decode: q rows must be contiguous and at least heads*head_dim long")
     _check_planes("attn_decode", kcache, vcache, nkv, page_size, hd)
     _i32("positions", positions, T); _i32("token_seq", token_seq, T); _i32("block_table", block_table)
-    n_splits = max(1, int(n_splits))
-    part_o = torch.empty(T * nh * n_splits * hd, dtype=torch.float32, device=out.device)
-    part_ml = torch.empty(T * nh * n_splits * 2, dtype=torch.float32, device=out.device)
-    arrivals = arrival_counters(out.device)
-    if T * nkv * ((nh // nkv + 15) // 16) > arrivals.numel():
-        raise KernelError(f"attn_decode: {T} tokens x {nkv} key-value heads need more than {arrivals.numel()} counters")
+    n_splits = decode_pieces(T, nh, nkv, n_splits, arrival_counters(out.device).numel())
+    part_o = part_ml = arrivals = None
+    if n_splits > 1:    # an uncut key range leaves no partial result and counts nobody in
+        part_o = torch.empty(T * nh * n_splits * hd, dtype=torch.float32, device=out.device)
+        part_ml = torch.empty(T * nh * n_splits * 2, dtype=torch.float32, device=out.device)
+        arrivals = arrival_counters(out.device)
     _call("blm_attn_decode", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
-          page_size, T, nh, nkv, hd, float(scale), int(window), n_splits, part_o.data_ptr(), part_ml.data_ptr(),
-          arrivals.data_ptr(), _stream())
+          page_size, T, nh, nkv, hd, float(scale), int(window), n_splits, _ptr(part_o), _ptr(part_ml),
+          _ptr(arrivals), _stream())
     return out
+
+
+def decode_pieces(T, nh, nkv, n_splits, n_counters):
+    """Into how many pieces attn_decode really cuts the key ranges: as asked, but not at all when
+    the (token, head tile) pairs outnumber the arrival counters (so many pairs are work enough for
+    the whole chip without cutting, as attn_paged decides too)."""
+    n_splits = max(1, int(n_splits))
+    if n_splits > 1 and T * nkv * ((nh // nkv + 15) // 16) > n_counters:
+        return 1
+    return n_splits
 
 
 def _check_mm(a, w, out):

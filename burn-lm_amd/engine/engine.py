@@ -11,6 +11,7 @@ reference's loop (crates/burn-lm-llama/src/generation/generate.rs:66-85) is one 
 """
 from __future__ import annotations
 
+import operator
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -55,6 +56,20 @@ class Engine:
             self.cache.close(s)
 
     # ---- the step ----------------------------------------------------------------------------
+    @staticmethod
+    def _integers(slot, what, values):
+        """values as Python integers; anything that is no integer (a float, a string, a bool) is refused
+        as such, numpy's and torch's integer scalars are taken."""
+        out = []
+        for v in values:
+            if isinstance(v, bool):
+                raise StepError(f"slot {slot}: {what} {v!r} is a {type(v).__name__}, not an integer")
+            try:
+                out.append(operator.index(v))
+            except TypeError:
+                raise StepError(f"slot {slot}: {what} {v!r} is a {type(v).__name__}, not an integer") from None
+        return out
+
     def _check(self, entries):
         if not entries:
             raise StepError("a step needs at least one sequence")
@@ -64,14 +79,14 @@ class Engine:
             if n == 0:
                 raise StepError(f"slot {slot}: a step must bring at least one token per sequence")
             for t in tokens:
-                if not (isinstance(t, int) and 0 <= t < V):
+                if not 0 <= t < V:
                     raise StepError(f"slot {slot}: token {t!r} is outside the vocabulary of {V}")
             for w in want:
-                if not (isinstance(w, int) and 0 <= w < n):
+                if not 0 <= w < n:
                     raise StepError(f"slot {slot}: wanted place {w!r} is outside this step's {n} tokens")
 
     def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> Optional[torch.Tensor]:
-        entries = [(int(s), list(t), list(w)) for s, t, w in entries]
+        entries = [(int(s), self._integers(s, "token", t), self._integers(s, "wanted place", w)) for s, t, w in entries]
         self._check(entries)
         lengths = [self.cache.length(s) for s, _, _ in entries]
         self.cache.reserve([(s, len(t)) for s, t, _ in entries])  # raises before any change

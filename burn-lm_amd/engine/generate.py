@@ -98,14 +98,17 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
     ahead = hasattr(engine, "step_ahead") and hasattr(sampler, "pick_device")
     for batch in batches:
         ids = [runnable[j] for j in batch]
-        live = [(i, engine.open()) for i in ids]
-        open_slots = {slot for _, slot in live}
+        live, open_slots = [], set()
 
         def close(slot):
             open_slots.discard(slot)
             engine.close(slot)
 
         try:
+            for i in ids:       # inside the try: a slot that cannot be had must not strand the ones already opened
+                slot = engine.open()
+                open_slots.add(slot)
+                live.append((i, slot))
             t0 = clock()
             logits = engine.step([(slot, list(prompts[i]), [len(prompts[i]) - 1]) for i, slot in live])
             picked = sampler.pick(logits, [i for i, _ in live], [0] * len(live))

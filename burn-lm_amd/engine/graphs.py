@@ -8,6 +8,12 @@ on replayed: the host only refreshes one int32 buffer (tokens, positions, page t
 launches the graph.  Two kinds of step are recorded: decode steps (one token per sequence, its
 logits wanted) and prompt steps (any number of tokens per sequence, the last one's logits wanted).
 
+A shape is recorded the second time it is met (a shape met once is not worth a graph), right after
+it has run once more eagerly *at the bucket's own size* (all padding), so that every kernel and
+library handle the recording needs exists beforehand.  At most ``MAX_GRAPHS`` shapes are kept; the
+one replayed longest ago makes room for a new one (a recorded shape holds its index and logits
+buffers and its share of the graphs' memory pool).
+
 Places of the bucket that nothing fills are padding: padding tokens belong to no sequence (index
 -1), so they write no cache; padding sequences bring no token; their rows are dropped.  The kernels
 compute every row on its own, so padding changes no result.  Only models whose parts all declare
@@ -25,6 +31,8 @@ import torch
 from .batch import Step
 
 BATCH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128)
+MAX_GRAPHS = 48         # recorded shapes kept at a time
+RECORD_AT_SIGHT = 2     # a shape is recorded when it is met for this many-th time
 
 
 def batch_bucket(n: int):
@@ -91,6 +99,7 @@ class _Captured:
                          max_len_after=span, is_decode=self.decode, host_slots=[], host_new=[])
         self.fill([], cache)       # all padding: valid contents while capturing
         self.dev.copy_(self.host)
+        engine.model.forward(self.step, cache)      # once eagerly at the bucket's size: what the recording meets exists
         self.graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize()
         # No garbage collection while the capture is open: a collected object that owns GPU memory or
@@ -149,10 +158,12 @@ class StepGraphs:
         # a weak reference: the engine owns this object, and a cycle would leave the graphs to the
         # cyclic collector, which may run at any time (see the note on capture above)
         self._engine = weakref.ref(engine)
-        self.captured: Dict[Tuple[int, int, int], _Captured] = {}
+        self.captured: Dict[Tuple[int, int, int], _Captured] = {}     # in order of last use, oldest first
+        self.sightings: Dict[Tuple[int, int, int], int] = {}
         self.pool = None
         self.enabled = all(p.graph_safe for p in engine.model.all_parts())
         self.replays = 0
+        self.evicted = 0
 
     def key_for(self, entries, lengths):
         """Bucket key (sequences, tokens or 0 for a decode step, table width) of a step, or None if
@@ -176,25 +187,41 @@ class StepGraphs:
     def run(self, key, entries):
         """Replays the step if its shape has been captured; returns None if it must run eagerly
         (the first time a shape is met; it is captured right after that run)."""
-        c = self.captured.get(key)
+        c = self._use(key)
         if c is None:
             return None
         self.replays += 1
         return c.run(entries, self._engine().cache)
 
+    def _use(self, key):
+        """The recorded shape, moved to the young end of the order of use; None if it is not recorded."""
+        c = self.captured.pop(key, None)
+        if c is not None:
+            self.captured[key] = c
+        return c
+
     def run_ahead(self, key, slots, rows, tokens_dev):
         """Replays a recorded decode shape with the tokens taken on the device; None if it is not recorded."""
-        c = self.captured.get(key)
+        c = self._use(key)
         if c is None:
             return None
         self.replays += 1
         return c.run_ahead(slots, rows, tokens_dev, self._engine().cache)
 
     def after_eager(self, key):
-        """The shape has just run eagerly (so every kernel and library handle it needs exists):
-        capture it for the next time."""
+        """The shape has just run eagerly.  Met for the second time it is recorded for the times to
+        come; the shape used longest ago goes if the table is full."""
         if key in self.captured:
+            return
+        self.sightings[key] = self.sightings.get(key, 0) + 1
+        if self.sightings[key] < RECORD_AT_SIGHT:
             return
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
+        while len(self.captured) >= MAX_GRAPHS:
+            oldest = next(iter(self.captured))
+            torch.cuda.synchronize()        # nothing of the old shape is still running when its buffers go
+            del self.captured[oldest]
+            self.sightings.pop(oldest, None)
+            self.evicted += 1
         self.captured[key] = _Captured(self._engine(), key[0], key[1], key[2], self.pool)

@@ -20,15 +20,19 @@ class Model:
         self.final_norm = registry.part("norm", plan.final_norm.kind)(plan.final_norm.params, plan.final_norm.names)
         self.head = registry.part("head", plan.head.kind)(plan.head.params, plan.head.names)
         self.blocks = []
-        for lp in plan.layers:
-            mp = dict(lp.mixer.params)
-            if lp.position is not None:
-                mp["position"] = self.positions[lp.position]
-            mixer = registry.part("mixer", lp.mixer.kind)(mp, lp.mixer.names)
-            ffn = registry.part("feed_forward", lp.feed_forward.kind)(lp.feed_forward.params, lp.feed_forward.names)
-            n1 = registry.part("norm", lp.mixer_norm.kind)(lp.mixer_norm.params, lp.mixer_norm.names)
-            n2 = registry.part("norm", lp.ffn_norm.kind)(lp.ffn_norm.params, lp.ffn_norm.names)
-            self.blocks.append(registry.part("block", lp.block)(mixer, ffn, n1, n2))
+        for li, lp in enumerate(plan.layers):
+            block_cls = registry.part("block", lp.block)
+            made = {}
+            for role, spec in lp.parts.items():
+                family = block_cls.roles.get(role)
+                if family is None:
+                    raise ValueError(f"layer {li}: the block {lp.block!r} has no role {role!r}; "
+                                     f"its roles: {', '.join(block_cls.roles) or 'none'}")
+                params = dict(spec.params)
+                if family == "mixer" and lp.position is not None:
+                    params["position"] = self.positions[lp.position]
+                made[role] = registry.part(family, spec.kind)(params, spec.names)
+            self.blocks.append(block_cls(made))
         for i, place in enumerate(plan.order):
             if not 0 <= place.layer < len(self.blocks):
                 raise ValueError(f"place {i} of the layer order names layer {place.layer}, "
@@ -61,7 +65,7 @@ class Model:
             p.bind(tensors, rt)
 
     def cache_needs(self) -> List:
-        return [self.blocks[pl.layer].mixer.cache_need() for pl in self.plan.order]
+        return [self.blocks[pl.layer].cache_need() for pl in self.plan.order]
 
     def reads_from(self) -> List:
         return [pl.reads_cache_of for pl in self.plan.order]

@@ -66,11 +66,14 @@ def plan(cfg: LlamaConfig, checkpoint_names=None) -> ModelPlan:
         + ((r"^lm_head\.weight$", r"^output\.weight$") if cfg.tie_word_embeddings else ()))
 
 
-def checkpoint_tensors(cfg: LlamaConfig):
-    """Name -> (shape, role) of a fresh Hugging Face-named checkpoint of this configuration."""
-    n = HF_NAMES
+def checkpoint_tensors(cfg: LlamaConfig, names: str = "hf"):
+    """Name -> (shape, role) of a fresh checkpoint of this configuration under Hugging Face names
+    (``names="hf"``) or Meta names (``"meta"``: q/k rows in the adjacent-pair order)."""
+    if names not in ("hf", "meta"):
+        raise ValueError(f"checkpoint names {names!r} unknown; 'hf' or 'meta'")
+    n = HF_NAMES if names == "hf" else META_NAMES
     d, hd = cfg.hidden_size, cfg.head_dim
-    out = {n["embedding"]: ((cfg.vocab_size, d), "matrix")}
+    out = {n["embedding"]: ((cfg.vocab_size, d), "table")}
     for i in range(cfg.num_hidden_layers):
         p = n["layer"].format(i=i)
         out[p + n["mixer_norm"]] = ((d,), "norm")
@@ -88,6 +91,20 @@ def checkpoint_tensors(cfg: LlamaConfig):
     return out
 
 
+def chat_template(messages) -> str:
+    """The Llama-3 chat framing of crates/burn-lm-llama/src/server/llama3.rs:561-576: every message
+    under a header with its role, closed by ``<|eot_id|>``, then the header of the assistant's turn."""
+    out = "".join(f"<|start_header_id|>{m['role'].lower()}<|end_header_id|>\n\n{m['content']}<|eot_id|>"
+                  for m in messages)
+    return out + "<|start_header_id|>assistant<|end_header_id|>\n\n"
+
+
+# the special tokens the reference's Llama-3 tokenizer knows by name and stops at
+# (crates/burn-lm-llama/src/tokenizer/tiktoken.rs:12-15, 126-132)
+SPECIAL_TOKENS = dict(bos="<|begin_of_text|>", eos="<|end_of_text|>",
+                      stops=("<|end_of_text|>", "<|eom_id|>", "<|eot_id|>"))
+
 LLAMA = Architecture(name="LlamaForCausalLM", read_config=LlamaConfig.from_dict, plan=plan,
-                     checkpoint_tensors=checkpoint_tensors, display_name="Llama 3", created_by="Meta")
+                     checkpoint_tensors=checkpoint_tensors, display_name="Llama 3", created_by="Meta",
+                     chat_template=chat_template, special_tokens=SPECIAL_TOKENS)
 register_architecture(LLAMA, "llama")

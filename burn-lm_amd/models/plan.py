@@ -13,14 +13,31 @@ from typing import Dict, List, Optional, Tuple
 from ..parts.base import PartSpec
 
 
-@dataclass(frozen=True)
 class LayerPlan:
-    block: str            # kind of arrangement, e.g. "pre_norm"
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
-    position: Optional[str] = None  # key into ModelPlan.positions, handed to the mixer
+    """One layer: the kind of arrangement (a registered block, e.g. "pre_norm") and the part chosen
+    for each role that this arrangement has.  Which roles there are is the block's business: the
+    pre-norm block has ``mixer``, ``feed_forward``, ``mixer_norm`` and ``ffn_norm``; another block
+    may have four norms, or no feed-forward.  Roles are given as a mapping or by keyword.
+    ``position`` is a key into ModelPlan.positions; that encoding is handed to the layer's mixers."""
+
+    def __init__(self, block: str, parts: Optional[Dict[str, PartSpec]] = None, position: Optional[str] = None,
+                 **roles: PartSpec):
+        self.block = block
+        self.parts: Dict[str, PartSpec] = dict(parts or {})
+        self.parts.update(roles)
+        self.position = position
+        for role, spec in self.parts.items():
+            if not isinstance(spec, PartSpec):
+                raise TypeError(f"layer plan: role {role!r} needs a PartSpec, got {type(spec).__name__}")
+
+    def __getattr__(self, role):        # plan.mixer, plan.feed_forward, ...
+        try:
+            return self.__dict__["parts"][role]
+        except KeyError:
+            raise AttributeError(role) from None
+
+    def __repr__(self):
+        return f"LayerPlan({self.block!r}, {self.parts!r}, position={self.position!r})"
 
 
 @dataclass(frozen=True)

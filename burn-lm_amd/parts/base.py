@@ -22,7 +22,8 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
   ``encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store)``; the attention mixer calls
   ``project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)``, whose default is the
   projection followed by ``encode_and_store`` and which an encoding may fuse.
-* ``Block.forward(h, delta, step, view) -> delta``: runs its parts; the returned delta has not
+* ``Block.roles`` (role -> family of the parts it arranges), ``Block.cache_need()`` and
+  ``Block.forward(h, delta, step, view) -> delta``: runs its parts; the returned delta has not
   been added to ``h`` yet (the next norm adds it, in float32).
 """
 from __future__ import annotations
@@ -118,14 +119,30 @@ class PositionEncoding(Part):
 
 
 class Block:
-    """Arrangement of a layer's parts."""
+    """Arrangement of a layer's parts.  ``roles`` says which roles the arrangement has and of which
+    family each is (the registry's families: mixer, feed_forward, norm); the model builder makes the
+    part a layer plan names for every role and hands the block the mapping role -> part.  The parts
+    are also reachable as attributes (``self.mixer`` ...).  A block whose cache need is not simply
+    that of a role called ``mixer`` overrides ``cache_need``."""
+    roles: Dict[str, str] = {}
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm):
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+    def __init__(self, parts: Dict[str, Part]):
+        missing = [r for r in self.roles if r not in parts]
+        unknown = [r for r in parts if r not in self.roles]
+        if missing or unknown:
+            raise ValueError(f"{type(self).__name__} has the roles {sorted(self.roles)}; the layer plan "
+                             f"lacks {missing} and names unknown {unknown}")
+        self._parts = dict(parts)
+        for role, part in parts.items():
+            setattr(self, role, part)
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+        """In the order the roles are declared (the order in which they are bound)."""
+        return tuple(self._parts[r] for r in self.roles)
+
+    def cache_need(self):
+        mixer = self._parts.get("mixer")
+        return mixer.cache_need() if mixer is not None else None
 
     def forward(self, h, delta, step, view):
         raise NotImplementedError

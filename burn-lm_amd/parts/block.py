@@ -10,6 +10,8 @@ from .base import Block
 
 
 class PreNormBlock(Block):
+    roles = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "feed_forward": "feed_forward"}
+
     def forward(self, h, delta, step, view):
         x = self.mixer_norm.add_norm(h, delta)
         a = self.mixer.forward(x, step, view)

@@ -24,9 +24,12 @@ class Architecture:
     name: str
     read_config: Callable  # dict (config.json) -> typed configuration
     plan: Callable         # (configuration, tensor names in the checkpoint or None) -> ModelPlan
-    checkpoint_tensors: Callable = None  # configuration -> {name: shape} of a fresh checkpoint (random mode)
+    checkpoint_tensors: Callable = None  # configuration -> {name: (shape, initialiser or role)} of a fresh checkpoint
     display_name: str = ""
     created_by: str = ""
+    # text side (used by the server and the command line, never by the engine):
+    chat_template: Callable = None       # list of {"role", "content"} messages -> prompt text; None: contents joined by newlines
+    special_tokens: dict = None          # names in tokenizer.json: {"bos": str, "eos": str, "stops": (str, ...)}
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}

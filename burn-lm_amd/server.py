@@ -144,15 +144,19 @@ class InferenceServer:
     def _tokenizer(self):
         if self.tokenizer is None:
             from .cli.tokenizer import for_folder
-            self.tokenizer = for_folder(self.folder, self.engine.vocab_size)
+            self.tokenizer = for_folder(self.folder, self.engine.vocab_size,
+                                        self.engine.model.architecture.special_tokens)
         return self.tokenizer
 
-    @staticmethod
-    def prompt(messages) -> str:
-        """The chat template of crates/burn-lm-llama/src/server/llama3.rs:561-576."""
-        out = "".join(f"<|start_header_id|>{m['role'].lower()}<|end_header_id|>\n\n{m['content']}<|eot_id|>"
-                      for m in messages)
-        return out + "<|start_header_id|>assistant<|end_header_id|>\n\n"
+    def prompt(self, messages) -> str:
+        """The prompt text of a list of messages: the architecture's chat template (the reference's
+        servers each carry their own, crates/burn-lm-llama/src/server/llama3.rs:561-576); an
+        architecture without one gets the contents joined by newlines."""
+        self.load()
+        template = self.engine.model.architecture.chat_template
+        if template is None:
+            return "\n".join(m["content"] for m in messages)
+        return template(messages)
 
     def run_job(self, task, on_text: Optional[Callable[[str], None]] = None, **options) -> Stats:
         """task: a prompt string, one message ``{"role", "content"}``, or a list of messages

@@ -35,7 +35,7 @@ TINIES = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (MID_C, 2)}
 TOL = {"float32": 1e-5, "bfloat16": 3e-2}
 
 
-def make_folder(path, cfg, seed, std=None, norm_jitter=0.1):
+def make_folder(path, cfg, seed, std=None, norm_jitter=0.1, **kw):
     """Weights N(0, std).  The tiny models take 0.08, so that their logits are far from uniform; at
     width 512 that scale sharpens the attention so much that bfloat16 activations alone (exact
     arithmetic between the roundings, on the CPU) put 1 logit row in 100 at 0.024 of the largest
@@ -43,7 +43,7 @@ def make_folder(path, cfg, seed, std=None, norm_jitter=0.1):
     import burn_lm_amd
     if std is None:
         std = 0.05 if cfg is MID_C else 0.08
-    return burn_lm_amd.write_random_model(str(path), cfg, seed=seed, std=std, norm_jitter=norm_jitter)
+    return burn_lm_amd.write_random_model(str(path), cfg, seed=seed, std=std, norm_jitter=norm_jitter, **kw)
 
 
 def random_tokens(seed, vocab, n):

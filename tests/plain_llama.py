@@ -21,6 +21,55 @@ import numpy as np
 
 
 # ----------------------------------------------------------------------------------------
+# optional rounding: where a bfloat16 engine rounds, so that its tests can be tight
+# ----------------------------------------------------------------------------------------
+def round_bf16(x):
+    """Nearest-even rounding of float64 values to bfloat16 (8 significant bits), returned as float64."""
+    a = np.ascontiguousarray(np.asarray(x, dtype=np.float64).astype(np.float32))
+    u = a.view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32).astype(np.float64).reshape(a.shape)
+
+
+class Rounding:
+    """Where values are rounded to bfloat16 between the exact formulas.  Always: the normalised
+    activations, q and k after the rotation, v, the attention output, the gated product, the final
+    norm's output.  The residual stream and its sums, the statistics of norms and softmax, and all
+    products' sums stay exact.  Options say whether a value is rounded as well, each one flag or
+    one flag per token of the sequence (a token keeps the flags of the step that fed it):
+    ``projections`` (q and k before their rotation), ``gate_up`` (gate and up before the gating),
+    ``attention_delta`` and ``feed_forward_delta`` (the output and the down projection before they
+    are added to the residual stream): an engine rounds there where it runs the steps as separate
+    kernels and not where it fuses them or hands on unrounded partial sums;
+    ``probabilities``: the softmax weights ``exp(score - maximum)`` before they multiply the values
+    and are summed, relative to the row's maximum; or, when keys are visited in pages of
+    ``probability_pages``, relative to the maximum of the pages up to the key's own
+    (``running_maximum``, one page after the other) or of the key's own page alone (every page on
+    its own), the weights then being scaled, exactly, to the row's maximum."""
+
+    def __init__(self, projections=True, gate_up=True, attention_delta=True, feed_forward_delta=True,
+                 probabilities=True, probability_pages=None, running_maximum=True):
+        self.projections, self.gate_up = projections, gate_up
+        self.attention_delta, self.feed_forward_delta = attention_delta, feed_forward_delta
+        self.probabilities, self.probability_pages, self.running_maximum = probabilities, probability_pages, running_maximum
+
+    r = staticmethod(round_bf16)
+
+
+def _r(rounding, x, when=True, token_axis=None):
+    """x rounded if a rounding is given and ``when`` holds; ``when`` may hold one flag per token,
+    x's axis ``token_axis`` then runs over the tokens."""
+    if rounding is None or when is False:
+        return x
+    if when is True:
+        return rounding.r(x)
+    flags = np.asarray(when, dtype=bool)
+    shape = [1] * np.ndim(x)
+    shape[token_axis] = flags.shape[0]
+    return np.where(flags.reshape(shape), rounding.r(x), x)
+
+
+# ----------------------------------------------------------------------------------------
 # parts
 # ----------------------------------------------------------------------------------------
 def rms_norm(x, gamma, eps):
@@ -111,7 +160,7 @@ def softmax(x, axis=-1):
     return e / np.sum(e, axis=axis, keepdims=True)
 
 
-def scaled_attention(q, k, v, mask):
+def scaled_attention(q, k, v, mask, rounding=None):
     """softmax(q k^T / sqrt(hd) + mask) v with the scale applied to the product
     (LL/nn/attention/mha.rs:143-171).  q [B,nh,T,hd]; k, v [B,nkv,S,hd]."""
     n_rep = q.shape[1] // k.shape[1]
@@ -120,10 +169,26 @@ def scaled_attention(q, k, v, mask):
     scores = np.matmul(q, np.swapaxes(k, 2, 3)) / math.sqrt(q.shape[-1])
     if mask is not None:
         scores = np.where(mask[None, None], -np.inf, scores)
-    return np.matmul(softmax(scores, axis=3), v)
+    if rounding is None or rounding.probabilities is False:
+        return np.matmul(softmax(scores, axis=3), v)
+    final = np.max(scores, axis=3, keepdims=True)
+    seen = final
+    if rounding.probability_pages:      # the maximum of the pages up to and including each key's own
+        n = rounding.probability_pages
+        pages = [np.max(scores[..., a:a + n], axis=3, keepdims=True) for a in range(0, scores.shape[3], n)]
+        own = np.concatenate(pages, axis=3)
+        running = np.maximum.accumulate(own, axis=3)
+        if rounding.running_maximum is not True:
+            flags = np.broadcast_to(np.asarray(rounding.running_maximum, dtype=bool), (scores.shape[2],))
+            running = np.where(flags.reshape(1, 1, -1, 1), running, own)
+        seen = np.repeat(running, n, axis=3)[..., :scores.shape[3]]
+        seen = np.where(np.isfinite(seen), seen, final)     # pages of which a query sees nothing
+    e = np.exp(scores - seen)                                   # weights in (0, 1]
+    e = _r(rounding, e, rounding.probabilities, token_axis=2) * np.exp(seen - final)
+    return np.matmul(e, v) / np.sum(e, axis=3, keepdims=True)
 
 
-def attention_layer(x, wq, wk, wv, wo, n_heads, n_kv_heads, head_dim, freqs, start_pos=0):
+def attention_layer(x, wq, wk, wv, wo, n_heads, n_kv_heads, head_dim, freqs, start_pos=0, rounding=None):
     """Whole-sequence attention sub-layer without cache (``forward_masked``,
     LL/nn/attention/mha.rs:50-69; projections :121-140).  x [B,T,D]; weights
     ``[d_out, d_in]`` already in the interleaved pair order."""
@@ -131,42 +196,49 @@ def attention_layer(x, wq, wk, wv, wo, n_heads, n_kv_heads, head_dim, freqs, sta
     q = (x @ wq.T).reshape(b, t, n_heads, head_dim).swapaxes(1, 2)
     k = (x @ wk.T).reshape(b, t, n_kv_heads, head_dim).swapaxes(1, 2)
     v = (x @ wv.T).reshape(b, t, n_kv_heads, head_dim).swapaxes(1, 2)
+    if rounding is not None:
+        q, k = _r(rounding, q, rounding.projections, 2), _r(rounding, k, rounding.projections, 2)
+        v = rounding.r(v)
     pos = np.arange(start_pos, start_pos + t)
-    q = rope_interleaved(q, pos, freqs)
-    k = rope_interleaved(k, pos, freqs)
-    o = scaled_attention(q, k, v, hidden_mask(t, t))
+    q = _r(rounding, rope_interleaved(q, pos, freqs))
+    k = _r(rounding, rope_interleaved(k, pos, freqs))
+    o = _r(rounding, scaled_attention(q, k, v, hidden_mask(t, t), rounding))
     o = o.swapaxes(1, 2).reshape(b, t, n_heads * head_dim)
-    return o @ wo.T
+    return o @ wo.T if rounding is None else _r(rounding, o @ wo.T, rounding.attention_delta, 1)
 
 
 def silu(z):
     return z / (1.0 + np.exp(-z))
 
 
-def swiglu_feed_forward(x, w_gate, w_up, w_down):
+def swiglu_feed_forward(x, w_gate, w_up, w_down, rounding=None):
     """(silu(x W1) * (x W3)) W2 (LL/nn/fftn.rs:44-46; W1 = swiglu.linear_inner = gate,
     W3 = swiglu.linear_outer = up, LL/nn/llama/import.rs:22-31).  Vector at fftn.rs:57-92."""
-    return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+    if rounding is None:
+        return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+    g, u = _r(rounding, x @ w_gate.T, rounding.gate_up, 1), _r(rounding, x @ w_up.T, rounding.gate_up, 1)
+    return _r(rounding, rounding.r(silu(g) * u) @ w_down.T, rounding.feed_forward_delta, 1)
 
 
-def block(x, lw, cfg, freqs, start_pos=0):
+def block(x, lw, cfg, freqs, start_pos=0, rounding=None):
     """h = x + attn(norm1(x)); out = h + ffn(norm2(h)) (LL/nn/transformer.rs:241-256)."""
-    h = x + attention_layer(rms_norm(x, lw["attention_norm"], cfg["eps"]),
+    h = x + attention_layer(_r(rounding, rms_norm(x, lw["attention_norm"], cfg["eps"])),
                             lw["wq"], lw["wk"], lw["wv"], lw["wo"],
-                            cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], freqs, start_pos)
-    return h + swiglu_feed_forward(rms_norm(h, lw["ffn_norm"], cfg["eps"]),
-                                   lw["w1"], lw["w3"], lw["w2"])
+                            cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], freqs, start_pos, rounding)
+    return h + swiglu_feed_forward(_r(rounding, rms_norm(h, lw["ffn_norm"], cfg["eps"])),
+                                   lw["w1"], lw["w3"], lw["w2"], rounding)
 
 
-def transformer_forward(ids, model, start_pos=0):
+def transformer_forward(ids, model, start_pos=0, rounding=None):
     """Embedding -> blocks -> final norm -> output projection, logits for every position
-    (LL/nn/transformer.rs:88-103).  ids [B,T] ints; returns [B,T,V] float64."""
+    (LL/nn/transformer.rs:88-103).  ids [B,T] ints; returns [B,T,V] float64.  With a ``Rounding``
+    the values a bfloat16 engine keeps in bfloat16 are rounded on the way (the formulas stay these)."""
     cfg = model["cfg"]
     ids = np.asarray(ids)
     h = model["tok_embeddings"][ids]
     for lw in model["layers"]:
-        h = block(h, lw, cfg, model["freqs"], start_pos)
-    h = rms_norm(h, model["norm"], cfg["eps"])
+        h = block(h, lw, cfg, model["freqs"], start_pos, rounding)
+    h = _r(rounding, rms_norm(h, model["norm"], cfg["eps"]))
     return h @ model["output"].T
 
 

@@ -134,11 +134,15 @@ def test_tokenizers_for_the_command_line(tmp_path):
     tok.pre_tokenizer = pre_tokenizers.Whitespace()
     tok.add_special_tokens(["<|begin_of_text|>", "<|end_of_text|>", "<|eot_id|>"])
     tok.save(str(tmp_path / "tokenizer.json"))
-    f = for_folder(str(tmp_path), 6)
+    from burn_lm_amd import registry
+    special = registry.architecture("LlamaForCausalLM").special_tokens     # the architecture names them, not the tokenizer
+    f = for_folder(str(tmp_path), 6, special)
     assert isinstance(f, FileTokenizer)
     assert f.encode("hello world") == [0, 1] and f.encode("hello", bos=True, eos=True) == [3, 0, 4]
     assert f.stop_ids() == [4, 5]            # <|eom_id|> is not in this file
     assert f.decode([3, 0, 1, 5]) == "hello world"
+    bare = for_folder(str(tmp_path), 6)      # an architecture that names no special tokens: none begin, end or stop
+    assert bare.stop_ids() == [] and bare.encode("hello", bos=True, eos=True) == [0]
 
 
 def test_decode_attention_split_rule():

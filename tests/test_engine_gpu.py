@@ -65,15 +65,31 @@ def test_first_tokens_of_a_sequence(folders, dtype):
 
 
 def test_a_far_key_among_hundreds_is_found(folders, tmp_path):
-    """One early key is made to stand out for the last query (its embedding row scaled up), so an
-    attention that loses keys far back, or a page of the table, changes the logits visibly."""
+    """One early key is made to stand out for every later query, so an attention that loses keys far
+    back, or a page of the table, changes the logits visibly.  In the first layer one lane of every
+    head's query and key (lane 7, whose rotary pair turns by 0.13 rad over 400 positions) reads one
+    feature of the normalised embedding; that feature is small and positive in every token's
+    embedding and is all there is in the embedding of token 255, whose key therefore scores about
+    e^6 against e^1 for every query."""
     from burn_lm_amd.weights import safetensors_io as st
     cfg, seed = TINIES["A"]
     f = st.open_folder(folders["A"])
     tensors = {n: f[n].tensor(n).clone() for n in f}
+    j, lane, c = 5, 7, 2.0
     emb = tensors["model.embed_tokens.weight"].float()
-    emb[255] *= 4.0
+    emb[:, j] = 0.1
+    emb[255] = 0.0
+    emb[255, j] = 1.0
     tensors["model.embed_tokens.weight"] = emb.bfloat16()
+    for name, heads in (("q_proj", cfg["num_attention_heads"]), ("k_proj", cfg["num_key_value_heads"])):
+        w = tensors[f"model.layers.0.self_attn.{name}.weight"].float()
+        for h in range(heads):
+            w[h * 16 + lane] = 0.0
+            w[h * 16 + lane, j] = c
+        tensors[f"model.layers.0.self_attn.{name}.weight"] = w.bfloat16()
+    g = tensors["model.layers.0.input_layernorm.weight"].float()
+    g[j] = 1.0
+    tensors["model.layers.0.input_layernorm.weight"] = g.bfloat16()
     folder = str(tmp_path / "m")
     os.makedirs(folder)
     st.write_file(os.path.join(folder, "model.safetensors"), tensors.items())
@@ -86,7 +102,7 @@ def test_a_far_key_among_hundreds_is_found(folders, tmp_path):
     without[3] = 7
     moved = P.transformer_forward([without], plain)[0]
     effect = [rel_err(moved[p], want[p]) for p in range(330, 400)]
-    assert sum(e > 0.1 for e in effect) >= 5, "the test's own premise: the far key matters to several late positions"
+    assert sum(e > 0.1 for e in effect) >= 60, "the test's own premise: the far key matters to the late positions"
     for dtype in ("float32", "bfloat16"):
         eng = load(folder, dtype)
         s = eng.open()
@@ -246,7 +262,8 @@ def test_prompt_steps_replayed_from_graphs(folders, name, dtype):
     plain = P.load_model_folder(folders[name])
     eng = load(folders[name], dtype, max_tokens=4096)
     V = cfg["vocab_size"]
-    batches = [[40, 7, 90], [64, 1, 20, 33], [100, 3], [5, 5, 5, 120], [130], [61, 2, 70, 1], [150, 30], [128]]
+    batches = [[40, 7, 90], [64, 1, 20, 33], [100, 3], [5, 5, 5, 120], [130], [61, 2, 70, 1], [150, 30], [128],
+               [44, 9, 85], [60, 3, 66, 2], [129], [2, 50, 77]]      # a shape is recorded when it is met the second time
     seen_replay = 0
     for bi, lens in enumerate(batches):
         prompts = [random_tokens(1000 + 10 * bi + i, V, n + 3) for i, n in enumerate(lens)]
@@ -271,7 +288,7 @@ def test_prompt_steps_replayed_from_graphs(folders, name, dtype):
             eng.close(s)
     assert eng.cache.pages_in_use() == 0
     prompt_shapes = [k for k in eng.graphs.captured if k[1] > 0]
-    # whole prompts replayed (batches 3 and 5 have the shape of batch 0), and the second chunks
+    # whole prompts replayed (several batches have the shape of batch 0), and the second chunks
     assert seen_replay >= 2 and len(prompt_shapes) >= 4 and eng.graphs.replays >= 8, (seen_replay, sorted(eng.graphs.captured))
 
 
@@ -655,19 +672,29 @@ def test_random_schedules_through_recorded_graphs(folders, name, dtype, seed):
 
 
 
-def test_the_benchmark_layer_shape_against_the_plain_implementation(tmp_path):
-    """Two layers of the Llama-3.2-1B shape (width 2048, 32 heads in 8 groups, feed-forward 8192,
-    vocabulary 128,256, tied head, the published frequency scaling): the sizes at which the
-    products' policies choose differently than at the small configurations (K-groups, the fused
-    gate/up product in whole rounds of tiles, the head over the whole vocabulary).  Prompts of
-    2,048, 700 and 76 tokens alone and in one batch, then twelve tokens one by one, in both dtypes."""
+@pytest.mark.parametrize("name,layers,vocab", [("llama3.2-1b", 2, None), ("llama3.2-3b", 1, 20008), ("llama3.1-8b", 1, 20008)])
+def test_the_benchmark_layer_shapes_against_the_plain_implementation(tmp_path, name, layers, vocab):
+    """Layers of the shapes that the measurements are quoted on, at which the products' policies choose
+    differently than at the small configurations.  Llama-3.2-1B (two layers, whole vocabulary of
+    128,256, tied head): width 2048, 32 heads in 8 groups, feed-forward 8192: K-groups, the fused
+    gate/up product in whole rounds of tiles, the head over the whole vocabulary.  Llama-3.2-3B: width
+    3072, 24 heads of size 128 in groups of 3.  Llama-3.1-8B: width 4096, feed-forward 14336, separate
+    head: long K in the down projection, the library's products above 32 rows.  (The two wide shapes
+    with one layer and a vocabulary of 20,008, which is no multiple of 16: their layers are what
+    differs.)  Prompts of 2,048, 700 and 76 tokens alone and in one batch, then twelve tokens one by
+    one at batch 1 and 3; then the three among 37 shorter prompts, a batch of 40, and twelve tokens
+    each; in both dtypes."""
     from burn_lm_amd.config.presets import preset
-    cfg = dict(preset("llama3.2-1b"))
-    cfg["num_hidden_layers"] = 2
+    cfg = dict(preset(name))
+    cfg["num_hidden_layers"] = layers
+    if vocab:
+        cfg["vocab_size"] = vocab
+        cfg.pop("eos_token_id", None), cfg.pop("bos_token_id", None)     # they lie beyond the smaller vocabulary
     folder = make_folder(tmp_path / "shape", cfg, seed=3, std=0.02)
     plain = P.load_model_folder(folder)
     n_dec = 12
-    reqs = [random_tokens(40 + i, cfg["vocab_size"], n + n_dec) for i, n in enumerate([2048, 700, 76])]
+    lengths = [2048, 700, 76] + [1 + (29 * i) % 150 for i in range(37)]
+    reqs = [random_tokens(40 + i, cfg["vocab_size"], n + n_dec) for i, n in enumerate(lengths)]
 
     def plain_rows(toks, rows):   # the plain blocks, with the head on the wanted rows only
         h = plain["tok_embeddings"][np.asarray([toks])]
@@ -680,21 +707,22 @@ def test_the_benchmark_layer_shape_against_the_plain_implementation(tmp_path):
         cut = len(r) - n_dec
         want.append(plain_rows(r, [0, cut // 2, cut - 1] + list(range(cut, len(r)))))
     for dtype, tol in (("float32", 1e-5), ("bfloat16", TOL["bfloat16"])):
-        eng = load(folder, dtype, max_tokens=4096, max_seqs=4)
-        for group in ([0], [1], [2], [0, 1, 2]):
+        eng = load(folder, dtype, max_tokens=2176 + 832 + 128 + 37 * 192, max_seqs=40)
+        for group in ([0], [1], [2], [0, 1, 2], list(range(40))):
             slots = {i: eng.open() for i in group}
             cut = {i: len(reqs[i]) - n_dec for i in group}
             got = eng.step([(slots[i], reqs[i][:cut[i]], [0, cut[i] // 2, cut[i] - 1]) for i in group]).double().cpu().numpy()
             for k, i in enumerate(group):
                 for j in range(3):
-                    assert rel_err(got[3 * k + j], want[i][j]) <= tol, f"{dtype} {group}: request {i}, prompt row {j}"
+                    assert rel_err(got[3 * k + j], want[i][j]) <= tol, f"{dtype} batch of {len(group)}: request {i}, prompt row {j}"
             for s in range(n_dec):
                 got = eng.step([(slots[i], [reqs[i][cut[i] + s]], [0]) for i in group]).double().cpu().numpy()
                 for k, i in enumerate(group):
-                    assert rel_err(got[k], want[i][3 + s]) <= tol, f"{dtype} {group}: request {i}, decode step {s}"
+                    assert rel_err(got[k], want[i][3 + s]) <= tol, f"{dtype} batch of {len(group)}: request {i}, decode step {s}"
             for i in group:
                 eng.close(slots[i])
         del eng
+        torch.cuda.empty_cache()
 
 
 def test_wanted_places_come_back_in_the_order_given(folders):
@@ -710,3 +738,119 @@ def test_wanted_places_come_back_in_the_order_given(folders):
     assert got.shape[0] == 6
     for row, want in zip(got, [wa[7], wa[0], wa[7], wa[3], wb[4], wb[1]]):
         assert rel_err(row, want) <= TOL["float32"]
+
+
+def test_checkpoints_stored_in_32_bit_and_in_float16(tmp_path, capsys):
+    """The same random model stored as float32, as bfloat16 and as float16.  A tensor stored in 32 bits
+    stays in 32 bits in a bfloat16 run (its products then run on the float kernels, and a note says so),
+    unless the loader is asked to round matrices to the run's type, which gives the very engine of the
+    bfloat16 folder.  Float16 is rounded to bfloat16 (three bits of each weight): the run then equals
+    the plain implementation *of the rounded weights* within the usual tolerance, and the stored ones
+    within 6 % of the largest logit; a float32 run of it is exact."""
+    cfg, seed = TINIES["C"]
+    toks = random_tokens(900, cfg["vocab_size"], 150)
+    f32 = make_folder(tmp_path / "f32", cfg, seed, dtype=torch.float32)
+    b16 = make_folder(tmp_path / "b16", cfg, seed, dtype=torch.bfloat16)
+    f16 = make_folder(tmp_path / "f16", cfg, seed, dtype=torch.float16)
+
+    def run(folder, dtype, **kw):
+        eng = load(folder, dtype, **kw)
+        s = eng.open()
+        whole = eng.step([(s, toks[:140], list(range(140)))]).double().cpu().numpy()
+        tail = [eng.step([(s, [t], [0])]).double().cpu().numpy()[0] for t in toks[140:]]
+        return eng, np.concatenate([whole, np.stack(tail)])
+
+    # stored in 32 bits, bfloat16 run: the matrices stay float32, and the run says so
+    want32 = P.transformer_forward([toks], P.load_model_folder(f32))[0]
+    capsys.readouterr()
+    eng, got = run(f32, "bfloat16")
+    note = capsys.readouterr().err
+    assert "stored in 32 bits" in note and "cast_32bit" in note
+    assert eng.model.blocks[0].mixer.w_qkv.dtype == torch.float32 and eng.model.blocks[0].mixer.w_qkv.packed is None
+    assert max(rel_err(got[p], want32[p]) for p in range(150)) <= TOL["bfloat16"]
+    # the same folder with its matrices rounded when they are loaded: the packed products, and the
+    # bfloat16 folder's logits to the bit (the weights are the same bytes then; norm weights stay wide)
+    eng_c, got_c = run(f32, "bfloat16", cast_32bit=True)
+    assert eng_c.model.blocks[0].mixer.w_qkv.dtype == torch.bfloat16 and eng_c.model.blocks[0].mixer.w_qkv.packed is not None
+    assert eng_c.model.blocks[0].mixer_norm.gamma.dtype == torch.float32
+    plain16 = P.load_model_folder(b16)
+    want16 = P.transformer_forward([toks], plain16)[0]
+    assert max(rel_err(got_c[p], want16[p]) for p in range(150)) <= TOL["bfloat16"]
+    # float32 run of the float32 folder
+    _, got = run(f32, "float32")
+    assert max(rel_err(got[p], want32[p]) for p in range(150)) <= TOL["float32"]
+    # float16: exact in a float32 run; rounded to bfloat16 in a bfloat16 run
+    plain_h = P.load_model_folder(f16)
+    want_h = P.transformer_forward([toks], plain_h)[0]
+    _, got = run(f16, "float32")
+    assert max(rel_err(got[p], want_h[p]) for p in range(150)) <= TOL["float32"]
+    rounded = dict(plain_h, tok_embeddings=P.round_bf16(plain_h["tok_embeddings"]), norm=P.round_bf16(plain_h["norm"]),
+                   layers=[{k: P.round_bf16(v) for k, v in lw.items()} for lw in plain_h["layers"]])
+    rounded["output"] = rounded["tok_embeddings"]     # config C ties its head
+    want_r = P.transformer_forward([toks], rounded)[0]
+    eng_h, got = run(f16, "bfloat16")
+    assert eng_h.model.blocks[0].mixer.w_qkv.dtype == torch.bfloat16
+    assert max(rel_err(got[p], want_r[p]) for p in range(150)) <= TOL["bfloat16"]
+    assert max(rel_err(got[p], want_h[p]) for p in range(150)) <= 6e-2
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_generation_that_runs_ahead_of_the_host_in_bfloat16(folders, name):
+    """The generation loop keeps the picked tokens on the GPU and starts the next step from them
+    before the host has seen them (step_ahead and pick_device, from recorded graphs).  In bfloat16, on
+    the matrix-core paths, it must give the tokens of the plain loop that reads every token first
+    (an engine shown without step_ahead), and the logits behind the first tokens must be the plain
+    implementation's within the tolerance."""
+    from burn_lm_amd.engine.generate import generate
+    from burn_lm_amd.sampling.sampler import Sampler
+    cfg, seed = TINIES[name]
+    eng = load(folders[name], "bfloat16", max_tokens=4096, max_seqs=8)
+    prompts = [random_tokens(700 + i, cfg["vocab_size"], n) for i, n in enumerate([5, 70, 17, 1, 33, 130, 9])]
+
+    class Plain:      # the same engine without the run-ahead entry: the loop then waits for every token
+        def __init__(self, e):
+            self.open, self.close, self.step, self.length = e.open, e.close, e.step, e.length
+            self.max_context, self.cache = e.max_context, e.cache
+
+    stop = 3
+    for temperature, top_p in ((0.0, 1.0), (0.7, 0.9)):
+        for _ in range(2):          # the second round replays what the first recorded
+            ahead, stats = generate(eng, prompts, Sampler(temperature, top_p, seed=5), 24, stop_ids=[stop], batch_size=4)
+            waited, _ = generate(Plain(eng), prompts, Sampler(temperature, top_p, seed=5), 24, stop_ids=[stop], batch_size=4)
+            assert [r.tokens for r in ahead] == [r.tokens for r in waited]
+            assert [r.finish_reason for r in ahead] == [r.finish_reason for r in waited]
+    assert eng.graphs.replays > 40 and eng.cache.pages_in_use() == 0
+    # the logits behind the first generated token of each request, against the plain implementation
+    plain = P.load_model_folder(folders[name])
+    for p in prompts:
+        s = eng.open()
+        got = eng.step([(s, p, [len(p) - 1])]).double().cpu().numpy()[0]
+        eng.close(s)
+        assert rel_err(got, P.transformer_forward([p], plain)[0, -1]) <= TOL["bfloat16"]
+
+
+def test_recorded_shapes_are_limited_and_the_oldest_goes(folders, monkeypatch):
+    """A shape is recorded at its second sight; with room for two recorded shapes a third one evicts
+    the shape replayed longest ago, and every step still gives the plain logits."""
+    from burn_lm_amd.engine import graphs
+    monkeypatch.setattr(graphs, "MAX_GRAPHS", 2)
+    cfg, seed = TINIES["A"]
+    plain = P.load_model_folder(folders["A"])
+    eng = load(folders["A"], "float32", max_tokens=4096, max_seqs=16)
+    seqs = [random_tokens(990 + i, cfg["vocab_size"], 30) for i in range(9)]
+    want = [P.transformer_forward([t], plain)[0] for t in seqs]
+    slots = [eng.open() for _ in seqs]
+    eng.step([(s, t[:4], []) for s, t in zip(slots, seqs)])
+    recorded_after = {}
+    for p in range(4, 30):
+        n = (1, 2, 3, 5, 9)[(p // 5) % 5]         # live sequences this step: buckets 1, 2, 4, 8, 16
+        live = list(range(9)) if p % 5 == 0 else list(range(n))
+        # every sequence must advance together, so the idle ones take the same step in a second call
+        got = eng.step([(slots[i], [seqs[i][p]], [0]) for i in live]).double().cpu().numpy()
+        for k, i in enumerate(live):
+            assert rel_err(got[k], want[i][p]) <= TOL["float32"], (p, i)
+        rest = [i for i in range(9) if i not in live]
+        if rest:
+            eng.step([(slots[i], [seqs[i][p]], []) for i in rest])
+        recorded_after[p] = len(eng.graphs.captured)
+    assert max(recorded_after.values()) <= 2 and eng.graphs.evicted >= 1 and eng.graphs.replays >= 4

@@ -184,7 +184,7 @@ def test_pre_norm_block(rt):
              registry.part("norm", "rmsnorm")(dict(width=D, eps=1e-5), dict(weight="n2"))]
     for p in parts:
         p.bind(on_gpu(t), rt)
-    block = registry.part("block", "pre_norm")(*parts)
+    block = registry.part("block", "pre_norm")(dict(mixer=parts[0], feed_forward=parts[1], mixer_norm=parts[2], ffn_norm=parts[3]))
     cache = Cache([parts[0].cache_need()], [None], 256, 2, 64, rt.page_size, rt.dtype, rt.device)
     s = cache.open()
     cache.reserve([(s, 19)])

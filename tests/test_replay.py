@@ -96,3 +96,63 @@ def test_cache_is_sized_by_max_tokens(case, tmp_path):
     assert out[0].shape[0] == 2
     with pytest.raises(AssertionError, match="pages"):
         run_trace(folder, "float32", tr, tmp_path / "short", max_tokens=128)
+
+
+# ---- many concurrent requests ------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def crowd(tmp_path_factory):
+    """Config C and 70 requests of unequal lengths with the plain logits of every position that a
+    crowd trace asks for (the last four places of each prefix and every decoded token)."""
+    cfg, seed = TINIES["C"]
+    folder = make_folder(tmp_path_factory.mktemp("crowdC"), cfg, seed)
+    plain = P.load_model_folder(folder)
+    lengths = [3 + (37 * i + 11 * (i % 7)) % 118 for i in range(70)]
+    reqs = {f"c{i}": random_tokens(5000 + i, cfg["vocab_size"], n) for i, n in enumerate(lengths)}
+    want = {rid: P.transformer_forward([t], plain)[0] for rid, t in reqs.items()}
+    return folder, reqs, want
+
+
+def crowd_trace(reqs):
+    """Batches of 20, 40 and 70 requests that start together, each batch run twice with other shares
+    of prefilled and decoded tokens, one batch after another on a cache that holds one batch: the
+    decode steps have 17 to 64 and more than 64 live sequences until the shorter ones have ended."""
+    tr = Trace()
+    ids = list(reqs)
+    for n, first in ((20, 0), (40, 20), (70, 0)):
+        for turn in (0, 1):
+            batch = ids[first:first + n]
+            entries, left = [], {}
+            for k, rid in enumerate(batch):
+                toks = reqs[rid]
+                d = min(len(toks) - 1, (5 * k + 3 * turn) % 14 + (3 if n == 70 else 0))   # tokens decoded one by one
+                p = len(toks) - d
+                entries.append((rid, 0, toks[:p], list(range(max(0, p - 4), p))))
+                left[rid] = p
+            tr.step(entries, end=[rid for rid, p in left.items() if p == len(reqs[rid])])
+            left = {rid: p for rid, p in left.items() if p < len(reqs[rid])}
+            while left:
+                entries = [(rid, p, [reqs[rid][p]], [0]) for rid, p in left.items()]
+                ending = [rid for rid, p in left.items() if p + 1 == len(reqs[rid])]
+                tr.step(entries, end=ending)
+                left = {rid: p + 1 for rid, p in left.items() if rid not in ending}
+    return tr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_of_twenty_forty_and_seventy_concurrent_requests(crowd, dtype, tmp_path):
+    folder, reqs, want = crowd
+    tr = crowd_trace(reqs)
+    out = run_trace(folder, dtype, tr, tmp_path / "out")
+    worst, rows_checked, widest = 0.0, 0, 0
+    for step, rows in tr.index.items():
+        got = out[step]
+        widest = max(widest, len({rid for rid, _ in rows}))
+        for k, (rid, pos) in enumerate(rows):
+            e = rel_err(got[k], want[rid][pos])
+            worst = max(worst, e)
+            rows_checked += 1
+            assert e <= TOL[dtype], (f"{dtype}: request {rid} position {pos} of {len(reqs[rid])} (step {step}, "
+                                     f"{len(rows)} rows) differs by {e:.3g} of the largest logit")
+    assert widest == 70 and rows_checked > 2000
+    print(f"crowd {dtype}: {rows_checked} rows, worst relative error {worst:.3g}")

@@ -64,9 +64,10 @@ def register_toy():
         attn = PartSpec("attention", dict(width=D, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim,
                                           scale=1 / math.sqrt(cfg.head_dim)),
                         dict(q="l0.q", k="l0.k", v="l0.v", o="l0.o"))
-        layers = [LayerPlan("pre_norm", attn, ffn(0), norm("l0.n1"), norm("l0.n2"), position="rope"),
-                  LayerPlan("pre_norm", PartSpec("toy_decay", dict(width=D, decay=cfg.decay), dict(w="l1.w")),
-                            ffn(1), norm("l1.n1"), norm("l1.n2"))]
+        layers = [LayerPlan("pre_norm", mixer=attn, feed_forward=ffn(0), mixer_norm=norm("l0.n1"), ffn_norm=norm("l0.n2"),
+                            position="rope"),
+                  LayerPlan("pre_norm", mixer=PartSpec("toy_decay", dict(width=D, decay=cfg.decay), dict(w="l1.w")),
+                            feed_forward=ffn(1), mixer_norm=norm("l1.n1"), ffn_norm=norm("l1.n2"))]
         return ModelPlan(vocab_size=cfg.vocab, width=D, max_positions=cfg.max_positions,
                          embedding=PartSpec("table", dict(vocab=cfg.vocab, width=D), dict(weight="emb")),
                          layers=layers, order=[Place(0), Place(1), Place(0, reads_cache_of=0)],
@@ -190,11 +191,12 @@ def test_a_windowed_attention_layer_beside_a_full_one(tmp_path):
         norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=cfg["eps"]), dict(weight=n))
         layer = lambda i, window: LayerPlan(
             "pre_norm",
-            PartSpec("attention", dict(width=D, heads=cfg["heads"], kv_heads=cfg["kv_heads"], head_dim=cfg["head_dim"],
-                                       scale=1 / _m.sqrt(cfg["head_dim"]), window=window),
-                     dict(q=f"l{i}.q", k=f"l{i}.k", v=f"l{i}.v", o=f"l{i}.o")),
-            PartSpec("swiglu", dict(width=D, inner=cfg["inner"]), dict(gate=f"l{i}.gate", up=f"l{i}.up", down=f"l{i}.down")),
-            norm(f"l{i}.n1"), norm(f"l{i}.n2"), position="rope")
+            mixer=PartSpec("attention", dict(width=D, heads=cfg["heads"], kv_heads=cfg["kv_heads"], head_dim=cfg["head_dim"],
+                                             scale=1 / _m.sqrt(cfg["head_dim"]), window=window),
+                           dict(q=f"l{i}.q", k=f"l{i}.k", v=f"l{i}.v", o=f"l{i}.o")),
+            feed_forward=PartSpec("swiglu", dict(width=D, inner=cfg["inner"]),
+                                  dict(gate=f"l{i}.gate", up=f"l{i}.up", down=f"l{i}.down")),
+            mixer_norm=norm(f"l{i}.n1"), ffn_norm=norm(f"l{i}.n2"), position="rope")
         return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
                          embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
                          layers=[layer(0, W), layer(1, 0)], order=[Place(0), Place(1)], final_norm=norm("norm"),

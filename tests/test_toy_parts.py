@@ -88,12 +88,14 @@ def register_toy():
         for e in range(cfg["experts"]):
             routed_names.update({f"gate{e}": f"l1.e{e}.gate", f"up{e}": f"l1.e{e}.up", f"down{e}": f"l1.e{e}.down"})
         layers = [
-            LayerPlan("pre_norm", attn(0), PartSpec("swiglu", dict(width=D, inner=cfg["inner"]),
-                                                    dict(gate="l0.gate", up="l0.up", down="l0.down")),
-                      norm("l0.n1"), norm("l0.n2"), position="rope"),
-            LayerPlan("pre_norm", attn(1), PartSpec("toy_routed", dict(width=D, inner=cfg["expert_inner"],
-                                                                      experts=cfg["experts"]), routed_names),
-                      norm("l1.n1"), norm("l1.n2"), position="fade")]
+            LayerPlan("pre_norm", mixer=attn(0),
+                      feed_forward=PartSpec("swiglu", dict(width=D, inner=cfg["inner"]),
+                                            dict(gate="l0.gate", up="l0.up", down="l0.down")),
+                      mixer_norm=norm("l0.n1"), ffn_norm=norm("l0.n2"), position="rope"),
+            LayerPlan("pre_norm", mixer=attn(1),
+                      feed_forward=PartSpec("toy_routed", dict(width=D, inner=cfg["expert_inner"],
+                                                               experts=cfg["experts"]), routed_names),
+                      mixer_norm=norm("l1.n1"), ffn_norm=norm("l1.n2"), position="fade")]
         return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
                          embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
                          layers=layers, order=[Place(0), Place(1)], final_norm=norm("norm"),
