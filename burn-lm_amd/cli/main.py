@@ -46,8 +46,15 @@ def build_parser():
     r.add_argument("model")
     add_cli_flags(r)
     r.add_argument("--no-stats", action="store_true", help="Disable display of statistics at the end of the inference")
-    r.add_argument("--tokens", action="store_true", help="The prompt is a comma-separated list of token ids")
-    r.add_argument("prompt", help="The prompt to send to the model")
+    r.add_argument("--tokens", action="store_true", help="Every prompt is a comma-separated list of token ids")
+    r.add_argument("--batch", type=int, default=None, metavar="N",
+                   help="Sequences that run together (default: as many as there are prompts, at most 64); "
+                        "more prompts than that run batch after batch")
+    r.add_argument("--prompts-file", default=None, metavar="FILE", help="More prompts, one a line")
+    r.add_argument("--cast-32bit", action="store_true",
+                   help="Round matrices that the checkpoint stores in 32 bits to the element type when loading")
+    r.add_argument("prompt", nargs="*", help="The prompt to send to the model; several prompts run as one batch "
+                                             "of unequal lengths, and one line per request is printed")
     c = sub.add_parser("chat", help="Start a chat session with the chosen model")
     c.add_argument("model")
     add_cli_flags(c)
@@ -110,24 +117,42 @@ def cmd_delete(args):
 
 
 def cmd_run(args):
-    server = InferenceServer(resolve_model(args.model), dtype=args.dtype, batch_size=1)
+    """``run <model> [flags] <prompt>`` (crates/burn-lm-cli/src/commands/run.rs:7-97: load, generate,
+    print the text as it comes, then the stats table).  Several prompts (more arguments, or the lines
+    of --prompts-file) run as batches of unequal lengths; each request then gets a line of its own."""
+    prompts = list(args.prompt)
+    if args.prompts_file:
+        with open(args.prompts_file) as f:
+            prompts += [line.rstrip("\n") for line in f if line.strip()]
+    if not prompts:
+        raise SystemExit("run: give a prompt (or several, or --prompts-file)")
+    batch = args.batch or min(len(prompts), 64)
+    if batch < 1:
+        raise SystemExit("run: --batch must be at least 1")
+    server = InferenceServer(resolve_model(args.model), dtype=args.dtype, batch_size=batch, cast_32bit=args.cast_32bit)
     server.parse_cli_config(args)
     print(f"loading model '{server.model_name()}'...", file=sys.stderr)
     server.load()
     print("model loaded!", file=sys.stderr)
     if args.tokens:
-        ids = [int(t) for t in args.prompt.replace(",", " ").split()]
-        results, stats = server.generate([ids])
-        stats.model_loading_seconds = server._load_seconds
-        r = results[0]
-        if r.finish_reason == "error":
-            raise SystemExit(r.error)
-        print(",".join(str(t) for t in r.tokens))
-    else:
-        stats = server.run_job({"role": "user", "content": args.prompt},
+        try:
+            ids = [[int(t) for t in p.replace(",", " ").split()] for p in prompts]
+        except ValueError as e:
+            raise SystemExit(f"run --tokens: a prompt is no list of token ids ({e})") from None
+        results, stats = server.generate(ids)
+        for r in results:
+            if r.finish_reason == "error" and len(results) == 1:
+                raise SystemExit(r.error)
+            print(",".join(str(t) for t in r.tokens) if r.finish_reason != "error" else f"error: {r.error}")
+    elif len(prompts) == 1:
+        stats = server.run_job({"role": "user", "content": prompts[0]},
                                on_text=lambda s: (sys.stdout.write(s), sys.stdout.flush()))
-        stats.model_loading_seconds = server._load_seconds
         print()
+    else:
+        texts, stats = server.run_jobs([{"role": "user", "content": p} for p in prompts])
+        for i, t in enumerate(texts):
+            print(f"[{i}] {t}")
+    stats.model_loading_seconds = server._load_seconds
     if not args.no_stats:
         print(stats.display_stats())
     server.unload()
@@ -190,7 +215,7 @@ def cmd_shell(dtype):
         if line in ("exit", "quit"):
             break
         try:
-            args = parser.parse_args(["-d", dtype] + shlex.split(line))
+            args = parse(parser, ["-d", dtype] + shlex.split(line))
             if args.command in (None, "shell"):
                 parser.print_help()
             else:
@@ -217,8 +242,19 @@ def dispatch(args):
         cmd_delete(args)
 
 
+def parse(parser, argv):
+    """argparse gives a sub-command's list of positionals only what stands in front of its first
+    flag; prompts that come after flags are picked up here."""
+    args, rest = parser.parse_known_args(argv)
+    if rest:
+        if args.command != "run" or any(r.startswith("-") for r in rest):
+            parser.error("unrecognized arguments: " + " ".join(rest))
+        args.prompt = list(args.prompt) + rest
+    return args
+
+
 def main(argv=None):
-    args = build_parser().parse_args(argv)
+    args = parse(build_parser(), argv)
     if args.backend != BACKEND:
         raise SystemExit(f"backend {args.backend!r} is not available; this build has {BACKEND} only")
     args.dtype = {"bf16": "bf16", "bfloat16": "bf16", "f32": "f32", "float32": "f32"}[args.dtype]

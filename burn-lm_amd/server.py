@@ -67,8 +67,10 @@ class InferenceServer:
     """One model folder behind the reference's server interface."""
 
     def __init__(self, folder: str, dtype: str = "bfloat16", config: Optional[ServerConfig] = None,
-                 batch_size: int = 8, device: str = "cuda:0", model_name: Optional[str] = None):
+                 batch_size: int = 8, device: str = "cuda:0", model_name: Optional[str] = None,
+                 cast_32bit: bool = False):
         self.folder, self.dtype, self.device = folder, dtype, device
+        self.cast_32bit = cast_32bit
         self.config = config or ServerConfig()
         self.batch_size = batch_size
         self.engine = None
@@ -101,7 +103,8 @@ class InferenceServer:
         _, cfg = read_config(self.folder)
         ctx = min(self.config.max_seq_len, cfg.max_position_embeddings)
         self.engine = load_engine(self.folder, dtype=self.dtype, max_tokens=ctx * self.batch_size,
-                                  max_seqs=self.batch_size, max_context=ctx, device=self.device)
+                                  max_seqs=self.batch_size, max_context=ctx, device=self.device,
+                                  cast_32bit=self.cast_32bit)
         st = Stats()
         st.model_loading_seconds = time.perf_counter() - t0
         self._load_seconds = st.model_loading_seconds
@@ -158,16 +161,29 @@ class InferenceServer:
             return "\n".join(m["content"] for m in messages)
         return template(messages)
 
+    def _text_of(self, task) -> str:
+        if isinstance(task, str):
+            return task
+        return self.prompt([task] if isinstance(task, dict) else list(task))
+
+    def run_jobs(self, tasks, **options):
+        """Several tasks (each as for run_job) as batches of unequal lengths -> (texts, Stats); a
+        request that cannot run (longer than the context) gives its error as its text."""
+        self.load()
+        tok = self._tokenizer()
+        ids = [tok.encode(self._text_of(t), False, False) for t in tasks]
+        stop = set(self.stop_ids())
+        results, stats = self.generate(ids, **options)
+        texts = [f"error: {r.error}" if r.finish_reason == "error" else tok.decode([t for t in r.tokens if t not in stop])
+                 for r in results]
+        self.last_generations = results
+        return texts, stats
+
     def run_job(self, task, on_text: Optional[Callable[[str], None]] = None, **options) -> Stats:
         """task: a prompt string, one message ``{"role", "content"}``, or a list of messages
         (InferenceTask::Prompt / Message / Context, crates/burn-lm-inference/src/job.rs:15-50)."""
         first = self.load()
-        if isinstance(task, str):
-            text = task
-        elif isinstance(task, dict):
-            text = self.prompt([task])
-        else:
-            text = self.prompt(list(task))
+        text = self._text_of(task)
         tok = self._tokenizer()
         ids = tok.encode(text, False, False)  # no BOS/EOS added (nn/llama/inference.rs:35-40)
         stop = set(self.stop_ids())

@@ -208,6 +208,16 @@ def test_command_line_runs_a_prompt(folders, capsys):
     assert "##### BurnLM Stats" in out and "Tokens Per Second" in out
     main(["run", folders["A"], "--sample-len", "4", "--temperature", "0.7", "--seed", "3", "--no-stats", "hi"])
     assert "BurnLM Stats" not in capsys.readouterr().out
+    # several prompts of unequal lengths: batches of two, one line per request, in the order given
+    prompts = [[5, 17, 3], [9], [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11], [200, 100]]
+    (tmp := os.path.join(folders["A"], "more.txt")) and open(tmp, "w").write("200 100\n")
+    main(["-d", "f32", "run", folders["A"], "--sample-len", "5", "--tokens", "--batch", "2", "--no-stats", "--prompts-file", tmp]
+         + [",".join(str(t) for t in p) for p in prompts[:3]])
+    lines = [l for l in capsys.readouterr().out.splitlines() if l and l[0].isdigit()]
+    assert lines == [",".join(str(t) for t in P.greedy_generate(plain, p, 5)) for p in prompts]
+    main(["run", folders["A"], "--sample-len", "3", "--no-stats", "hi", "a longer prompt"])
+    out = capsys.readouterr().out
+    assert "[0] " in out and "[1] " in out
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -435,18 +445,9 @@ def _write_folder(path, cfg, tensors):
 def test_the_references_whole_model_vector_in_32_bit(tmp_path):
     """crates/burn-lm-llama/src/nn/transformer.rs:299-349: vocabulary 8, 2 layers, width 8, inner 16,
     2 heads on 1 KV head (head_dim 4), every tensor arange(n)*5/n in the reference's [d_in, d_out]
-    order, token ids [[0, 1], [2, 3]].  The engine reads the same numbers as a Meta-named 32-bit
-    checkpoint ([d_out, d_in], so each matrix transposed) and must give the reference's logits."""
-    r = lambda *s: torch.arange(int(np.prod(s)), dtype=torch.float64).mul(5.0 / int(np.prod(s))).reshape(*s)
-    lin = lambda d_in, d_out: r(d_in, d_out).T.contiguous().float()
-    t = {"tok_embeddings.weight": r(8, 8).float(), "norm.weight": r(8).float(), "output.weight": lin(8, 8)}
-    for i in range(2):
-        p = f"layers.{i}."
-        t.update({p + "attention.wq.weight": lin(8, 8), p + "attention.wk.weight": lin(8, 4),
-                  p + "attention.wv.weight": lin(8, 4), p + "attention.wo.weight": lin(8, 8),
-                  p + "feed_forward.w1.weight": lin(8, 16), p + "feed_forward.w3.weight": lin(8, 16),
-                  p + "feed_forward.w2.weight": lin(16, 8), p + "attention_norm.weight": r(8).float(),
-                  p + "ffn_norm.weight": r(8).float()})
+    order (the Range initialiser of the random-weights mode, whose tensors tests/test_weights.py checks),
+    token ids [[0, 1], [2, 3]].  The engine reads them as a Meta-named 32-bit checkpoint and must give
+    the reference's logits."""
     cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=8, intermediate_size=16, num_hidden_layers=2,
                num_attention_heads=2, num_key_value_heads=1, vocab_size=8, rms_norm_eps=1e-5, rope_theta=10000.0,
                tie_word_embeddings=False, max_position_embeddings=64)
@@ -454,7 +455,10 @@ def test_the_references_whole_model_vector_in_32_bit(tmp_path):
                       [56.374626, 57.77171, 59.168793, 60.56588, 61.962963, 63.360046, 64.75713, 66.15422]],
                      [[56.374252, 57.771328, 59.168407, 60.565487, 61.962566, 63.359642, 64.75672, 66.1538],
                       [56.37408, 57.771156, 59.168232, 60.565304, 61.96238, 63.359455, 64.75653, 66.15361]]])
-    eng = load(_write_folder(tmp_path / "ref", cfg, t), "float32")
+    import burn_lm_amd
+    from burn_lm_amd.weights.random_init import Range
+    folder = burn_lm_amd.write_random_model(str(tmp_path / "ref"), cfg, init=Range(0.0, 5.0), names="meta", dtype=torch.float32)
+    eng = load(folder, "float32")
     a, b = eng.open(), eng.open()
     got = eng.step([(a, [0, 1], [0, 1]), (b, [2, 3], [0, 1])]).double().cpu().numpy().reshape(2, 2, 8)
     np.testing.assert_allclose(got, want, rtol=2e-6)
@@ -854,3 +858,26 @@ def test_recorded_shapes_are_limited_and_the_oldest_goes(folders, monkeypatch):
             eng.step([(slots[i], [seqs[i][p]], []) for i in rest])
         recorded_after[p] = len(eng.graphs.captured)
     assert max(recorded_after.values()) <= 2 and eng.graphs.evicted >= 1 and eng.graphs.replays >= 4
+
+
+def test_random_weights_are_the_same_bytes_on_the_gpu_and_in_a_folder(tmp_path):
+    """An engine with random weights made on the GPU is the engine loaded from the folder that the
+    random-weights mode writes on the CPU for the same configuration and seed: the tensors are equal
+    to the byte, so the logits are equal to the bit."""
+    from burn_lm_amd import registry
+    from burn_lm_amd.engine.loading import random_engine
+    from burn_lm_amd.weights.random_init import random_tensors
+    cfg, _ = TINIES["B"]
+    arch = registry.architecture_of(cfg)
+    on_cpu = dict(random_tensors(arch, arch.read_config(cfg), 21, std=0.08, norm_jitter=0.1))
+    on_gpu = dict(random_tensors(arch, arch.read_config(cfg), 21, std=0.08, norm_jitter=0.1, device="cuda"))
+    assert list(on_cpu) == list(on_gpu)
+    for n in on_cpu:
+        assert on_gpu[n].is_cuda and torch.equal(on_cpu[n], on_gpu[n].cpu()), n
+    folder = make_folder(tmp_path / "m", cfg, 21)
+    toks = random_tokens(77, cfg["vocab_size"], 40)
+    for dtype in ("float32", "bfloat16"):
+        a = load(folder, dtype)
+        b = random_engine(cfg, seed=21, dtype=dtype, max_tokens=1024, std=0.08, norm_jitter=0.1)
+        sa, sb = a.open(), b.open()
+        assert torch.equal(a.step([(sa, toks, list(range(40)))]), b.step([(sb, toks, list(range(40)))]))

@@ -1,0 +1,162 @@
+"""Other arrangements of a layer, defined here in the test and registered without a change to the
+framework's files: a block with four norms around its two parts (a norm before and one after each),
+and a block that has a mixer and no feed-forward at all.  The feed-forward of the first is a toy that
+needs an integer table, which the random-weights mode makes from the toy architecture's own list of
+checkpoint tensors.  The toy is no model of anyone's."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+
+TOY = dict(architectures=["ToyBlocksLM"], width=96, heads=6, kv_heads=3, head_dim=16, vocab=203, eps=1e-5,
+           theta=10000.0, max_positions=256)
+
+
+def register_toy():
+    import math
+    from burn_lm_amd import registry
+    from burn_lm_amd.models.plan import LayerPlan, ModelPlan, Place
+    from burn_lm_amd.parts.base import Block, FeedForward, PartSpec, TensorSpec
+    from burn_lm_amd.weights.random_init import IntegerTable, Normal
+
+    class GatherFeedForward(FeedForward):
+        """params: width.  names: table (integers), scale.  delta[:, j] = x[:, table[j]] * scale[j]."""
+
+        def tensor_specs(self):
+            D = self.params["width"]
+            return {self.names["table"]: TensorSpec((D,), kind="int"), self.names["scale"]: TensorSpec((D,))}
+
+        def bind(self, tensors, rt):
+            self.rt = rt
+            self.table = tensors[self.names["table"]].long()
+            self.scale = tensors[self.names["scale"]].float()
+
+        def forward(self, x, step):
+            return (x.float()[:, self.table] * self.scale).to(self.rt.dtype)
+
+    class SandwichBlock(Block):
+        """h = x + post1(mixer(pre1(x))); y = h + post2(ffn(pre2(h)))."""
+        roles = {"pre_mixer_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm",
+                 "pre_ffn_norm": "norm", "feed_forward": "feed_forward", "post_ffn_norm": "norm"}
+
+        def forward(self, h, delta, step, view):
+            x = self.pre_mixer_norm.add_norm(h, delta)
+            a = self.mixer.forward(x, step, view)
+            if a.dim() == 3:
+                a = a.sum(0)
+            a = self.post_mixer_norm.add_norm(a.float().contiguous(), None, write_h=False)   # a norm of the delta alone
+            x = self.pre_ffn_norm.add_norm(h, a)
+            f = self.feed_forward.forward(x, step)
+            return self.post_ffn_norm.add_norm(f.float().contiguous(), None, write_h=False)
+
+    class MixerOnlyBlock(Block):
+        """y = x + mixer(norm(x)): a layer without a feed-forward."""
+        roles = {"mixer_norm": "norm", "mixer": "mixer"}
+
+        def forward(self, h, delta, step, view):
+            return self.mixer.forward(self.mixer_norm.add_norm(h, delta), step, view)
+
+    def plan(cfg, names=None):
+        D = cfg["width"]
+        norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=cfg["eps"]), dict(weight=n))
+        attn = lambda i: PartSpec("attention", dict(width=D, heads=cfg["heads"], kv_heads=cfg["kv_heads"],
+                                                    head_dim=cfg["head_dim"], scale=1 / math.sqrt(cfg["head_dim"])),
+                                  dict(q=f"l{i}.q", k=f"l{i}.k", v=f"l{i}.v", o=f"l{i}.o"))
+        layers = [LayerPlan("toy_sandwich", position="rope", pre_mixer_norm=norm("l0.n1"), mixer=attn(0),
+                            post_mixer_norm=norm("l0.n2"), pre_ffn_norm=norm("l0.n3"),
+                            feed_forward=PartSpec("toy_gather", dict(width=D), dict(table="l0.table", scale="l0.scale")),
+                            post_ffn_norm=norm("l0.n4")),
+                  LayerPlan("toy_mixer_only", {"mixer_norm": norm("l1.n1"), "mixer": attn(1)}, position="rope")]
+        return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
+                         embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         layers=layers, order=[Place(0), Place(1)], final_norm=norm("norm"),
+                         head=PartSpec("linear", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         positions={"rope": PartSpec("rope", dict(head_dim=cfg["head_dim"], theta=cfg["theta"],
+                                                                  pairing="interleaved", scaling=None))})
+
+    def checkpoint_tensors(cfg):
+        D, hd = cfg["width"], cfg["head_dim"]
+        t = {"emb": ((cfg["vocab"], D), "table"), "norm": ((D,), "norm"), "l0.table": ((D,), IntegerTable(D)),
+             "l0.scale": ((D,), Normal(std=0.5)), "l1.n1": ((D,), "norm")}
+        for n in ("n1", "n2", "n3", "n4"):
+            t[f"l0.{n}"] = ((D,), "norm")
+        for i in (0, 1):
+            t.update({f"l{i}.q": ((cfg["heads"] * hd, D), "matrix"), f"l{i}.k": ((cfg["kv_heads"] * hd, D), "matrix"),
+                      f"l{i}.v": ((cfg["kv_heads"] * hd, D), "matrix"), f"l{i}.o": ((D, cfg["heads"] * hd), "matrix")})
+        return t
+
+    registry.register_part("feed_forward", "toy_gather", GatherFeedForward)
+    registry.register_part("block", "toy_sandwich", SandwichBlock)
+    registry.register_part("block", "toy_mixer_only", MixerOnlyBlock)
+    registry.register_architecture(registry.Architecture("ToyBlocksLM", read_config=lambda d: d, plan=plan,
+                                                         checkpoint_tensors=checkpoint_tensors))
+
+
+def toy_plain(tokens, w):
+    c = TOY
+    hd = c["head_dim"]
+    freqs = P.rope_base_frequencies(hd, c["theta"])
+    attn = lambda x, i: P.attention_layer(x, w[f"l{i}.q"], w[f"l{i}.k"], w[f"l{i}.v"], w[f"l{i}.o"],
+                                          c["heads"], c["kv_heads"], hd, freqs)
+    n = lambda x, name: P.rms_norm(x, w[name], c["eps"])
+    h = w["emb"][np.asarray(tokens)][None]
+    h = h + n(attn(n(h, "l0.n1"), 0), "l0.n2")
+    x = n(h, "l0.n3")
+    h = h + n(x[..., w["l0.table"].astype(np.int64)] * w["l0.scale"], "l0.n4")
+    h = h + attn(n(h, "l1.n1"), 1)
+    return (n(h, "norm") @ w["emb"].T)[0]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_a_block_with_four_norms_and_a_layer_without_a_feed_forward(tmp_path, dtype, tol):
+    import burn_lm_amd
+    from burn_lm_amd.engine.loading import load_engine
+    from burn_lm_amd.weights import safetensors_io as st
+    register_toy()
+    folder = burn_lm_amd.write_random_model(str(tmp_path), TOY, seed=4, std=0.12, norm_jitter=0.1)
+    f = st.open_folder(folder)
+    stored = {n: f[n].tensor(n) for n in f}
+    assert stored["l0.table"].dtype == torch.int32 and 0 <= int(stored["l0.table"].min()) and int(stored["l0.table"].max()) < TOY["width"]
+    assert len(set(stored["l0.table"].tolist())) > TOY["width"] // 3      # a table of many different places
+    w = {k: v.double().numpy() for k, v in stored.items()}
+    eng = load_engine(folder, dtype=dtype, max_tokens=1024, max_seqs=4)
+    kinds = [type(b).__name__ for b in eng.model.blocks]
+    assert kinds == ["SandwichBlock", "MixerOnlyBlock"] and not hasattr(eng.model.blocks[1], "feed_forward")
+    assert len(eng.model.blocks[0].parts()) == 6 and len(eng.model.blocks[1].parts()) == 2
+    rng = np.random.default_rng(3)
+    reqs = [[int(x) for x in rng.integers(0, TOY["vocab"], L)] for L in (130, 11, 66)]
+    want = [toy_plain(r, w) for r in reqs]
+    slots = [eng.open() for _ in reqs]
+    cut = [len(r) - 5 for r in reqs]
+    got = eng.step([(s, r[:k], list(range(k))) for s, r, k in zip(slots, reqs, cut)]).double().cpu().numpy()
+    o = 0
+    for i, k in enumerate(cut):
+        for p in range(k):
+            assert np.abs(got[o + p] - want[i][p]).max() / np.abs(want[i]).max() <= tol, (dtype, i, p)
+        o += k
+    for j in range(5):
+        got = eng.step([(s, [r[k + j]], [0]) for s, r, k in zip(slots, reqs, cut)]).double().cpu().numpy()
+        for i in range(3):
+            assert np.abs(got[i] - want[i][cut[i] + j]).max() / np.abs(want[i]).max() <= tol, (dtype, i, cut[i] + j)
+    for s in slots:
+        eng.close(s)
+    assert eng.cache.pages_in_use() == 0
+
+
+def test_a_plan_that_names_a_role_its_block_does_not_have_is_refused(tmp_path):
+    from burn_lm_amd import registry
+    from burn_lm_amd.engine.model import Model
+    from burn_lm_amd.parts.base import PartSpec
+    register_toy()
+    plan = registry.architecture("ToyBlocksLM").plan(TOY)
+    plan.layers[1].parts["feed_forward"] = PartSpec("toy_gather", dict(width=TOY["width"]), dict(table="t", scale="s"))
+    with pytest.raises(ValueError, match="no role 'feed_forward'"):
+        Model(plan)
+    plan = registry.architecture("ToyBlocksLM").plan(TOY)
+    del plan.layers[0].parts["post_ffn_norm"]
+    with pytest.raises(ValueError, match="lacks"):
+        Model(plan)

@@ -3,6 +3,7 @@ wrong with a checkpoint (no GPU)."""
 import json
 import os
 
+import numpy as np
 import pytest
 import torch
 
@@ -125,3 +126,48 @@ def test_sharded_folder(tmp_path):
         {"weight_map": {"a": "s1.safetensors", "b": "s2.safetensors"}}))
     f = st.open_folder(str(tmp_path))
     assert f["a"].tensor("a").tolist() == [1, 1] and f["b"].shape("b") == (3,)
+
+
+def test_random_weights_are_a_function_of_seed_name_and_index():
+    """Every value depends on (seed, tensor name, element index) alone: the same tensor comes out
+    whole or in pieces, first or last, and another seed or name gives another one; the values are
+    normal to within what an initialisation can tell."""
+    from burn_lm_amd.weights import random_init as R
+    key = R.tensor_key(3, "a.weight")
+    whole = R.standard_normal(key, 0, 5000)
+    assert torch.equal(whole[1234:1300], R.standard_normal(key, 1234, 66))
+    assert not torch.equal(whole[:100], R.standard_normal(R.tensor_key(4, "a.weight"), 0, 100))
+    assert not torch.equal(whole[:100], R.standard_normal(R.tensor_key(3, "b.weight"), 0, 100))
+    z = R.standard_normal(key, 0, 400000).double()
+    assert abs(float(z.mean())) < 0.01 and abs(float(z.std()) - 1) < 0.01
+    assert abs(float((z ** 4).mean()) - 3) < 0.2 and float(z.abs().max()) > 3.5
+    a = R.make_tensor("w", (70, 33), "matrix", seed=9, std=0.02)
+    b = R.make_tensor("w", (70, 33), "matrix", seed=9, std=0.02)
+    assert a.dtype == torch.bfloat16 and torch.equal(a, b) and 0.018 < float(a.float().std()) < 0.022
+    assert torch.equal(R.make_tensor("n", (8,), "norm", seed=9), torch.ones(8, dtype=torch.bfloat16))
+    table = R.make_tensor("t", (1000,), R.IntegerTable(7), seed=9)
+    assert table.dtype == torch.int32 and set(table.tolist()) == set(range(7))
+    with pytest.raises(ValueError, match="role"):
+        R.make_tensor("x", (3,), "matrices", seed=0)
+
+
+def test_the_range_initialiser_is_the_references_fixture(tmp_path):
+    """crates/burn-lm-llama/src/lib.rs:142-148: arange(n) * (max - min) / n + min, over a linear weight
+    in the reference's [d_in, d_out] order.  As a Meta-named checkpoint of the reference's tiny test
+    model it holds exactly the tensors the reference's whole-model vector is computed from
+    (crates/burn-lm-llama/src/nn/transformer.rs:299-349)."""
+    import burn_lm_amd
+    from burn_lm_amd.weights.random_init import Range
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=8, intermediate_size=16, num_hidden_layers=2,
+               num_attention_heads=2, num_key_value_heads=1, vocab_size=8, rms_norm_eps=1e-5, rope_theta=10000.0,
+               tie_word_embeddings=False, max_position_embeddings=64)
+    folder = burn_lm_amd.write_random_model(str(tmp_path), cfg, init=Range(0.0, 5.0), names="meta", dtype=torch.float32)
+    f = st.open_folder(folder)
+    r = lambda *s: torch.arange(int(np.prod(s)), dtype=torch.float64).mul(5.0 / int(np.prod(s))).reshape(*s)
+    assert torch.equal(f["tok_embeddings.weight"].tensor("tok_embeddings.weight"), r(8, 8).float())
+    assert torch.equal(f["norm.weight"].tensor("norm.weight"), r(8).float())
+    wk = f["layers.1.attention.wk.weight"].tensor("layers.1.attention.wk.weight")
+    assert wk.shape == (4, 8) and torch.equal(wk, r(8, 4).T.contiguous().float())      # [d_out, d_in] of a [d_in, d_out] ramp
+    w2 = f["layers.0.feed_forward.w2.weight"].tensor("layers.0.feed_forward.w2.weight")
+    assert w2.shape == (8, 16) and torch.equal(w2, r(16, 8).T.contiguous().float())
+    assert "output.weight" in f and "layers.1.ffn_norm.weight" in f and len(f) == 3 + 2 * 9
