@@ -3,14 +3,29 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers L]
     python bench.py --preset llama3.2-3b --unequal 16 [--generate 256]     (an unequal batch, end to end)
 
-A "step" is one decode step of the whole batch: the engine's step function on one token per
-sequence, the sampling kernel, and the tokens' trip to the host, as the generation loop does it.
-The default run has the layer sizes of the Llama-3.2-1B shape with random weights, a batch of 8
-and a context of 4096 tokens per sequence.  One JSON line is printed.
+A "step" is one decode step of the whole batch as the generation loop runs it: the engine's step
+function on one token per sequence, the sampling kernel, and the tokens' trip to the host.  Decoding
+is measured *through the generation loop itself* (``engine.generate.generate``): prompts that bring
+every sequence to the context length, W untimed steps, then exactly K steps between two
+synchronisations.  The default run has the layer sizes of the Llama-3.2-1B shape with random weights,
+a batch of 8 and a context of 4096 tokens per sequence.  One JSON line is printed:
+
+* ``value``: decoded tokens a second over the K steps; ``ms_per_step`` their mean; ``step_ms_median``
+  the median of the single steps (HIP events, one after every step).
+* ``roofline``: the bytes a decode step has to read (every weight it uses once and the cache of the
+  live requests, as the model's own parts count them) / its time, against 8 TB/s; ``prefill``: a
+  prompt of 2,048 tokens through the step function, its flops / time against the dense bf16 peak.
+* ``points``: decode at batch 1 and 64 at the same context, with their roofline fractions;
+  ``workload_512_256``: the workload BASELINE.json names (512-token prompts, 256 generated tokens, at
+  batch 1, 8 and 64) as decoded tokens a second over the whole decode phase.
+* ``measured``: what this machine reaches with a kernel that only reads (GB/s) and one that only
+  issues matrix instructions (TFLOP/s), as second denominators; ``kernels``: time and achieved GB/s
+  (decode) or TFLOP/s (prefill) of the dominant kernels alone at the benchmark's shape.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -21,82 +36,56 @@ HBM_PEAK_GBS = 8000.0                                   # MI355X HBM3E, publishe
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}          # dense, published
 
 
-def weight_bytes(cfg, layers, itemsize):
-    d, hd = cfg.hidden_size, cfg.head_dim
-    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * hd * d + d * cfg.num_attention_heads * hd
-                 + 3 * cfg.intermediate_size * d + 2 * d)
-    head = cfg.vocab_size * d
-    return (layers * per_layer + d + head) * itemsize   # the embedding rows read are negligible; tied or not, the head is read once
-
-
-def kv_bytes_per_token(cfg, layers, itemsize):
-    return 2 * layers * cfg.num_key_value_heads * cfg.head_dim * itemsize
-
-
-def prefill_flops(cfg, layers, T, rows_out=1):
-    d, hd, nh, nkv = cfg.hidden_size, cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
-    lin = 2 * T * ((nh + 2 * nkv) * hd * d + d * nh * hd + 3 * cfg.intermediate_size * d)
-    attn = 2 * 2 * nh * hd * (T * (T + 1) // 2)
-    return layers * (lin + attn) + 2 * rows_out * cfg.vocab_size * d
-
-
-def fill_cache(engine, n_seqs, length, seed=0):
-    """Sequences that already hold `length` tokens: pages reserved, lengths set, keys and values
-    random (synthetic; what they hold does not change the work of a decode step)."""
-    import torch
-    g = torch.Generator(device=engine.rt.device).manual_seed(seed)
-    for grp in engine.cache.groups:
-        grp.storage.normal_(0.0, 1.0, generator=g)
-    slots = []
-    for _ in range(n_seqs):
-        s = engine.open()
-        engine.cache.reserve([(s, length)])
-        engine.cache.advance(s, length)
-        slots.append(s)
-    return slots
+def random_prompts(engine, n, length, seed=0):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    return [[int(t) for t in rng.integers(0, engine.vocab_size, length)] for _ in range(n)]
 
 
 def time_decode(engine, sampler, batch, context, steps, warmup):
+    """-> (seconds per step over `steps` steps, median seconds of the single steps).  The batch runs
+    through the generation loop: its prompts end `warmup + steps + 2` tokens before the context."""
     import torch
-    for s in list(engine.cache.live_slots):
-        engine.close(s)
-    start = context - (steps + warmup + 1)
-    slots = fill_cache(engine, batch, start)
-    reqs = list(range(batch))
-    rows = list(range(batch))
+    from burn_lm_amd.engine.generate import generate
 
-    def run(n, first_index, picked):
-        """n decode steps the way the generation loop runs them: the next step starts from the tokens
-        left on the GPU, then the host reads the tokens of the step before."""
-        for i in range(n):
-            logits = engine.step_ahead(slots, rows, picked)
-            if logits is None:      # a shape without a recorded graph yet: the plain step, which records it
-                logits = engine.step([(s, [t], [0]) for s, t in zip(slots, picked.tokens())])
-            nxt = sampler.pick_device(logits, reqs, [first_index + i] * batch)
-            picked.tokens()
-            picked = nxt
-        return picked
+    n_new = warmup + steps + 2
+    prompts = random_prompts(engine, batch, context - n_new)
+    seen, marks, events = [0], {}, []
 
-    logits = engine.step([(s, [1], [0]) for s in slots])
-    picked = run(warmup, 0, sampler.pick_device(logits, reqs, [0] * batch))
-    picked.tokens()
+    def on_token(request, token):
+        if request != 0:
+            return
+        seen[0] += 1        # token 1 comes from the prompt step, token 1 + k from decode step k
+        k = seen[0] - 1
+        if k in (warmup, warmup + steps):
+            torch.cuda.synchronize()
+            marks[k] = time.perf_counter()
+        if warmup <= k <= warmup + steps:
+            e = torch.cuda.Event(enable_timing=True)
+            e.record()
+            events.append(e)
+
+    generate(engine, prompts, sampler, n_new, stop_ids=(), batch_size=batch, on_token=on_token)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    picked = run(steps, warmup, picked)
-    picked.tokens()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    for s in slots:
-        engine.close(s)
-    return dt / steps
+    singles = [a.elapsed_time(b) * 1e-3 for a, b in zip(events[1:-1], events[2:])]   # the first one follows a synchronisation
+    return (marks[warmup + steps] - marks[warmup]) / steps, statistics.median(singles) if singles else float("nan")
 
 
-def time_prefill(engine, T, reps=3):
+def decode_roofline(engine, batch, context, steps, sec):
+    mean_ctx = int(context - steps / 2)
+    c = engine.model.step_costs([mean_ctx - 1] * batch, [1] * batch, batch, engine.cache)
+    achieved = (c["weight_bytes"] + c["cache_bytes"]) / sec / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4)}
+
+
+def time_prefill(engine, T, reps=5):
+    """Median seconds of a prompt of T tokens through the step function (the first run records nothing: a
+    prompt step is replayed from a graph from its second sight on, as in serving)."""
     import torch
-    import numpy as np
-    toks = [int(x) for x in np.random.default_rng(0).integers(0, engine.vocab_size, T)]
-    best = None
-    for r in range(reps + 1):
+    toks = random_prompts(engine, 1, T)[0]
+    times = []
+    for r in range(reps + 2):
         s = engine.open()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -104,9 +93,141 @@ def time_prefill(engine, T, reps=3):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         engine.close(s)
-        if r > 0:
-            best = dt if best is None else min(best, dt)
-    return best
+        if r >= 2:
+            times.append(dt)
+    return statistics.median(times)
+
+
+def time_workload(engine, batch, prompt_len=512, generated=256):
+    """BASELINE.json's decode workload through the generation loop: decoded tokens a second over the
+    decode phase of the second of two runs (the first records the graphs)."""
+    from burn_lm_amd.engine.generate import generate
+    from burn_lm_amd.sampling.sampler import Sampler
+    prompts = random_prompts(engine, batch, prompt_len, seed=1)
+    for _ in range(2):
+        _, stats = generate(engine, prompts, Sampler(temperature=0.0), generated, stop_ids=(), batch_size=batch)
+    return stats.decode_tokens / stats.decode_seconds, stats.prompt_tokens / stats.prompt_seconds
+
+
+def event_time(fn, reps=10, warm=2):
+    """Median seconds of fn() between two events."""
+    import torch
+    for _ in range(warm):
+        fn()
+    pairs = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    return statistics.median(a.elapsed_time(b) for a, b in pairs) * 1e-3
+
+
+def machine_rates(device):
+    import torch
+    from burn_lm_amd.csrc import ops
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    buf.zero_()
+    n = ops.probe_read(buf)
+    read = n / event_time(lambda: ops.probe_read(buf)) / 1e9
+    del buf
+    flops = ops.probe_mfma(iters=2048, blocks=2048, device=device)
+    mfma = flops / event_time(lambda: ops.probe_mfma(iters=2048, blocks=2048, device=device)) / 1e12
+    return {"read_gbs": round(read, 1), "mfma_bf16_tflops": round(mfma, 1)}
+
+
+def kernel_rates(engine, batch, context, prefill_tokens):
+    """The dominant kernels alone, at the shapes of the benchmark's decode step and of its prefill, through
+    the parts' own methods (so the kernels are the ones a step runs).  A kernel is timed as a recorded
+    graph that runs it many times in a row, every time on other weights (the layers' own and copies
+    of them, 768 MB and more in all, so that they come from memory as they do in a step and not from
+    the 256 MB last-level cache) or on another layer's cache; the time is what one kernel adds to a
+    chain of dependent kernels, as in a step.  Decode: achieved GB/s of the weights (or keys and
+    values) a kernel reads once; prefill: achieved TFLOP/s."""
+    import torch
+    from burn_lm_amd.engine.runtime import LinearWeight
+    rt, model = engine.rt, engine.model
+    blocks = [(model.blocks[pl.layer], engine.cache.views[i]) for i, pl in enumerate(model.plan.order)]
+    out = {}
+
+    def spread(weights, least=768 << 20):
+        """The layers' weights of one kind and as many copies as it takes to span `least` bytes."""
+        size = sum(w.w.numel() * w.w.element_size() for w in weights)
+        all_ = list(weights)
+        while size < least:
+            for w in weights:
+                all_.append(LinearWeight(w.w.clone(), None if w.packed is None else w.packed.clone(), w.gated))
+            size *= 2
+        return all_
+
+    def graph_time(calls):
+        """Seconds per call of the calls recorded one after another."""
+        for c in calls[:2]:
+            c()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for c in calls:
+                c()
+        return event_time(g.replay) / len(calls)
+
+    def rate(name, calls, nbytes=None, flops=None):
+        sec = graph_time(calls)
+        r = {"us": round(sec * 1e6, 2)}
+        if nbytes is not None:
+            r["gbs"] = round(nbytes / sec / 1e9, 1)
+        if flops is not None:
+            r["tflops"] = round(flops / sec / 1e12, 1)
+        out[name] = r
+
+    width = model.plan.width
+    m0, f0, v0 = blocks[0][0].mixer, blocks[0][0].feed_forward, blocks[0][1]
+    w_bytes = lambda w: w.w.numel() * w.w.element_size()
+    nh, nkv, hd = m0.heads, m0.kv_heads, m0.head_dim
+    qkvs, os_ = spread([b.mixer.w_qkv for b, _ in blocks]), spread([b.mixer.w_o for b, _ in blocks])
+    gus, downs = spread([b.feed_forward.w_gate_up for b, _ in blocks]), spread([b.feed_forward.w_down for b, _ in blocks])
+    # ---- a decode step of `batch` sequences that hold `context - 1` tokens ----
+    slots = [engine.open() for _ in range(batch)]
+    for s in slots:
+        engine.cache.reserve([(s, context)])
+        engine.cache.advance(s, context - 1)
+    step = engine.build_step([(s, [1], [0]) for s in slots], [context - 1] * batch)
+    x = torch.randn(batch, width, device=rt.device).to(rt.dtype)
+    qkv = m0.project(x, step, v0)
+    att = m0.attend(qkv, step, v0)
+    act = rt.gated_linear(x, f0.w_gate_up)
+    kv_bytes = batch * 2 * nkv * hd * context * v0.k.element_size()
+    rate("decode_qkv_rope", [lambda w=w: m0.position.project_encode_store(x, w, step, v0, nh, nkv, hd) for w in qkvs],
+         nbytes=w_bytes(m0.w_qkv))
+    rate("decode_attention", [lambda b=b, v=v: b.mixer.attend(qkv, step, v) for b, v in blocks * 2], nbytes=kv_bytes)
+    rate("decode_o", [lambda w=w: rt.linear(att, w, partials=True) for w in os_], nbytes=w_bytes(m0.w_o))
+    rate("decode_gate_up", [lambda w=w: rt.gated_linear(x, w) for w in gus], nbytes=w_bytes(f0.w_gate_up))
+    rate("decode_down", [lambda w=w: rt.linear(act, w, partials=True) for w in downs], nbytes=w_bytes(f0.w_down))
+    heads = spread([model.head.weight])
+    rate("decode_head", [lambda w=w: rt.linear(x, w, out_dtype=torch.float32) for w in heads], nbytes=w_bytes(model.head.weight))
+    del heads
+    for s in slots:
+        engine.close(s)
+    # ---- a prompt of `prefill_tokens` tokens ----
+    T = prefill_tokens
+    s = engine.open()
+    engine.cache.reserve([(s, T)])
+    step = engine.build_step([(s, [1] * T, [T - 1])], [0])
+    x = torch.randn(T, width, device=rt.device).to(rt.dtype)
+    qkv = m0.project(x, step, v0)
+    att = m0.attend(qkv, step, v0)
+    act = rt.gated_linear(x, f0.w_gate_up)
+    n = len(blocks)
+    rate("prefill_qkv_rope", [lambda w=w: m0.position.project_encode_store(x, w, step, v0, nh, nkv, hd) for w in qkvs[:n]],
+         flops=2 * T * m0.w_qkv.w.numel())
+    rate("prefill_attention", [lambda b=b, v=v: b.mixer.attend(qkv, step, v) for b, v in blocks], flops=m0.mixing_flops(0, T))
+    rate("prefill_o", [lambda w=w: rt.linear(att, w, partials=True) for w in os_[:n]], flops=2 * T * m0.w_o.w.numel())
+    rate("prefill_gate_up", [lambda w=w: rt.gated_linear(x, w) for w in gus[:n]], flops=2 * T * f0.w_gate_up.w.numel())
+    rate("prefill_down", [lambda w=w: rt.linear(act, w, partials=True) for w in downs[:n]], flops=2 * T * f0.w_down.w.numel())
+    engine.close(s)
+    return out
 
 
 def run_unequal(args):
@@ -126,7 +247,7 @@ def run_unequal(args):
                            max_seqs=args.unequal, max_context=context)
     prompts = [[int(t) for t in rng.integers(0, engine.vocab_size, n)] for n in lens]
     best = None
-    for _ in range(3):      # the first run records the graphs of its shapes
+    for _ in range(3):      # the first runs record the graphs of their shapes
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         _, stats = generate(engine, prompts, Sampler(temperature=0.0), args.generate, batch_size=args.unequal)
@@ -157,7 +278,7 @@ def main():
     ap.add_argument("--preset", default="llama3.2-1b")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 decode points")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points, the 512+256 workload and the single kernels")
     ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of picking greedily (0: greedy)")
     ap.add_argument("--top-p", type=float, default=1.0, help="nucleus mass when sampling")
     ap.add_argument("--unequal", type=int, default=0, metavar="N",
@@ -171,7 +292,6 @@ def main():
     if args.unequal:
         return run_unequal(args)
 
-    import torch
     from burn_lm_amd.config.presets import preset
     from burn_lm_amd.engine.loading import random_engine
     from burn_lm_amd.sampling.sampler import Sampler
@@ -184,31 +304,35 @@ def main():
     engine = random_engine(config, seed=0, dtype=args.dtype, max_tokens=biggest * args.context,
                            max_seqs=biggest, max_context=args.context)
     cfg = engine.config
-    itemsize = 2 if args.dtype == "bfloat16" else 4
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
     sampler = Sampler(temperature=args.temperature, top_p=args.top_p, seed=1)
 
-    sec = time_decode(engine, sampler, args.batch, args.context, args.steps, args.warmup)
+    sec, median = time_decode(engine, sampler, args.batch, args.context, args.steps, args.warmup)
     value = args.batch / sec
-    mean_ctx = args.context - args.steps / 2
-    step_bytes = weight_bytes(cfg, layers, itemsize) + kv_bytes_per_token(cfg, layers, itemsize) * mean_ctx * args.batch
-    achieved = step_bytes / sec / 1e9
 
     T = args.prefill_tokens
     psec = time_prefill(engine, T)
-    pf = prefill_flops(cfg, layers, T)
-    peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
+    pflops = engine.model.step_costs([0], [T], 1)["flops"]
 
-    points = {}
+    points, workload, kernels, measured = {}, {}, {}, {}
     if not args.no_points:
         for b in (1, 64):
-            s = time_decode(engine, sampler, b, args.context, max(8, args.steps // 2), 4)
+            s, _ = time_decode(engine, sampler, b, args.context, max(20, args.steps // 2), 4)
             points[f"decode_b{b}"] = round(b / s, 1)
+            points[f"decode_b{b}_ms"] = round(s * 1e3, 4)
+            points[f"decode_b{b}_hbm_frac"] = decode_roofline(engine, b, args.context, max(20, args.steps // 2), s)["frac"]
+        for b in (1, 8, 64):
+            d, p = time_workload(engine, b)
+            workload[f"decode_b{b}"] = round(d, 1)
+            workload[f"prefill_b{b}"] = round(p, 1)
+        measured = machine_rates(engine.rt.device)
+        kernels = kernel_rates(engine, args.batch, args.context, T)
 
     out = {
         "metric": "decode_tokens_per_second", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic (seeded random weights N(0, 0.02), random token ids, random cache contents)",
+        "scaling": "weak", "vs_baseline": None, "dtype": short,
+        "data": "synthetic (seeded random weights N(0, 0.02), random token ids)",
         "config": {"model": args.preset, "batch": args.batch, "context": args.context, "layers": layers,
                    "layers_of_shape": full_layers, "hidden_size": cfg.hidden_size,
                    "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
@@ -216,10 +340,11 @@ def main():
                    "tied_head": cfg.tie_word_embeddings, "page_size": engine.cache.page_size,
                    "sampling": "greedy" if args.temperature == 0 else f"temperature {args.temperature:g} top-p {args.top_p:g}",
                    "parallelism": "single GPU"},
-        "prefill": {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3), "frac": round(pf / psec / peak, 4)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
-        "points": points,
+        "step_ms_median": round(median * 1e3, 4),
+        "prefill": {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
+                    "frac": round(pflops / psec / MFMA_PEAK[short], 4)},
+        "roofline": decode_roofline(engine, args.batch, args.context, args.steps, sec),
+        "points": points, "workload_512_256": workload, "measured": measured, "kernels": kernels,
     }
     print(json.dumps(out))
 

@@ -216,6 +216,17 @@ class Cache:
             g.pool = PagePool(g.n_pages, _native=_core.NativePool(g.n_pages, handle=lib.blm_cache_pool(self._h, gi)))
             g.tables = _Tables(self, gi)
 
+    def bytes_read(self, length: int) -> int:
+        """Bytes of keys and values that one step reads for a sequence of `length` tokens: every
+        place of the order reads its group's keys and values (a place that shares another's cache
+        reads them again), all of them or the last window."""
+        total = 0
+        for v in self.views:
+            if isinstance(v, KVView):
+                keys = min(length, v.need.window) if v.need.window > 0 else length
+                total += 2 * v.need.n_kv_heads * v.need.head_dim * keys * v.k.element_size()
+        return total
+
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 _lib = None
 _lock = threading.Lock()
 
@@ -55,6 +55,8 @@ _SIGNATURES = {
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
+    "blm_probe_read": [_c_void_p, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p],
+    "blm_probe_mfma": [_c_int, _c_int, _c_void_p, _c_void_p],
     "blm_static_scratch_init": [],
     "blm_argmax_static": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p, _c_void_p,
@@ -562,3 +564,30 @@ def sample(logits, uniforms, temperature, top_p=1.0, out=None):
     _call("blm_sample", logits.data_ptr(), uniforms.data_ptr(), out.data_ptr(), R, V, logits.stride(0),
           float(temperature), float(top_p), scratch.data_ptr(), counters.data_ptr(), _stream())
     return out
+
+
+def probe_read(buffer, blocks=2048):
+    """Launches the read-only measuring kernel over the whole buffer (see probe.hip); returns the bytes it reads."""
+    _gpu(buffer)
+    _contig("buffer", buffer)
+    n = buffer.numel() * buffer.element_size() // 16 * 16
+    sink = _probe_sink(buffer.device)
+    _call("blm_probe_read", buffer.data_ptr(), n, sink.data_ptr(), int(blocks), _stream())
+    return n
+
+
+def probe_mfma(iters=4096, blocks=2048, device="cuda"):
+    """Launches the matrix-instruction measuring kernel; returns the floating-point operations it does."""
+    sink = _probe_sink(torch.device(device))
+    _call("blm_probe_mfma", int(iters), int(blocks), sink.data_ptr(), _stream())
+    return blocks * 4 * iters * 4 * 2 * 32 * 32 * 16
+
+
+_sinks = {}
+
+
+def _probe_sink(device):
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _sinks:
+        _sinks[index] = torch.zeros(4, dtype=torch.float32, device=f"cuda:{index}")
+    return _sinks[index]

@@ -74,6 +74,26 @@ class Model:
         for p in self.positions.values():
             p.prepare(n_positions, self.rt)
 
+    def step_costs(self, pasts, news, wanted_rows, cache=None):
+        """What one step costs at the least: sequences that hold pasts[i] tokens get news[i] more and
+        wanted_rows logits rows are asked for.  -> dict(weight_bytes: every tensor the step uses,
+        read once; cache_bytes: the keys and values it reads (given the cache); flops: its matrix
+        products and its attention).  The parts answer for themselves, so this holds for any plan."""
+        rows = sum(news)
+        weight_bytes = self.embedding.step_bytes(rows) + self.final_norm.step_bytes(wanted_rows) + self.head.step_bytes(wanted_rows)
+        flops = self.head.step_flops(wanted_rows)
+        for place in self.plan.order:
+            block = self.blocks[place.layer]
+            for part in block.parts():
+                weight_bytes += part.step_bytes(rows)
+                flops += part.step_flops(rows)
+                if hasattr(part, "mixing_flops"):
+                    flops += sum(part.mixing_flops(p, n) for p, n in zip(pasts, news))
+        cache_bytes = 0
+        if cache is not None:
+            cache_bytes = sum(cache.bytes_read(p + n) for p, n in zip(pasts, news))
+        return dict(weight_bytes=weight_bytes, cache_bytes=cache_bytes, flops=flops)
+
     def forward(self, step, cache):
         """Logits (float32, [wanted rows, vocab]) of one step, or None when no row is wanted."""
         h = self.embedding.forward(step.token_ids)

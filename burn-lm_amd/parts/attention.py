@@ -74,18 +74,40 @@ class Attention(Mixer):
         self.w_qkv = rt.weight(torch.cat(ws, dim=0))
         self.w_o = rt.weight(tensors[self.names["o"]])
 
+    def step_bytes(self, rows):
+        return sum(w.w.numel() * w.w.element_size() for w in (self.w_qkv, self.w_o))
+
+    def step_flops(self, rows):
+        return 2 * rows * (self.w_qkv.w.numel() + self.w_o.w.numel())
+
+    def mixing_flops(self, past, new):
+        """Scores and weighted values: 2 * 2 * heads * head_dim per (query, visible key) pair."""
+        keys = sum(min(past + t + 1, self.window) if self.window else past + t + 1 for t in range(new)) if self.window \
+            else new * past + new * (new + 1) // 2
+        return 4 * self.heads * self.head_dim * keys
+
     def forward(self, x, step, view):
+        return self.output(self.attend(self.project(x, step, view), step, view))
+
+    def project(self, x, step, view):
+        """q, k, v of the step's tokens, q and k encoded by position, k and v stored in the cache."""
+        return self.position.project_encode_store(x, self.w_qkv, step, view, self.heads, self.kv_heads, self.head_dim)
+
+    def output(self, attended):
+        return self.rt.linear(attended, self.w_o, partials=True)   # the block's next norm sums partial products
+
+    def attend(self, qkv, step, view):
+        """Every token's queries over its sequence's cached keys and values -> [tokens, heads * head_dim]."""
         rt = self.rt
         nh, nkv, hd = self.heads, self.kv_heads, self.head_dim
-        qkv = self.position.project_encode_store(x, self.w_qkv, step, view, nh, nkv, hd)
-        out = torch.empty(x.shape[0], nh * hd, dtype=rt.dtype, device=x.device)
+        out = torch.empty(qkv.shape[0], nh * hd, dtype=rt.dtype, device=qkv.device)
         table = view.block_table(step)
         aligned = qkv.shape[1] % 8 == 0
         if step.max_new == 1 and aligned and rt.ops.attn_decode_supported(rt.dtype, hd, view.page_size):
             # decode: cut each sequence's keys so that the whole chip has work
             span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
             pages = (span + view.page_size - 1) // view.page_size
-            blocks = x.shape[0] * nkv * ((nh // nkv + 15) // 16)
+            blocks = qkv.shape[0] * nkv * ((nh // nkv + 15) // 16)
             n_splits = decode_splits(pages, blocks, hd)
             rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                                view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
@@ -98,7 +120,7 @@ class Attention(Mixer):
             n_splits = 1
             if step.max_new == 1:
                 span = step.max_len_after if not self.window else min(step.max_len_after, self.window)
-                n_splits = max(1, min((span + 255) // 256, (4 * DECODE_TARGET_BLOCKS) // max(1, x.shape[0] * nh)))
+                n_splits = max(1, min((span + 255) // 256, (4 * DECODE_TARGET_BLOCKS) // max(1, qkv.shape[0] * nh)))
             rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                               view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
-        return rt.linear(out, self.w_o, partials=True)   # the block's next norm sums partial products
+        return out

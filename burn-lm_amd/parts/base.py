@@ -80,6 +80,15 @@ class Part:
     def bind(self, tensors: Dict[str, torch.Tensor], rt) -> None:
         self.rt = rt
 
+    # What a step costs at the least, for measurements against the machine's limits (a bound part answers):
+    def step_bytes(self, rows: int) -> int:
+        """Bytes of this part's tensors that a step over `rows` tokens has to read, each once."""
+        return 0
+
+    def step_flops(self, rows: int) -> int:
+        """Floating-point operations of this part's matrix products for `rows` tokens."""
+        return 0
+
 
 class Norm(Part):
     def add_norm(self, h, delta, rows=None, write_h=True):
@@ -89,6 +98,11 @@ class Norm(Part):
 class Mixer(Part):
     def cache_need(self):
         return None
+
+    def mixing_flops(self, past: int, new: int) -> int:
+        """Operations that move information between tokens (not the projections) when a sequence that
+        holds `past` tokens gets `new` more."""
+        return 0
 
     def forward(self, x, step, view):
         raise NotImplementedError

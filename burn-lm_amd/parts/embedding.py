@@ -23,6 +23,9 @@ class Embedding(Part):
         self.rt = rt
         self.table = tensors[self.names["weight"]].contiguous()
 
+    def step_bytes(self, rows):
+        return rows * self.params["width"] * self.table.element_size()      # the rows that are looked up
+
     def forward(self, ids):
         h = torch.empty(ids.shape[0], self.params["width"], dtype=torch.float32, device=ids.device)
         return self.rt.ops.embed_gather(self.table, ids, h)
@@ -39,6 +42,12 @@ class LMHead(Part):
     def bind(self, tensors, rt):
         self.rt = rt
         self.weight = rt.weight(tensors[self.names["weight"]])
+
+    def step_bytes(self, rows):
+        return self.weight.w.numel() * self.weight.w.element_size() if rows else 0
+
+    def step_flops(self, rows):
+        return 2 * rows * self.weight.w.numel()
 
     def forward(self, x):
         return self.rt.linear(x, self.weight, out_dtype=torch.float32)

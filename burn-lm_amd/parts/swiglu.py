@@ -29,6 +29,12 @@ class SwiGLU(FeedForward):
         self.w_down = rt.weight(tensors[self.names["down"]])
         self.inner = self.params["inner"]
 
+    def step_bytes(self, rows):
+        return sum(w.w.numel() * w.w.element_size() for w in (self.w_gate_up, self.w_down))
+
+    def step_flops(self, rows):
+        return 2 * rows * (self.w_gate_up.w.numel() + self.w_down.w.numel())
+
     def forward(self, x, step):
         rt = self.rt
         return rt.linear(rt.gated_linear(x, self.w_gate_up), self.w_down, partials=True)
