@@ -86,6 +86,7 @@ class Engine:
                     raise StepError(f"slot {slot}: wanted place {w!r} is outside this step's {n} tokens")
 
     def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> Optional[torch.Tensor]:
+        self.rt.check_fault()
         entries = [(int(s), self._integers(s, "token", t), self._integers(s, "wanted place", w)) for s, t, w in entries]
         self._check(entries)
         lengths = [self.cache.length(s) for s, _, _ in entries]

@@ -58,6 +58,7 @@ class Runtime:
         ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
         ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
         ops.static_scratch_init(self.device)   # likewise: the address of the library's own scratch array
+        ops.grid_sync(self.device)             # likewise: the counters and the fault word of resident-grid kernels
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         asked = os.environ.get("BURN_LM_AMD_FUSED_GATE_UP")   # "1": wherever it can run, "0": nowhere, unset: where it is ahead
         self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if asked == "1" else (0, -1)
@@ -68,6 +69,13 @@ class Runtime:
         # from 33 rows on those are 1-2 % ahead at some shapes and as much behind at others)
         self.skinny_gated_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_GATED_ROWS", MFMA_SKINNY_MAX_ROWS))
         self.skinny_planes_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_PLANES_ROWS", MFMA_SKINNY_MAX_ROWS))
+        # "1": the feed-forward half of a decode layer as one resident-grid kernel (ops.decode_ffn) instead of
+        # three kernels.  Off unless asked for: measured 36-53 us against 24-29 us for the three kernels (a
+        # hand-over between blocks through device-wide counters costs more than a kernel boundary here).
+        self.resident_decode = os.environ.get("BURN_LM_AMD_RESIDENT_DECODE") == "1"
+
+    def check_fault(self):
+        ops.check_fault(self.device)
 
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)

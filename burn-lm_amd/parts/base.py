@@ -94,6 +94,11 @@ class Norm(Part):
     def add_norm(self, h, delta, rows=None, write_h=True):
         raise NotImplementedError
 
+    def rms_constants(self):
+        """(gamma, eps) if this norm is ``v / sqrt(mean(v^2) + eps) * gamma`` of ``v = h + delta`` and
+        nothing else, so that a part behind it may form it inside a kernel of its own; else None."""
+        return None
+
 
 class Mixer(Part):
     def cache_need(self):
@@ -111,6 +116,12 @@ class Mixer(Part):
 class FeedForward(Part):
     def forward(self, x, step):
         raise NotImplementedError
+
+    def forward_after_norm(self, h, delta, norm, step):
+        """``forward(norm.add_norm(h, delta), step)``: the pending delta added to the residual stream,
+        the norm, and this feed-forward.  A feed-forward may run the three as one kernel where it
+        has one (it then must leave h as add_norm would)."""
+        return self.forward(norm.add_norm(h, delta), step)
 
 
 class PositionEncoding(Part):

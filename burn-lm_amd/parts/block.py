@@ -15,5 +15,4 @@ class PreNormBlock(Block):
     def forward(self, h, delta, step, view):
         x = self.mixer_norm.add_norm(h, delta)
         a = self.mixer.forward(x, step, view)
-        x = self.ffn_norm.add_norm(h, a)
-        return self.feed_forward.forward(x, step)
+        return self.feed_forward.forward_after_norm(h, a, self.ffn_norm, step)

@@ -27,6 +27,9 @@ class RMSNorm(Norm):
     def step_bytes(self, rows):
         return self.gamma.numel() * self.gamma.element_size()
 
+    def rms_constants(self):
+        return self.gamma, self.eps
+
     def add_norm(self, h, delta, rows=None, write_h=True):
         n = h.shape[0] if rows is None else rows.shape[0]
         out = torch.empty(n, h.shape[1], dtype=self.rt.dtype, device=h.device)
