@@ -193,7 +193,7 @@ def kernel_rates(engine, batch, context, prefill_tokens):
     for s in slots:
         engine.cache.reserve([(s, context)])
         engine.cache.advance(s, context - 1)
-    step = engine.build_step([(s, [1], [0]) for s in slots], [context - 1] * batch)
+    step = engine.build_step([(s, [1], [0]) for s in slots])
     x = torch.randn(batch, width, device=rt.device).to(rt.dtype)
     qkv = m0.project(x, step, v0)
     att = m0.attend(qkv, step, v0)
@@ -214,7 +214,7 @@ def kernel_rates(engine, batch, context, prefill_tokens):
     T = prefill_tokens
     s = engine.open()
     engine.cache.reserve([(s, T)])
-    step = engine.build_step([(s, [1] * T, [T - 1])], [0])
+    step = engine.build_step([(s, [1] * T, [T - 1])])
     x = torch.randn(T, width, device=rt.device).to(rt.dtype)
     qkv = m0.project(x, step, v0)
     att = m0.attend(qkv, step, v0)

@@ -307,22 +307,45 @@ class Cache:
             _raise(code)
         return [list(out[i * width:(i + 1) * width]) for i in range(len(slots))]
 
-    def fill_step(self, entries, pad_seqs: int, pad_tokens: int, width: int, out_ptr: int, capacity: int):
-        """Writes the index arrays of a step for entries (slot, tokens, want) into int32 host memory
-        at out_ptr (see blm_step_fill in csrc/host/cache_core.h for the layout and for the padding
-        to pad_seqs sequences and pad_tokens tokens; 0: none) and returns (tokens, wanted rows, most
-        tokens of one sequence, greatest length after the step)."""
-        slots, counts, tokens, want_counts, wants = [], [], [], [], []
-        for slot, toks, want in entries:
-            slots.append(slot)
-            counts.append(len(toks))
-            tokens.extend(toks)
-            want_counts.append(len(want))
-            wants.extend(want)
+    # ---- a step's entries, packed (cache.core.Packed) ------------------------------------------
+    def check_step(self, packed, vocab: int) -> None:
+        """Slots open, at least one token each, tokens inside the vocabulary, wanted places inside each
+        sequence's tokens: CacheError with the first fault's text, nothing changed."""
+        code = self._lib.blm_step_check(self._h, packed.n, packed.slots, packed.counts, packed.tokens,
+                                        packed.want_counts, packed.wants, int(vocab))
+        if code:
+            _raise(code)
+
+    def reserve_step(self, packed) -> None:
+        detail = (_core.ctypes.c_int * 2)()
+        code = self._lib.blm_cache_reserve(self._h, packed.n, _core.ctypes.cast(packed.slots, _core._ints),
+                                           _core.ctypes.cast(packed.counts, _core._ints), detail)
+        if code == _core.E_OVERFLOW:
+            raise ContextOverflow(detail[0], detail[1])
+        if code:
+            _raise(code)
+
+    def advance_step(self, packed) -> None:
+        code = self._lib.blm_cache_advance_all(self._h, packed.n, packed.slots, packed.counts)
+        if code:
+            _raise(code)
+
+    def lengths_of(self, packed):
+        out = (_core.ctypes.c_int * max(packed.n, 1))()
+        code = self._lib.blm_cache_lengths(self._h, packed.n, packed.slots, out)
+        if code:
+            _raise(code)
+        return out
+
+    def fill_step(self, entries, pad_seqs: int, pad_tokens: int, width: int, out_ptr: int, capacity: int, vocab: int = 0):
+        """Writes the index arrays of a step for entries ((slot, tokens, want) tuples, or a Packed) into
+        int32 host memory at out_ptr (see blm_step_fill in csrc/host/cache_core.h for the layout and for
+        the padding to pad_seqs sequences and pad_tokens tokens; 0: none) and returns (tokens, wanted
+        rows, most tokens of one sequence, greatest length after the step)."""
+        packed = entries if isinstance(entries, _core.Packed) else _core.Packed(entries)
         meta = (_core.ctypes.c_int * 4)()
-        code = self._lib.blm_step_fill(self._h, len(slots), _core.ints(slots), _core.ints(counts), _core.ints(tokens),
-                                       _core.ints(want_counts), _core.ints(wants), pad_seqs, pad_tokens, width, out_ptr,
-                                       capacity, meta)
+        code = self._lib.blm_step_fill(self._h, packed.n, packed.slots, packed.counts, packed.tokens, packed.want_counts,
+                                       packed.wants, pad_seqs, pad_tokens, width, out_ptr, capacity, meta, int(vocab))
         if code:
             _raise(code)
         return tuple(meta)

@@ -8,7 +8,7 @@ from typing import List, Sequence
 
 from ..csrc import build as _build
 
-HOST_ABI = 2
+HOST_ABI = 3
 OK, E_FULL, E_OVERFLOW, E_USAGE = 0, 1, 2, 3
 
 _lib = None
@@ -28,8 +28,18 @@ _SIGNATURES = {
     "blm_cache_page_table": ([_ptr, _int, _int, _ints, _int, _ints], _int), "blm_cache_pool": ([_ptr, _int], _ptr),
     "blm_cache_n_free_slots": ([_ptr], _int), "blm_cache_free_slots": ([_ptr, _ints], _int),
     "blm_cache_live_slots": ([_ptr, _ints], _int),
+    "blm_cache_advance_all": ([_ptr, _int, _ptr, _ptr], _int), "blm_cache_lengths": ([_ptr, _int, _ptr, _ints], _int),
     "blm_step_size": ([_int, _int, _int, _int, _int], _ll),
-    "blm_step_fill": ([_ptr, _int, _ints, _ints, _ints, _ints, _ints, _int, _int, _int, _ptr, _ll, _ints], _int),
+    # the five arrays of a step's entries come as addresses of array('i') buffers (see Packed)
+    "blm_step_fill": ([_ptr, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _int, _int, _int, _ptr, _ll, _ints, _int], _int),
+    "blm_step_check": ([_ptr, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _int], _int),
+    "blm_step_key": ([_int, _ptr, _ints, _ptr, _ptr, _int, _ints, _int, _ints, _int, _int, _int, _ints], None),
+    "blm_plan_batches": ([_int, _ints, _int, _int, _int, _int, _int, _int, _ints], _int),
+    "blm_gen_new": ([_int, _ints, _int, _int, _int, _ints], _ptr), "blm_gen_free": ([_ptr], None),
+    "blm_gen_start": ([_ptr, _int, _ints], _int), "blm_gen_ahead_rows": ([_ptr, _ints], _int),
+    "blm_gen_launched": ([_ptr, _int, _ints], _int), "blm_gen_take": ([_ptr, _ints, _ints], _int),
+    "blm_gen_live": ([_ptr, _ints, _ints], _int), "blm_gen_count": ([_ptr, _int], _int),
+    "blm_uniforms": ([ctypes.c_ulonglong, _int, _ints, _ints, _ptr], None),
 }
 
 
@@ -58,6 +68,55 @@ def last_error() -> str:
 
 def ints(values: Sequence[int]):
     return (ctypes.c_int * len(values))(*values)
+
+
+class Packed:
+    """The entries of one step, (slot, tokens, wanted places) per sequence, as five flat int32 arrays
+    that the native core reads in place: slots, token counts, all tokens, want counts, all wanted
+    places.  Built at C speed; anything that is no integer (a float, a string) raises TypeError, an
+    integer that does not fit 32 bits OverflowError."""
+    __slots__ = ("n", "slots", "counts", "tokens", "want_counts", "wants", "_keep")
+
+    def __init__(self, entries):
+        from array import array
+        slots, counts, tokens, want_counts, wants = array("i"), array("i"), array("i"), array("i"), array("i")
+        for slot, toks, want in entries:
+            slots.append(slot)
+            counts.append(len(toks))
+            tokens.extend(toks)
+            want_counts.append(len(want))
+            wants.extend(want)
+        for a in (tokens, wants):       # an address of an empty array is not one the core may read: give it a word
+            if not len(a):
+                a.append(0)
+        self.n = len(slots)
+        self._keep = (slots, counts, tokens, want_counts, wants)
+        self.slots, self.counts, self.tokens, self.want_counts, self.wants = (a.buffer_info()[0] for a in self._keep)
+
+    @classmethod
+    def one_token_each(cls, slots):
+        """A decode step's entries whose tokens are not known to the host: token 0, its place wanted."""
+        from array import array
+        n = len(slots)
+        self = cls.__new__(cls)
+        self.n = n
+        self._keep = (array("i", slots), array("i", [1]) * n, array("i", [0]) * n, array("i", [1]) * n, array("i", [0]) * n)
+        self.slots, self.counts, self.tokens, self.want_counts, self.wants = (a.buffer_info()[0] for a in self._keep)
+        return self
+
+    def slot_list(self):
+        return self._keep[0].tolist()
+
+    def count_list(self):
+        return self._keep[1].tolist()
+
+    @property
+    def n_tokens(self):
+        return sum(self._keep[1])
+
+    @property
+    def n_wanted(self):
+        return sum(self._keep[3])
 
 
 class NativePool:

@@ -210,6 +210,30 @@ extern "C" int blm_cache_advance(BlmCache* c, int slot, int n) {
   return BLM_OK;
 }
 
+extern "C" int blm_cache_advance_all(BlmCache* c, int n, const int* slots, const int* counts) {
+  for (int i = 0; i < n; ++i) {
+    if (!is_open(*c, slots[i])) return fail(BLM_E_USAGE, "slot %d is not open", slots[i]);
+    if (counts[i] < 0 || c->length[slots[i]] + counts[i] > c->max_context)
+      return fail(BLM_E_USAGE, "slot %d cannot advance by %d", slots[i], counts[i]);
+    for (const Group& g : c->groups)
+      if (pages_for(*c, c->length[slots[i]] + counts[i]) > (int)g.tables[slots[i]].size())
+        return fail(BLM_E_USAGE, "slot %d advances by %d tokens that no page was reserved for", slots[i], counts[i]);
+  }
+  for (int i = 0; i < n; ++i) {
+    const int rc = blm_cache_advance(c, slots[i], counts[i]);
+    if (rc) return rc;
+  }
+  return BLM_OK;
+}
+
+extern "C" int blm_cache_lengths(const BlmCache* c, int n, const int* slots, int* out) {
+  for (int i = 0; i < n; ++i) {
+    if (!is_open(*c, slots[i])) return fail(BLM_E_USAGE, "slot %d is not open", slots[i]);
+    out[i] = c->length[slots[i]];
+  }
+  return BLM_OK;
+}
+
 extern "C" int blm_cache_table_len(const BlmCache* c, int group, int slot) {
   if (group < 0 || group >= (int)c->groups.size() || !is_open(*c, slot)) return -1;
   return (int)c->groups[group].tables[slot].size();
@@ -265,10 +289,35 @@ extern "C" long long blm_step_size(int n_groups, int T, int B, int R, int width)
   return 3LL * T + B + (B + 1) + B + R + (long long)n_groups * B * width;
 }
 
+extern "C" int blm_step_check(const BlmCache* c, int n, const int* slots, const int* counts, const int* tokens,
+                              const int* want_counts, const int* wants, int vocab) {
+  if (n <= 0) return fail(BLM_E_USAGE, "a step needs at least one sequence");
+  long long src = 0, wsrc = 0;
+  for (int i = 0; i < n; ++i) {
+    if (!is_open(*c, slots[i])) return fail(BLM_E_USAGE, "slot %d is not open", slots[i]);
+    if (counts[i] <= 0) return fail(BLM_E_USAGE, "slot %d: a step must bring at least one token per sequence", slots[i]);
+    if (want_counts[i] < 0) return fail(BLM_E_USAGE, "slot %d: bad want count", slots[i]);
+    if (vocab > 0)
+      for (int k = 0; k < counts[i]; ++k)
+        if (tokens[src + k] < 0 || tokens[src + k] >= vocab)
+          return fail(BLM_E_USAGE, "slot %d: token %d is outside the vocabulary of %d", slots[i], tokens[src + k], vocab);
+    src += counts[i];
+    for (int k = 0; k < want_counts[i]; ++k)
+      if (wants[wsrc + k] < 0 || wants[wsrc + k] >= counts[i])
+        return fail(BLM_E_USAGE, "slot %d: wanted place %d is outside this step's %d tokens", slots[i], wants[wsrc + k], counts[i]);
+    wsrc += want_counts[i];
+  }
+  return BLM_OK;
+}
+
 extern "C" int blm_step_fill(const BlmCache* c, int n, const int* slots, const int* counts, const int* tokens,
                              const int* want_counts, const int* wants, int pad_seqs_to, int pad_tokens_to, int width,
-                             int* out, long long cap, int* meta) {
+                             int* out, long long cap, int* meta, int vocab) {
   if (n <= 0) return fail(BLM_E_USAGE, "a step needs at least one sequence");
+  if (vocab > 0) {
+    const int rc = blm_step_check(c, n, slots, counts, tokens, want_counts, wants, vocab);
+    if (rc) return rc;
+  }
   const int B = std::max(n, pad_seqs_to);
   long long real = 0, R = 0;
   int max_new = 0, max_after = 0;

@@ -10,7 +10,7 @@
 extern "C" {
 #endif
 
-#define BLM_HOST_ABI 2
+#define BLM_HOST_ABI 3
 
 #define BLM_OK 0
 #define BLM_E_FULL 1      // no free slot, or not enough free pages
@@ -45,6 +45,10 @@ int blm_cache_length(const BlmCache*, int slot);         // -1 if the slot is no
 int blm_cache_reserve(BlmCache*, int n, const int* slots, const int* n_new, int* detail);
 // The reserved step has run: the sequence is n longer; pages that fell out of a window go back.
 int blm_cache_advance(BlmCache*, int slot, int n);
+// the same for the n sequences of a step, each by counts[i]: checked for all of them first
+int blm_cache_advance_all(BlmCache*, int n, const int* slots, const int* counts);
+// lengths of n slots; BLM_E_USAGE if one is not open
+int blm_cache_lengths(const BlmCache*, int n, const int* slots, int* out);
 int blm_cache_table_len(const BlmCache*, int group, int slot);   // -1 if the slot is not open
 int blm_cache_table(const BlmCache*, int group, int slot, int* out);
 // rows of `width` page numbers for the given slots, -1 where a sequence has no page (a slot < 0
@@ -68,11 +72,16 @@ int blm_cache_live_slots(const BlmCache*, int* out);     // ascending; returns t
 // token (slot -1, length 0, their wanted row is row 0 and is dropped by the caller); padding tokens
 // stand behind the real ones and belong to no sequence (token 0, position 0, sequence -1).
 // meta: T, R, most tokens of one sequence, greatest length after the step.  The caller sizes
-// `out` with blm_step_size.
+// `out` with blm_step_size.  vocab > 0: every token id must lie in [0, vocab) (BLM_E_USAGE names the
+// first that does not); wanted places outside a sequence's tokens are refused likewise.
 long long blm_step_size(int n_groups, int T, int B, int R, int width);
 int blm_step_fill(const BlmCache*, int n, const int* slots, const int* counts, const int* tokens,
                   const int* want_counts, const int* wants, int pad_seqs_to, int pad_tokens_to, int width,
-                  int* out, long long cap, int* meta);
+                  int* out, long long cap, int* meta, int vocab);
+// The same checks without writing anything: slots open, counts positive, tokens in the vocabulary,
+// wanted places inside each sequence's tokens.
+int blm_step_check(const BlmCache*, int n, const int* slots, const int* counts, const int* tokens,
+                   const int* want_counts, const int* wants, int vocab);
 
 #ifdef __cplusplus
 }

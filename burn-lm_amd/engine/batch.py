@@ -30,16 +30,19 @@ class Step:
     host_image: object = None    # the pinned host buffer the index arrays were copied from
 
 
-def build_step(entries: Sequence, lengths: Sequence[int], cache, device) -> Step:
-    """entries: (slot, tokens, want) per sequence; lengths: what each already holds.  The native
+def build_step(entries, cache, device) -> Step:
+    """entries: (slot, tokens, want) per sequence, or the same packed (cache.core.Packed).  The native
     core writes all index arrays into one host buffer, which goes to the device in one copy."""
-    news = [len(e[1]) for e in entries]
-    T, B, R = sum(news), len(entries), sum(len(e[2]) for e in entries)
+    from ..cache.core import Packed
+    packed = entries if isinstance(entries, Packed) else Packed(entries)
+    news = packed.count_list()
+    lengths = list(cache.lengths_of(packed))[:packed.n]
+    T, B, R = sum(news), packed.n, packed.n_wanted
     max_after = max(past + n for past, n in zip(lengths, news))
     width = max(1, (max_after + cache.page_size - 1) // cache.page_size)
     size = cache.step_size(T, B, R, width)
     host = torch.empty(size, dtype=torch.int32, pin_memory=device.type == "cuda")
-    cache.fill_step(entries, 0, 0, width, host.data_ptr(), size)
+    cache.fill_step(packed, 0, 0, width, host.data_ptr(), size)
     dev = host.to(device, non_blocking=True)
     o = 0
 
@@ -55,6 +58,6 @@ def build_step(entries: Sequence, lengths: Sequence[int], cache, device) -> Step
     step = Step(n_tokens=T, n_seqs=B, n_wanted=R, token_ids=token_ids, positions=positions, token_seq=token_seq,
                 seq_slots=seq_slots, cu_seqlens=cu_seqlens, lens_after=lens_after, want_rows=want_rows,
                 block_tables=block_tables, max_new=max(news), max_position=max_after - 1, max_len_after=max_after,
-                is_decode=all(n == 1 for n in news), host_slots=[e[0] for e in entries], host_new=news)
+                is_decode=all(n == 1 for n in news), host_slots=packed.slot_list(), host_new=news)
     step.host_image = host   # the pinned source of the copy stays alive as long as the step
     return step

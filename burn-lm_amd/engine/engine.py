@@ -11,12 +11,12 @@ reference's loop (crates/burn-lm-llama/src/generation/generate.rs:66-85) is one 
 """
 from __future__ import annotations
 
-import operator
 from typing import Optional, Sequence, Tuple
 
 import torch
 
-from ..cache.cache import Cache
+from ..cache.cache import Cache, CacheError
+from ..cache.core import Packed
 
 
 class StepError(ValueError):
@@ -56,50 +56,33 @@ class Engine:
             self.cache.close(s)
 
     # ---- the step ----------------------------------------------------------------------------
-    @staticmethod
-    def _integers(slot, what, values):
-        """values as Python integers; anything that is no integer (a float, a string, a bool) is refused
-        as such, numpy's and torch's integer scalars are taken."""
-        out = []
-        for v in values:
-            if isinstance(v, bool):
-                raise StepError(f"slot {slot}: {what} {v!r} is a {type(v).__name__}, not an integer")
-            try:
-                out.append(operator.index(v))
-            except TypeError:
-                raise StepError(f"slot {slot}: {what} {v!r} is a {type(v).__name__}, not an integer") from None
-        return out
-
-    def _check(self, entries):
-        if not entries:
+    def _pack(self, entries):
+        """The step's entries as flat arrays for the native core, everything about them checked there:
+        slots open, at least one token per sequence, tokens inside the vocabulary, wanted places inside
+        each sequence's tokens.  StepError before anything changes."""
+        try:
+            packed = Packed(entries)
+        except (TypeError, OverflowError, ValueError) as e:
+            raise StepError(f"a step's slots, tokens and wanted places must be integers that fit 32 bits: {e}") from None
+        if packed.n == 0:
             raise StepError("a step needs at least one sequence")
-        V = self.vocab_size
-        for slot, tokens, want in entries:
-            n = len(tokens)
-            if n == 0:
-                raise StepError(f"slot {slot}: a step must bring at least one token per sequence")
-            for t in tokens:
-                if not 0 <= t < V:
-                    raise StepError(f"slot {slot}: token {t!r} is outside the vocabulary of {V}")
-            for w in want:
-                if not 0 <= w < n:
-                    raise StepError(f"slot {slot}: wanted place {w!r} is outside this step's {n} tokens")
+        try:
+            self.cache.check_step(packed, self.vocab_size)
+        except CacheError as e:
+            raise StepError(str(e)) from None
+        return packed
 
     def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> Optional[torch.Tensor]:
         self.rt.check_fault()
-        entries = [(int(s), self._integers(s, "token", t), self._integers(s, "wanted place", w)) for s, t, w in entries]
-        self._check(entries)
-        lengths = [self.cache.length(s) for s, _, _ in entries]
-        self.cache.reserve([(s, len(t)) for s, t, _ in entries])  # raises before any change
-        key = self.graphs.key_for(entries, lengths) if self.graphs is not None else None
-        logits = self.graphs.run(key, entries) if key is not None else None
+        packed = self._pack(entries)
+        self.cache.reserve_step(packed)  # raises before any change
+        key = self.graphs.key_for(packed) if self.graphs is not None else None
+        logits = self.graphs.run(key, packed) if key is not None else None
         if logits is None:
-            step = self.build_step(entries, lengths)
-            logits = self.model.forward(step, self.cache)
+            logits = self.model.forward(self.build_step(packed), self.cache)
             if key is not None:
                 self.graphs.after_eager(key)
-        for s, t, _ in entries:
-            self.cache.advance(s, len(t))
+        self.cache.advance_step(packed)
         return logits
 
     def step_ahead(self, slots: Sequence[int], rows: Sequence[int], picked) -> Optional[torch.Tensor]:
@@ -111,20 +94,19 @@ class Engine:
         step (a sampler's pick) reads them safely, a caller that keeps them longer must copy them."""
         if self.graphs is None:
             return None
-        slots = [int(s) for s in slots]
-        rows = [int(r) for r in rows]
-        if not slots or len(rows) != len(slots) or any(not 0 <= r < picked.device.shape[0] for r in rows):
+        n_picked = picked.device.shape[0]
+        if not slots or len(rows) != len(slots) or min(rows) < 0 or max(rows) >= n_picked:
             raise StepError("step_ahead needs one row of the picked tokens for every sequence")
-        lengths = [self.cache.length(s) for s in slots]
-        key = self.graphs.key_for([(s, [0], [0]) for s in slots], lengths)
+        packed = Packed.one_token_each(slots)
+        key = self.graphs.key_for(packed)
         if key is None or key not in self.graphs.captured:
             return None
-        self.cache.reserve([(s, 1) for s in slots])  # raises before any change
-        logits = self.graphs.run_ahead(key, slots, rows, picked.device)
-        for s in slots:
-            self.cache.advance(s, 1)
+        self.cache.reserve_step(packed)  # raises before any change
+        logits = self.graphs.run_ahead(key, packed, rows, picked.device)
+        self.cache.advance_step(packed)
         return logits
 
-    def build_step(self, entries, lengths):
+    def build_step(self, entries):
+        """The eager step's index arrays on the device; entries: (slot, tokens, want) tuples or a Packed."""
         from .batch import build_step
-        return build_step(entries, lengths, self.cache, self.rt.device)
+        return build_step(entries, self.cache, self.rt.device)

@@ -28,6 +28,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Callable, List, Optional, Sequence
 
+from ..cache import core as _core
 from .stats import Stats
 
 
@@ -49,25 +50,64 @@ class Generation:
     error: Optional[str] = None
 
 
-def _pages(n_tokens, page):
-    return (n_tokens + page - 1) // page
-
-
 def plan_batches(prompt_lens: Sequence[int], sample_len: int, batch_size: int, max_context: int,
                  page_size: int, n_pages: int, n_slots: int) -> List[List[int]]:
     """Cuts the requests, in order, into batches that fit: at most batch_size sequences and slots,
-    and pages enough for every sequence of the batch to reach its longest possible length."""
-    batches, cur, used = [], [], 0
-    for i, n in enumerate(prompt_lens):
-        need = _pages(min(n + sample_len, max_context), page_size)
-        if cur and (len(cur) >= min(batch_size, n_slots) or used + need > n_pages):
-            batches.append(cur)
-            cur, used = [], 0
-        cur.append(i)
-        used += need
-    if cur:
-        batches.append(cur)
+    and pages enough for every sequence of the batch to reach its longest possible length (decided
+    by the native core, blm_plan_batches)."""
+    n = len(prompt_lens)
+    if n == 0:
+        return []
+    batch_of = (_core.ctypes.c_int * n)()
+    n_batches = _core.library().blm_plan_batches(n, _core.ints(list(prompt_lens)), int(sample_len), int(batch_size),
+                                                 int(max_context), int(page_size), int(n_pages), int(n_slots), batch_of)
+    batches = [[] for _ in range(n_batches)]
+    for i in range(n):
+        batches[batch_of[i]].append(i)
     return batches
+
+
+class _Book:
+    """The generation's bookkeeping in the native core (csrc/host/generation.h): how many tokens each
+    request has, how long its sequence is, what a token means for it, who may run ahead."""
+    GOES_ON, STOP, LENGTH, DROPPED = 0, 1, 2, -1
+
+    def __init__(self, prompt_lens, sample_len, max_context, stop_ids):
+        self._lib = _core.library()
+        stops = sorted(stop_ids)
+        self._h = self._lib.blm_gen_new(len(prompt_lens), _core.ints(list(prompt_lens)), int(sample_len), int(max_context),
+                                        len(stops), _core.ints(stops))
+        if not self._h:
+            raise ValueError("bad sizes for a generation")
+        self._buf = (_core.ctypes.c_int * max(1, len(prompt_lens)))()
+        self._buf2 = (_core.ctypes.c_int * max(1, len(prompt_lens)))()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.blm_gen_free(self._h)
+            self._h = None
+
+    def start(self, requests):
+        if self._lib.blm_gen_start(self._h, len(requests), _core.ints(list(requests))):
+            raise ValueError("a batch names a request that does not exist")
+
+    def ahead_rows(self):
+        n = self._lib.blm_gen_ahead_rows(self._h, self._buf)
+        return self._buf[:n]
+
+    def launched(self, rows):
+        if self._lib.blm_gen_launched(self._h, len(rows), _core.ints(list(rows))):
+            raise ValueError("a launched row is not a live entry")
+
+    def take(self, tokens):
+        """-> (entries that go on, what each entry's token means)"""
+        n = len(tokens)
+        going = self._lib.blm_gen_take(self._h, _core.ints(list(tokens)), self._buf)
+        return going, self._buf[:n]
+
+    def live(self):
+        n = self._lib.blm_gen_live(self._h, self._buf, self._buf2)
+        return self._buf[:n], self._buf2[:n]
 
 
 def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int, stop_ids: Sequence[int] = (),
@@ -96,9 +136,11 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
     batches = plan_batches([len(prompts[i]) for i in runnable], sample_len, batch_size, engine.max_context,
                            cache.page_size, cache.n_pages, cache.max_seqs)
     ahead = hasattr(engine, "step_ahead") and hasattr(sampler, "pick_device")
+    book = _Book([len(p) for p in prompts], sample_len, engine.max_context, stop)
+    reason_names = {_Book.STOP: "stop", _Book.LENGTH: "length"}
     for batch in batches:
         ids = [runnable[j] for j in batch]
-        live, open_slots = [], set()
+        slot_of, open_slots = {}, set()
 
         def close(slot):
             open_slots.discard(slot)
@@ -108,35 +150,34 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
             for i in ids:       # inside the try: a slot that cannot be had must not strand the ones already opened
                 slot = engine.open()
                 open_slots.add(slot)
-                live.append((i, slot))
+                slot_of[i] = slot
             t0 = clock()
-            logits = engine.step([(slot, list(prompts[i]), [len(prompts[i]) - 1]) for i, slot in live])
-            picked = sampler.pick(logits, [i for i, _ in live], [0] * len(live))
-            stats.prompt_tokens += sum(len(prompts[i]) for i, _ in live)
+            logits = engine.step([(slot_of[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in ids])
+            picked = sampler.pick(logits, ids, [0] * len(ids))
+            stats.prompt_tokens += sum(len(prompts[i]) for i in ids)
             stats.prompt_seconds += clock() - t0
             stats.steps += 1
             t0 = clock()
             from_prompt = True
-            dropped = set()     # requests among `live` that ended before the step in flight: their token is ignored
+            book.start(ids)
+            live = list(ids)        # requests whose token is pending, in the order of the pending tokens
             while True:
                 # the step after the one whose tokens are still on their way, for every sequence that
                 # cannot end at that token for a reason known beforehand
                 launched = None
                 if ahead and hasattr(picked, "tokens"):
-                    rows = [k for k, (i, slot) in enumerate(live)
-                            if i not in dropped and len(results[i].tokens) + 1 < sample_len
-                            and engine.length(slot) + 1 <= engine.max_context]
+                    rows = book.ahead_rows()
                     if rows:
-                        logits = engine.step_ahead([live[k][1] for k in rows], rows, picked)
+                        logits = engine.step_ahead([slot_of[live[k]] for k in rows], rows, picked)
                         if logits is not None:
+                            book.launched(rows)
                             nxt = [live[k] for k in rows]
-                            launched = (nxt, sampler.pick_device(logits, [i for i, _ in nxt],
-                                                                 [len(results[i].tokens) + 1 for i, _ in nxt]))
+                            launched = sampler.pick_device(logits, nxt, [len(results[i].tokens) + 1 for i in nxt])
                             stats.steps += 1
                 tokens = picked.tokens() if hasattr(picked, "tokens") else picked
-                survivors = []
-                for (i, slot), tok in zip(live, tokens):
-                    if i in dropped:
+                going, reasons = book.take(tokens)
+                for i, tok, why in zip(live, tokens, reasons):
+                    if why == _Book.DROPPED:    # it had ended before the step in flight: this token is ignored
                         continue
                     r = results[i]
                     r.tokens.append(tok)
@@ -145,29 +186,21 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
                         stats.decode_tokens += 1
                     if on_token is not None:
                         on_token(i, tok)
-                    if tok in stop:
-                        r.finish_reason = "stop"
-                    elif len(r.tokens) >= sample_len:
-                        r.finish_reason = "length"
-                    elif engine.length(slot) + (0 if launched and (i, slot) in launched[0] else 1) > engine.max_context:
-                        r.finish_reason = "length"
-                    if r.finish_reason is None:
-                        survivors.append((i, slot))
-                    else:
-                        close(slot)
+                    if why != _Book.GOES_ON:
+                        r.finish_reason = reason_names[why]
+                        close(slot_of[i])
                 from_prompt = False
+                live, _ = book.live()
                 if launched is not None:
-                    live, picked = launched
-                    dropped = {i for i, _ in live if results[i].finish_reason is not None}
-                    if len(dropped) == len(live):
+                    picked = launched
+                    if going == 0:
                         break
                     continue
-                live, dropped = survivors, set()
                 if not live:
                     break
-                logits = engine.step([(slot, [results[i].tokens[-1]], [0]) for i, slot in live])
-                requests, indices = [i for i, _ in live], [len(results[i].tokens) for i, _ in live]
-                picked = sampler.pick_device(logits, requests, indices) if ahead else sampler.pick(logits, requests, indices)
+                logits = engine.step([(slot_of[i], [results[i].tokens[-1]], [0]) for i in live])
+                indices = [len(results[i].tokens) for i in live]
+                picked = sampler.pick_device(logits, live, indices) if ahead else sampler.pick(logits, live, indices)
                 stats.steps += 1
             stats.decode_seconds += clock() - t0
         except BaseException:

@@ -22,12 +22,14 @@ needed, by kernels).
 """
 from __future__ import annotations
 
+import ctypes
 import gc
 import weakref
 from typing import Dict, Tuple
 
 import torch
 
+from ..cache import core as _core
 from .batch import Step
 
 BATCH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128)
@@ -57,11 +59,18 @@ def token_bucket(n: int):
     return None
 
 
+_BATCH_BUCKETS = _core.ints(BATCH_BUCKETS)
+_TOKEN_BUCKETS = _core.ints(TOKEN_BUCKETS)
+
+
 def width_bucket(pages: int, max_width: int) -> int:
     w = 8
     while w < pages:
         w *= 2
     return min(w, max(max_width, 1))
+
+
+_LIB = _core.library
 
 
 class _Captured:
@@ -97,7 +106,7 @@ class _Captured:
                          token_seq=token_seq, seq_slots=seq_slots, cu_seqlens=cu, lens_after=after, want_rows=rows,
                          block_tables=tables, max_new=1 if self.decode else T, max_position=span - 1,
                          max_len_after=span, is_decode=self.decode, host_slots=[], host_new=[])
-        self.fill([], cache)       # all padding: valid contents while capturing
+        self.fill(None, cache)     # all padding: valid contents while capturing
         self.dev.copy_(self.host)
         engine.model.forward(self.step, cache)      # once eagerly at the bucket's size: what the recording meets exists
         self.graph = torch.cuda.CUDAGraph()
@@ -115,11 +124,12 @@ class _Captured:
         torch.cuda.synchronize()
 
     def fill(self, entries, cache):
-        """Host image of the index buffer for these (slot, tokens, [last]) entries, the rest padding;
+        """Host image of the index buffer for these packed (slot, tokens, [last]) entries, the rest padding
+        (None: all padding);
         written by the native core straight into the pinned buffer."""
         B, W = self.B, self.W
         NT = B if self.decode else self.T
-        if entries:
+        if entries is not None:
             cache.fill_step(entries, B, NT, W, self.host.data_ptr(), self.src_at)
             return
         # all padding (used while recording): token 0, position 0, no sequence, no slot, no pages
@@ -135,15 +145,15 @@ class _Captured:
         self.copied = torch.cuda.Event()
         self.copied.record()
         self.graph.replay()
-        return self.logits[: len(entries)].clone()   # the graph's own output buffer is overwritten by the next replay
+        return self.logits[: entries.n].clone()   # the graph's own output buffer is overwritten by the next replay
 
-    def run_ahead(self, slots, rows, tokens_dev, cache):
+    def run_ahead(self, packed, rows, tokens_dev, cache):
         """Like run() for a decode step, but row i's token is tokens_dev[rows[i]], taken on the device:
         the host need not have seen the tokens of the step before.  The logits come back without a copy."""
         if self.copied is not None:
             self.copied.synchronize()
-        n = len(slots)
-        self.fill([(s, [0], [0]) for s in slots], cache)
+        n = packed.n
+        self.fill(packed, cache)
         self.host_np[self.src_at: self.src_at + n] = rows
         self.dev.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()
@@ -165,24 +175,18 @@ class StepGraphs:
         self.replays = 0
         self.evicted = 0
 
-    def key_for(self, entries, lengths):
-        """Bucket key (sequences, tokens or 0 for a decode step, table width) of a step, or None if
-        the step cannot be replayed from a graph."""
-        if not self.enabled or any(w != [len(t) - 1] for _, t, w in entries):
+    def key_for(self, packed):
+        """Bucket key (sequences, tokens or 0 for a decode step, table width) of a step (its packed
+        entries), or None if the step cannot be replayed from a graph; decided by the native core."""
+        if not self.enabled:
             return None
         cache = self._engine().cache
-        tokens = sum(len(t) for _, t, _ in entries)
-        B = batch_bucket(len(entries))
-        if B is None:
-            return None
-        if tokens == len(entries):
-            T = 0
-        else:
-            T = token_bucket(tokens)
-            if T is None or B > PROMPT_MAX_SEQS:
-                return None
-        pages = (max(past + len(t) for past, (_, t, _) in zip(lengths, entries)) + cache.page_size - 1) // cache.page_size
-        return B, T, width_bucket(pages, cache.table_width)
+        lengths = cache.lengths_of(packed)
+        key = (ctypes.c_int * 3)()
+        _LIB().blm_step_key(packed.n, packed.counts, lengths, packed.want_counts, packed.wants, len(BATCH_BUCKETS),
+                            _BATCH_BUCKETS, len(TOKEN_BUCKETS), _TOKEN_BUCKETS, PROMPT_MAX_SEQS, cache.page_size,
+                            cache.table_width, key)
+        return None if key[0] < 0 else (key[0], key[1], key[2])
 
     def run(self, key, entries):
         """Replays the step if its shape has been captured; returns None if it must run eagerly
@@ -200,13 +204,13 @@ class StepGraphs:
             self.captured[key] = c
         return c
 
-    def run_ahead(self, key, slots, rows, tokens_dev):
+    def run_ahead(self, key, packed, rows, tokens_dev):
         """Replays a recorded decode shape with the tokens taken on the device; None if it is not recorded."""
         c = self._use(key)
         if c is None:
             return None
         self.replays += 1
-        return c.run_ahead(slots, rows, tokens_dev, self._engine().cache)
+        return c.run_ahead(packed, rows, tokens_dev, self._engine().cache)
 
     def after_eager(self, key):
         """The shape has just run eagerly.  Met for the second time it is recorded for the times to

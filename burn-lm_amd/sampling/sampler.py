@@ -64,11 +64,12 @@ class Sampler:
         self._ops = ops
         self._ring, self._next = [], 0
 
-    def _pinned_uniforms(self, values):
+    def _pinned_uniforms(self, requests, indices):
         """The uniforms of one step in pinned host memory that the kernel reads in place: no copy is
         queued and no pinned buffer is allocated per step.  A ring of buffers; one is written again
-        only after the kernel that read it has run."""
-        n = len(values)
+        only after the kernel that read it has run.  The numbers are written by the native core
+        (blm_uniforms: the same function as ``uniform`` above)."""
+        n = len(requests)
         if len(self._ring) < UNIFORM_RING:
             self._ring.append([torch.empty(max(n, 64), dtype=torch.float32).pin_memory(), None])
             slot = self._ring[-1]
@@ -79,7 +80,9 @@ class Sampler:
             slot[1].synchronize()     # the kernel that read this buffer last has run (long since, as a rule)
         if slot[0].numel() < n:
             slot[0] = torch.empty(n, dtype=torch.float32).pin_memory()
-        slot[0].numpy()[:n] = values
+        from ..cache import core as _core
+        _core.library().blm_uniforms(self.seed & _MASK, n, _core.ints(list(requests)), _core.ints(list(indices)),
+                                     slot[0].data_ptr())
         return slot
 
     @property
@@ -99,7 +102,7 @@ class Sampler:
         if self.greedy:
             out = ops.argmax(logits)
         else:
-            slot = self._pinned_uniforms(self.uniforms(requests, indices))
+            slot = self._pinned_uniforms(requests, indices)
             out = ops.sample(logits, slot[0][:logits.shape[0]], self.temperature, self.top_p)
             slot[1] = torch.cuda.Event()
             slot[1].record()

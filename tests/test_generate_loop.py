@@ -241,3 +241,43 @@ def test_running_ahead_stops_at_the_end_of_the_context_without_an_extra_step():
     assert max(n for st in eng.steps for _, n in st if n == 1) == 1
     for s in eng.opened:
         assert s not in eng.cache.live_slots
+
+
+def test_the_native_core_draws_the_same_uniforms_and_plans_the_same_batches():
+    """The host core (C++) holds the loop's decisions; its random numbers are the function `uniform`."""
+    import ctypes
+    from burn_lm_amd.cache import core
+    from burn_lm_amd.engine.generate import plan_batches
+    reqs, idx = [0, 3, 7, 100, 2 ** 20], [0, 1, 5000, 3, 9]
+    out = (ctypes.c_float * 5)()
+    core.library().blm_uniforms(12345678901234567, 5, core.ints(reqs), core.ints(idx), ctypes.cast(out, ctypes.c_void_p))
+    assert list(out) == [uniform(12345678901234567, r, i) for r, i in zip(reqs, idx)]
+    # batches: at most 3 sequences, and pages for prompt + sample_len each (pages of 64, 10 pages in all)
+    assert plan_batches([5, 200, 70, 1, 300, 9], 60, 3, 1024, 64, 10, 8) == [[0, 1], [2, 3], [4, 5]]
+    assert plan_batches([5, 5, 5, 5], 10, 3, 1024, 64, 100, 2) == [[0, 1], [2, 3]]      # two slots only
+    assert plan_batches([], 10, 3, 1024, 64, 100, 2) == []
+
+
+def test_the_native_core_decides_which_steps_are_replayed():
+    """blm_step_key: the bucket of a step that wants each sequence's last token only; -1 otherwise."""
+    import ctypes
+    from burn_lm_amd.cache import core
+    from burn_lm_amd.engine import graphs
+
+    def key(counts, lengths, wants):
+        p = core.Packed([(i, [0] * c, w) for i, (c, w) in enumerate(zip(counts, wants))])
+        k = (ctypes.c_int * 3)()
+        core.library().blm_step_key(p.n, p.counts, core.ints(lengths), p.want_counts, p.wants, len(graphs.BATCH_BUCKETS),
+                                    graphs._BATCH_BUCKETS, len(graphs.TOKEN_BUCKETS), graphs._TOKEN_BUCKETS,
+                                    graphs.PROMPT_MAX_SEQS, 64, 64, k)
+        return tuple(k) if k[0] >= 0 else None
+
+    assert key([1, 1, 1], [10, 700, 3], [[0], [0], [0]]) == (4, 0, 16)          # decode: 3 -> bucket 4, 11 pages -> 16
+    assert key([1], [5], [[0]]) == (1, 0, 8)
+    assert key([40, 7, 90], [0, 0, 0], [[39], [6], [89]]) == (4, 256, 8)        # prompts: 137 tokens -> 256
+    assert key([40, 7], [0, 0], [[39], [5]]) is None                            # not the last token
+    assert key([40, 7], [0, 0], [[39], []]) is None                             # nothing wanted
+    assert key([3000], [0], [[2999]]) is None                                   # beyond the token buckets
+    assert key([2] * 17, [0] * 17, [[1]] * 17) is None                          # too many sequences for a prompt step
+    assert key([1] * 129, [0] * 129, [[0]] * 129) is None                       # beyond the batch buckets
+    assert key([1], [64 * 64 - 1], [[0]]) == (1, 0, 64)                         # the widest table

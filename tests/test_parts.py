@@ -116,7 +116,7 @@ def test_attention_part(rt, pairing, heads, kv_heads, hd):
                     entries.append((slots[i], [0] * c, []))
                     idx.append((i, d, c))
             cache.reserve([(s, len(tk)) for s, tk, _ in entries])
-            step = build_step(entries, [cache.length(s) for s, _, _ in entries], cache, rt.device)
+            step = build_step(entries, cache, rt.device)
             x = torch.cat([xs[i][d:d + c] for i, d, c in idx]).to("cuda")
             y = attn.forward(x, step, cache.views[0])
             o = 0
@@ -188,7 +188,7 @@ def test_pre_norm_block(rt):
     cache = Cache([parts[0].cache_need()], [None], 256, 2, 64, rt.page_size, rt.dtype, rt.device)
     s = cache.open()
     cache.reserve([(s, 19)])
-    step = build_step([(s, [0] * 19, [])], [0], cache, rt.device)
+    step = build_step([(s, [0] * 19, [])], cache, rt.device)
     x0 = torch.randn(19, D, generator=torch.Generator().manual_seed(9))
     pending = (torch.randn(19, D, generator=torch.Generator().manual_seed(10)) * 0.1).to(rt.dtype)
     h = x0.to("cuda")
