@@ -253,7 +253,8 @@ def test_the_native_core_draws_the_same_uniforms_and_plans_the_same_batches():
     core.library().blm_uniforms(12345678901234567, 5, core.ints(reqs), core.ints(idx), ctypes.cast(out, ctypes.c_void_p))
     assert list(out) == [uniform(12345678901234567, r, i) for r, i in zip(reqs, idx)]
     # batches: at most 3 sequences, and pages for prompt + sample_len each (pages of 64, 10 pages in all)
-    assert plan_batches([5, 200, 70, 1, 300, 9], 60, 3, 1024, 64, 10, 8) == [[0, 1], [2, 3], [4, 5]]
+    assert plan_batches([5, 200, 70, 1, 300, 9], 60, 3, 1024, 64, 10, 8) == [[0, 1, 2], [3, 4, 5]]   # 2 + 5 + 3 pages, then 1 + 6 + 2
+    assert plan_batches([5, 200, 70, 1, 300, 9], 60, 3, 1024, 64, 9, 8) == [[0, 1], [2, 3], [4, 5]]      # one page fewer
     assert plan_batches([5, 5, 5, 5], 10, 3, 1024, 64, 100, 2) == [[0, 1], [2, 3]]      # two slots only
     assert plan_batches([], 10, 3, 1024, 64, 100, 2) == []
 
