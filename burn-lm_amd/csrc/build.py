@@ -144,6 +144,55 @@ def build_host(verbose=True):
     return os.path.join(od, HOST_LIB_NAME)
 
 
+REF_LIB_NAME = "libburnlm_ref.so"
+REF_DIR = os.path.join(HERE, "ref")
+
+
+def ref_hash():
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(REF_DIR)):
+        if name.endswith((".cpp", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(REF_DIR, name), "rb") as f:
+                h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()
+
+
+def ref_lib_path():
+    return os.path.join(out_dir(), REF_LIB_NAME)
+
+
+def build_ref(verbose=True):
+    """Compile the plain C++ references of the kernels (ref/*.cpp; the kernel tests compare against
+    them).  No GPU and no ROCm needed.  Always compiles; returns the library path."""
+    cxx = find_cxx()
+    od = out_dir()
+    tmp = os.path.join(od, "_build", REF_LIB_NAME + f".{os.getpid()}.tmp")
+    t0 = time.time()
+    srcs = [os.path.join(REF_DIR, s) for s in sorted(os.listdir(REF_DIR)) if s.endswith(".cpp")]
+    r = subprocess.run([cxx, *HOST_FLAGS, "-I", REF_DIR, *srcs, "-o", tmp], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"{cxx} failed on the reference library:\n{r.stdout}")
+    os.replace(tmp, ref_lib_path())
+    with open(os.path.join(od, "_build", "ref.sha256"), "w") as f:
+        f.write(ref_hash())
+    if verbose:
+        print(f"[burn-lm_amd build] built {ref_lib_path()} in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    return ref_lib_path()
+
+
+def ensure_ref_built(verbose=True):
+    try:
+        with open(os.path.join(out_dir(), "_build", "ref.sha256")) as f:
+            if os.path.exists(ref_lib_path()) and f.read().strip() == ref_hash():
+                return ref_lib_path()
+    except OSError:
+        pass
+    return build_ref(verbose=verbose)
+
+
 def ensure_host_built(verbose=True):
     if host_is_current():
         return host_lib_path()
@@ -160,8 +209,10 @@ def find_hipcc():
 
 def build(verbose=True, jobs=None):
     """Compile every HIP source and link the kernel library, and compile the host library.  Always
-    compiles; returns the kernel library's path."""
+    compiles; returns the kernel library's path.  The plain C++ references that the kernel tests use
+    are compiled along."""
     build_host(verbose=verbose)
+    build_ref(verbose=verbose)
     hipcc = find_hipcc()
     od = out_dir()
     bdir = os.path.join(od, "_build")
