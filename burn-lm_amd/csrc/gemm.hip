@@ -1,7 +1,10 @@
 // Matrix products C[M,N] = A[M,K] * W[N,K]^T (W in checkpoint layout, K contiguous).
 //   gemm_tiled   : any sizes, any mix of float / bf16 operands, float accumulation with plain
 //                  fused multiply-adds.  It is the true 32-bit product of the float path and the
-//                  always-right fallback.
+//                  always-right fallback.  From 32 rows and 32 columns on the multiply-adds are
+//                  those of the matrix cores' float instruction (v_mfma_f32_32x32x2_f32: float
+//                  operands, float products, float sums, nothing narrowed), which does the same
+//                  arithmetic about five times as fast.
 //   gemv_skinny  : M <= 8 rows (decode).  Streams each weight row once with 16-byte loads;
 //                  every wavefront owns output columns and reduces over K across its lanes.
 #include "common.h"
@@ -70,9 +73,85 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// the same product on the matrix cores' float instruction: 128x128 tile per 256 threads, each
+// wavefront a 64x64 quarter as 2x2 instructions of 32x32, K in steps of 16 through shared memory
+// (operands of either type become float there).  Lane l of a 32x32x2 instruction supplies
+// A[l % 32][l / 32] and B[l / 32][l % 32] and holds C[8 (v / 4) + 4 (l / 32) + v % 4][l % 32], v < 16.
+// ---------------------------------------------------------------------------------------
+#define GF_BM 128
+#define GF_BN 128
+#define GF_BK 16
+typedef __attribute__((ext_vector_type(16))) float gf_f32x16;
+
+template <typename TA, typename TW, typename TC>
+__global__ void __launch_bounds__(256)
+    gemm_f32_mfma_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
+                         int lda, int ldc) {
+  __shared__ float As[GF_BK][GF_BM + 4];
+  __shared__ float Ws[GF_BK][GF_BN + 4];
+  const int tid = threadIdx.x, wave = tid / BLM_WAVE, lane = tid & (BLM_WAVE - 1);
+  const int m0 = blockIdx.y * GF_BM, n0 = blockIdx.x * GF_BN;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int li = lane & 31, lk = lane >> 5;
+  gf_f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += GF_BK) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {   // 128 rows x 16 k per operand, 8 elements per thread, k fastest
+      const int idx = tid + e * 256;
+      const int r = idx / GF_BK, kk = idx % GF_BK;
+      const int gk = k0 + kk;
+      float a = 0.f, w = 0.f;
+      if (gk < K) {
+        if (m0 + r < M) a = to_float(A[(size_t)(m0 + r) * lda + gk]);
+        if (n0 + r < N) w = to_float(W[(size_t)(n0 + r) * K + gk]);
+      }
+      As[kk][r] = a;
+      Ws[kk][r] = w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GF_BK; kk += 2) {
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = As[kk + lk][wm + i * 32 + li];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = Ws[kk + lk][wn + j * 32 + li];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3), n = n0 + wn + j * 32 + li;
+        if (m < M && n < N) C[(size_t)m * ldc + n] = from_float<TC>(acc[i][j][v]);
+      }
+}
+
 template <typename TA, typename TW, typename TC>
 static int launch_tiled(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldc,
                         hipStream_t stream) {
+  if (M >= 32 && N >= 32) {
+    dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM), block(256);
+    if (grid.y > 65535) return blm_fail("gemm_tiled: M=%d too large", M);
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)A, (const TW*)W,
+                       (TC*)C, M, N, K, lda, ldc);
+    BLM_LAUNCH_CHECK("gemm_f32_mfma");
+    return 0;
+  }
   dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM), block(256);
   if (grid.y > 65535) return blm_fail("gemm_tiled: M=%d too large", M);
   hipLaunchKernelGGL((gemm_tiled_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)A, (const TW*)W,

@@ -342,9 +342,10 @@ def test_attn_paged_refuses_what_it_cannot_do(ops):
 
 @pytest.mark.parametrize("a,w,c", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
                                    ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
-def test_gemm_tiled(ops, a, w, c):
+@pytest.mark.parametrize("M,N,K", [(70, 130, 50), (20, 130, 50), (300, 31, 64), (257, 129, 1000), (32, 32, 2)])
+def test_gemm_tiled(ops, a, w, c, M, N, K):
+    """With fewer than 32 rows or columns the scalar kernel runs, else the matrix cores' float instruction."""
     g = torch.Generator().manual_seed(5)
-    M, N, K = 70, 130, 50
     A = torch.randn(M, K, generator=g).to(DT[a])
     W = torch.randn(N, K, generator=g).to(DT[w])
     out = torch.empty(M, N, dtype=DT[c], device="cuda")
@@ -366,6 +367,11 @@ def test_float32_product_is_true_32_bit(ops):
         out = torch.empty(3, 65, device="cuda")
         fn(dev(A), dev(W), out)
         assert torch.equal(out.cpu(), torch.full((3, 65), 16.0 + 2.0 ** -16))
+    # many rows: the matrix cores' float instruction, which must be as exact
+    A, W = torch.full((150, K), 1.0 + 2.0 ** -20), torch.ones(70, K)
+    out = torch.empty(150, 70, device="cuda")
+    ops.gemm_tiled(dev(A), dev(W), out)
+    assert torch.equal(out.cpu(), torch.full((150, 70), 16.0 + 2.0 ** -16))
 
 
 @pytest.mark.parametrize("dtype,out_dtype", [("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")])
