@@ -16,6 +16,8 @@
 // Decode:  they are the query heads that share a key-value head, for one token; the key range is
 //          cut into splits that are merged afterwards (float partial results).
 // Visibility: query at position p sees keys j <= p of its sequence and, with a window w, p - j < w.
+#include <stdlib.h>
+
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -320,6 +322,235 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 }
 
 // ---------------------------------------------------------------------------------------
+// prefill with 32 queries per wavefront (head sizes that are multiples of 32, up to 128)
+//
+// The same arrangement on the 32x32x16 instruction: a wavefront owns 32 consecutive tokens of one
+// head, so every key and value fragment it takes from shared memory serves twice as many queries
+// (the shared-memory reads, which bound the 16-query form, are halved per matrix instruction).
+//   S^T = K Q^T      A = 32 keys x 16 dims (lane l: key l % 32, dims 8 (l / 32) ..), B = Q^T (lane l:
+//                    query l % 32, the same dims); the result leaves lane (j = l % 32, hb = l / 32)
+//                    with the scores of query j for keys 8 (v / 4) + 4 hb + v % 4, v < 16, of the tile.
+//   O^T += V^T P^T   A = 32 dims x 16 keys, B = P^T.  The 16 keys of instruction n of a 32-key tile are
+//                    the ones whose scores sit in accumulator values 8 n .. 8 n + 7: lane hb supplies
+//                    keys 16 n + 4 hb .. + 3 and 16 n + 8 + 4 hb .. + 3, which are exactly those values,
+//                    so the probabilities never move; the matching V^T fragment is two 8-byte reads.
+// The softmax of a query lives in the two lanes j and j + 32; the denominator is summed by one
+// two-element dot product with ones per pair of rounded probabilities (v_dot2c_f32_bf16).
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+// acc + lo + hi of a pair of bf16 in one instruction
+__device__ __forceinline__ float am_dot2_ones(uint32_t pair, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 am_bf16x2;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(am_bf16x2, pair), __builtin_bit_cast(am_bf16x2, 0x3f803f80u), acc, false);
+}
+
+// One half page (32 keys from key0) for one wavefront: the softmax state advances once per 32 keys, so
+// only 16 scores per lane are alive at a time.
+template <int HD, bool FULL, int KSTR, int VSTR>
+__device__ __forceinline__ void attn_half32(const bf16* __restrict__ kp, const bf16* __restrict__ vp, const uint4* qf,
+                                            int key0, int qpos, int lo, int max_key, float scale2, float& m,
+                                            float& l, f32x16_t* o) {
+  constexpr int KS = HD / 16, RT = HD / 32;
+  const int lane = threadIdx.x & (BLM_WAVE - 1);
+  const int j = lane & 31, hb = lane >> 5;
+  f32x16_t s;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const uint4 kf = *reinterpret_cast<const uint4*>(kp + (size_t)j * KSTR + ks * 16 + hb * 8);
+    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf), __builtin_bit_cast(bf16x8_t, qf[ks]), s, 0, 0, 0);
+  }
+  if (!FULL) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int kj = key0 + 8 * (v >> 2) + 4 * hb + (v & 3);
+      s[v] = (kj <= qpos && kj >= lo) ? s[v] : -INFINITY;
+    }
+  }
+  float mx = s[0];
+#pragma unroll
+  for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+  mx = fmaxf(mx, __shfl_xor(mx, 32, BLM_WAVE));
+  const float m_new = fmaxf(m, mx * scale2);
+  const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    if (FULL) s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale2, -m_new));
+    else s[v] = (s[v] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale2, -m_new));
+  }
+  if (__any(m != m_new)) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[rt][v] *= corr;
+    l *= corr;
+  }
+  m = m_new;
+  const bool tail = !FULL && key0 + 31 > max_key;   // uniform: the half holds places past the data
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    uint4 pf;
+    pf.x = pack_bf16x2(s[8 * n + 0], s[8 * n + 1]);
+    pf.y = pack_bf16x2(s[8 * n + 2], s[8 * n + 3]);
+    pf.z = pack_bf16x2(s[8 * n + 4], s[8 * n + 5]);
+    pf.w = pack_bf16x2(s[8 * n + 6], s[8 * n + 7]);
+    // the denominator takes the rounded probabilities, two per instruction (a dot product with ones);
+    // a lane sums its own keys, the two lanes of a query are added at the end
+    l = am_dot2_ones(pf.x, l); l = am_dot2_ones(pf.y, l); l = am_dot2_ones(pf.z, l); l = am_dot2_ones(pf.w, l);
+    const int kb = 16 * n + 4 * hb;   // this lane's keys of the instruction: kb .. kb + 3 and kb + 8 .. kb + 11
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const bf16* vrow = vp + (size_t)(rt * 32 + j) * VSTR + kb;
+      uint2 v0 = *reinterpret_cast<const uint2*>(vrow), v1 = *reinterpret_cast<const uint2*>(vrow + 8);
+      if (tail) {   // 0 * garbage must stay 0
+        v0 = keep_first(v0, max_key - (key0 + kb) + 1);
+        v1 = keep_first(v1, max_key - (key0 + kb + 8) + 1);
+      }
+      const uint4 va = make_uint4(v0.x, v0.y, v1.x, v1.y);
+      o[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, pf), o[rt], 0, 0, 0);
+    }
+  }
+}
+
+template <int HD, bool FULL, int KSTR, int VSTR>
+__device__ __forceinline__ void attn_page32(const bf16* __restrict__ kp, const bf16* __restrict__ vp, const uint4* qf,
+                                            int key0, int qpos, int lo, int max_key, float scale2, float& m,
+                                            float& l, f32x16_t* o) {
+  attn_half32<HD, FULL, KSTR, VSTR>(kp, vp, qf, key0, qpos, lo, max_key, scale2, m, l, o);
+  // the second half of a page on the diagonal may lie wholly behind the tile's last query
+  if (FULL || key0 + 32 <= max_key)
+    attn_half32<HD, FULL, KSTR, VSTR>(kp + 32 * KSTR, vp + 32, qf, key0 + 32, qpos, lo, max_key, scale2, m, l, o);
+}
+
+// grid (ceil(G * q_tiles32 / 4), kv heads, sequences); the block order and the page staging are those
+// of the 16-query kernel above
+template <int HD>
+__global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 4 : 2, HD <= 64 ? 4 : 2)))
+    attn_prefill32_kernel(const bf16* __restrict__ q, int q_row_stride, bf16* __restrict__ out,
+                          const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
+                          const int* __restrict__ block_table, int table_width,
+                          const bf16* __restrict__ kcache, const bf16* __restrict__ vcache, int nh, int nkv,
+                          float scale, int window) {
+  static_assert(HD % 32 == 0 && HD <= 128, "32-query prefill: head sizes 32, 64, 96, 128");
+  constexpr int KS = HD / 16, RT = HD / 32, QT = 32;
+  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 4;
+  constexpr int CHUNKS = AM_PAGE * HD / 8;
+  constexpr int PER_THREAD = (CHUNKS + AM_WAVES * BLM_WAVE - 1) / (AM_WAVES * BLM_WAVE);
+  __shared__ __align__(16) bf16 k_lds[2][AM_PAGE * KSTR];
+  __shared__ __align__(16) bf16 v_lds[2][HD * VSTR];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int j = lane & 31, hb = lane >> 5;
+  const int G = nh / nkv;
+  const int b = blockIdx.z;
+  const int row_begin = cu_seqlens[b];
+  const int n_b = cu_seqlens[b + 1] - row_begin;
+  const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+  const int kvh = lin % nkv;
+  int x = lin / nkv;
+  {
+    const int seg = x >> 5;
+    if ((seg & 1) && seg * 32 + 32 <= (int)gridDim.x) x = seg * 32 + 31 - (x & 31);
+  }
+  const int u0 = ((int)gridDim.x - 1 - x) * AM_WAVES;
+  if ((u0 / G) * QT >= n_b) return;   // the whole block lies past the sequence's end (uniform)
+  const int u = u0 + wave;
+  const int g = u % G, qt = u / G;
+  const bool active = qt * QT < n_b;
+  const int head = kvh * G + g;
+  const int nq = active ? min(QT, n_b - qt * QT) : 1;
+  const int row = row_begin + (active ? qt * QT + min(j, nq - 1) : 0);   // columns past the tile's end repeat its last query
+  const int qpos = positions[row];
+  const int qpos_first = positions[row_begin + (active ? qt * QT : 0)];
+  const int qpos_last = positions[row_begin + (active ? qt * QT + nq - 1 : 0)];
+  const int lo = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  const int lo_tile = (window > 0 && qpos_first - window + 1 > 0) ? qpos_first - window + 1 : 0;
+  const int lo_last = (window > 0 && qpos_last - window + 1 > 0) ? qpos_last - window + 1 : 0;
+  const int my_first = active ? lo_tile / AM_PAGE : 0x7fffffff, my_last = active ? qpos_last / AM_PAGE : -1;
+  const int qt_lo = u0 / G, qt_hi = min((u0 + AM_WAVES - 1) / G, (n_b - 1) / QT);
+  const int blk_qfirst = positions[row_begin + qt_lo * QT];
+  const int blk_qlast = positions[row_begin + min(qt_hi * QT + QT - 1, n_b - 1)];
+  const int blk_first = ((window > 0 && blk_qfirst - window + 1 > 0) ? blk_qfirst - window + 1 : 0) / AM_PAGE;
+  const int blk_last = blk_qlast / AM_PAGE;
+
+  uint4 qf[KS];
+  {
+    const bf16* qrow = q + (size_t)row * q_row_stride + (size_t)head * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 16 + hb * 8);
+  }
+  float m = -INFINITY;
+  float lsum = 0.f;
+  f32x16_t o[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[rt][v] = 0.f;
+  const float scale2 = scale * 1.4426950408889634f;
+  const int* bt = block_table + (size_t)b * table_width;
+
+  u32x4_t kreg[PER_THREAD], vreg[PER_THREAD];
+#define AP_FETCH(pi)                                                                          \
+  {                                                                                           \
+    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;                          \
+    _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                  \
+      const int jj = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                   \
+      if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || jj < CHUNKS) {                               \
+        kreg[i] = *reinterpret_cast<const u32x4_t*>(kcache + base + (size_t)jj * 8);            \
+        vreg[i] = *reinterpret_cast<const u32x4_t*>(vcache + base + (size_t)jj * 8);            \
+      }                                                                                       \
+    }                                                                                         \
+  }
+#define AP_STAGE(buf)                                                                                         \
+  _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                                      \
+    const int jj = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                                       \
+    if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || jj < CHUNKS) {                                                   \
+      const int kr = jj / (HD / 8), kc = jj - kr * (HD / 8);                                                    \
+      *reinterpret_cast<u32x4_t*>(k_lds[buf] + kr * KSTR + kc * 8) = kreg[i];                                   \
+      const int vr = jj / (AM_PAGE / 8), vc = jj - vr * (AM_PAGE / 8);                                          \
+      u32x2_t* vd = reinterpret_cast<u32x2_t*>(v_lds[buf] + vr * VSTR + vc * 8);                                \
+      vd[0] = u32x2_t{vreg[i].x, vreg[i].y};                                                                    \
+      vd[1] = u32x2_t{vreg[i].z, vreg[i].w};                                                                    \
+    }                                                                                                           \
+  }
+#define AP_USE(buf)                                                                                           \
+  if (pi >= my_first && pi <= my_last) {                                                                        \
+    const int key0 = pi * AM_PAGE;                                                                              \
+    if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)                                                    \
+      attn_page32<HD, true, KSTR, VSTR>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o);  \
+    else                                                                                                        \
+      attn_page32<HD, false, KSTR, VSTR>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o); \
+  }
+  AP_FETCH(blk_first);
+  AP_STAGE(0)
+  __syncthreads();
+  for (int pi = blk_first; pi <= blk_last; ++pi) {
+    const int cur = (pi - blk_first) & 1;
+    if (pi < blk_last) AP_FETCH(pi + 1);   // travels while this page is used
+    AP_USE(cur)
+    if (pi < blk_last) { AP_STAGE(cur ^ 1) }   // the other buffer: nobody reads it now
+    __syncthreads();   // the next page is in place, and everybody is done with this one
+  }
+#undef AP_STAGE
+#undef AP_USE
+#undef AP_FETCH
+  lsum += __shfl_xor(lsum, 32, BLM_WAVE);   // the two lanes of a query hold the sums over their own keys
+  if (!active || j >= nq) return;
+  const float inv = 1.0f / lsum;
+  bf16* orow = out + (size_t)row * nh * HD + (size_t)head * HD;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {   // four neighbouring dims per store: rt * 32 + 8 gq + 4 hb ..
+      uint2 w;
+      w.x = pack_bf16x2(o[rt][4 * gq + 0] * inv, o[rt][4 * gq + 1] * inv);
+      w.y = pack_bf16x2(o[rt][4 * gq + 2] * inv, o[rt][4 * gq + 3] * inv);
+      *reinterpret_cast<uint2*>(orow + rt * 32 + 8 * gq + 4 * hb) = w;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 #define AD_MERGE 32   // splits whose partial results are asked for together when they are merged
 
 // decode: grid (splits, kv heads * head tiles, tokens); partial results per split
@@ -530,6 +761,37 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
   BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0,
               "attn_prefill_mfma: q rows must be 16-byte aligned");
   const int G = nh / nkv;
+  // 32 queries per wavefront (half the shared-memory reads per matrix instruction) once its blocks are
+  // three times the compute units: with fewer, all blocks run at once and the step lasts as long as
+  // the block with the most pages, whose pages take longer one after another than those of the
+  // 16-query form (measured at 32 heads of 64: 2,048 tokens 49.5 against 43.6 us, 4,096 tokens 108
+  // against 137 us; 24 heads of 128: 68 against 58 us, 141 against 187 us).
+  // BURN_LM_AMD_PREFILL_TILE=16 or 32 forces one form (for measurements).
+  const long long units32 = (long long)G * ((max_new + 31) / 32);
+  const long long blocks32 = (units32 + AM_WAVES - 1) / AM_WAVES * nkv * n_seqs;
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    else cus = 256;
+  }
+  const char* forced = getenv("BURN_LM_AMD_PREFILL_TILE");
+  const bool wide = forced ? forced[0] == '3' : blocks32 >= 3LL * cus;
+  if (hd % 32 == 0 && hd <= 128 && wide) {
+    dim3 grid32((unsigned)((units32 + AM_WAVES - 1) / AM_WAVES), nkv, n_seqs), block32(AM_WAVES * BLM_WAVE);
+#define BLM_AP32(HD)                                                                                             \
+  case HD:                                                                                                       \
+    hipLaunchKernelGGL((attn_prefill32_kernel<HD>), grid32, block32, 0, stream, (const bf16*)q, q_row_stride,     \
+                       (bf16*)out, positions, cu_seqlens, block_table, table_width, (const bf16*)kcache,          \
+                       (const bf16*)vcache, nh, nkv, scale, window);                                              \
+    break
+    switch (hd) {
+      BLM_AP32(32); BLM_AP32(64); BLM_AP32(96); BLM_AP32(128);
+    }
+#undef BLM_AP32
+    BLM_LAUNCH_CHECK("attn_prefill32");
+    return 0;
+  }
   const long long units = (long long)G * ((max_new + 15) / 16);
   dim3 grid((unsigned)((units + AM_WAVES - 1) / AM_WAVES), nkv, n_seqs), block(AM_WAVES * BLM_WAVE);
 #define BLM_AP(HD)                                                                                               \

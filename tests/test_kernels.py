@@ -298,10 +298,16 @@ def test_attn_decode(ops, nh, nkv, hd, window, splits):
 
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (6, 1, 32, 0), (5, 5, 64, 0), (8, 2, 128, 0), (2, 1, 256, 0),
                                                (4, 2, 64, 90), (6, 2, 48, 0), (3, 3, 80, 0), (4, 1, 96, 50), (2, 2, 112, 0)])
-def test_attn_prefill_mfma(ops, nh, nkv, hd, window):
+@pytest.mark.parametrize("tile", ["16", "32"])
+def test_attn_prefill_mfma(ops, nh, nkv, hd, window, tile, monkeypatch):
     """The matrix-core prefill kernel on packed sequences: a whole prompt from position 0 (not a
     multiple of 16 long), a chunk that continues a long past, one token on top of a past that ends at
-    a page edge, a single first token; a far key stands out; unused places hold NaN."""
+    a page edge, a single first token; a far key stands out; unused places hold NaN.  Both forms: 16
+    queries per wavefront, and 32 (head sizes that are multiples of 32; the entry point picks it by
+    itself only for steps of many blocks, so it is forced here)."""
+    if tile == "32" and hd % 32:
+        pytest.skip("the 32-query form takes head sizes that are multiples of 32")
+    monkeypatch.setenv("BURN_LM_AMD_PREFILL_TILE", tile)
     assert ops.attn_prefill_mfma_supported(torch.bfloat16, hd) and not ops.attn_prefill_mfma_supported(torch.float32, hd)
     g = torch.Generator().manual_seed(15)
     lens = [150, 333, 65, 1, 40]             # length of each sequence after the step

@@ -115,11 +115,15 @@ def test_rope_kv_write(ops, ref, dtype, pairing):
 
 @pytest.mark.parametrize("kind,nh,nkv,hd,window", [("generic32", 6, 2, 40, 0), ("generic", 6, 2, 40, 0), ("generic", 3, 3, 24, 50),
                                                    ("decode", 12, 4, 48, 0), ("decode", 4, 1, 112, 90), ("prefill", 10, 5, 80, 0),
-                                                   ("prefill", 2, 2, 16, 70)])
-def test_attention(ops, ref, kind, nh, nkv, hd, window):
+                                                   ("prefill", 2, 2, 16, 70), ("prefill32", 6, 3, 96, 0), ("prefill32", 9, 3, 32, 70),
+                                                   ("prefill32", 4, 1, 128, 0)])
+def test_attention(ops, ref, kind, nh, nkv, hd, window, monkeypatch):
     """The generic kernel (float32 and bfloat16), the matrix-core decode kernel with cut key ranges and the
-    matrix-core prefill kernel: one C++ loop nest is the reference of all three."""
+    matrix-core prefill kernels (16 and 32 queries per wavefront): one C++ loop nest is the reference of all."""
     g = torch.Generator().manual_seed(33)
+    if kind == "prefill32":     # the form with 32 queries per wavefront, which small steps do not pick by themselves
+        monkeypatch.setenv("BURN_LM_AMD_PREFILL_TILE", "32")
+        kind = "prefill"
     dtype = torch.float32 if kind == "generic32" else torch.bfloat16
     page, scale = 64, 1.0 / math.sqrt(hd)
     lens = [200, 65, 7]
