@@ -284,6 +284,9 @@ def main():
     ap.add_argument("--unequal", type=int, default=0, metavar="N",
                     help="instead of the decode measurement: N prompts of 64..2048 tokens through the generation loop")
     ap.add_argument("--generate", type=int, default=256, help="tokens generated per prompt with --unequal")
+    ap.add_argument("--profile", choices=["decode", "prefill"], default=None,
+                    help="run only this part, for a profiler: the decode steps of the batch, or the prompt step ten times; "
+                         "prints its time and no JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this library has no multi-GPU path (run with --gpus 1)")
@@ -307,7 +310,13 @@ def main():
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     sampler = Sampler(temperature=args.temperature, top_p=args.top_p, seed=1)
 
+    if args.profile == "prefill":
+        print(f"prefill of {args.prefill_tokens} tokens: {time_prefill(engine, args.prefill_tokens, reps=10) * 1e3:.3f} ms")
+        return
     sec, median = time_decode(engine, sampler, args.batch, args.context, args.steps, args.warmup)
+    if args.profile == "decode":
+        print(f"decode step of batch {args.batch} at context {args.context}: {sec * 1e3:.4f} ms")
+        return
     value = args.batch / sec
 
     T = args.prefill_tokens
