@@ -119,10 +119,14 @@ class KVGroup:
         self.need, self.places = need, places
         self.page_size = page_size
         self.n_pages = n_pages
-        # [place in group, key|value, page, kv head, token in page * head_dim]; a key page is
-        # [token][head_dim], a value page is stored transposed, [head_dim][token]
-        self.storage = torch.empty(len(places), 2, n_pages, need.n_kv_heads, page_size * need.head_dim,
-                                   dtype=dtype, device=device)
+        # keys [place in group, page, kv head, token in page * head_dim]: a key page is [token][head_dim];
+        # values [place in group, page, value head, value_dim * token in page]: a value page is stored
+        # transposed, [value_dim][token].  Keys and values have storage of their own, so their head sizes
+        # and counts may differ.
+        self.k_storage = torch.empty(len(places), n_pages, need.n_kv_heads, page_size * need.head_dim,
+                                     dtype=dtype, device=device)
+        self.v_storage = torch.empty(len(places), n_pages, need.v_heads, need.v_dim * page_size,
+                                     dtype=dtype, device=device)
         self.pool: Optional[PagePool] = None      # set by the cache once its core exists
         self.tables: Optional[_Tables] = None
 
@@ -143,9 +147,9 @@ class KVView:
 
     def __init__(self, group: KVGroup, group_index: int, plane: int, store: bool):
         self.group_index, self.store = group_index, store
-        n_pages, nkv, hd = group.storage.shape[2], group.need.n_kv_heads, group.need.head_dim
-        self.k = group.storage[plane, 0].view(n_pages, nkv, group.page_size, hd)
-        self.v = group.storage[plane, 1].view(n_pages, nkv, hd, group.page_size)
+        n_pages, need = group.k_storage.shape[1], group.need
+        self.k = group.k_storage[plane].view(n_pages, need.n_kv_heads, group.page_size, need.head_dim)
+        self.v = group.v_storage[plane].view(n_pages, need.v_heads, need.v_dim, group.page_size)
         self.page_size = group.page_size
         self.need = group.need
 
@@ -198,7 +202,8 @@ class Cache:
                     raise CacheError(f"place {i} of the layer order reads the cache of place {src}, which must be "
                                      f"an earlier place that keeps keys and values of its own")
                 sv = self.views[src]
-                if isinstance(need, KVNeed) and (need.n_kv_heads, need.head_dim) != (sv.need.n_kv_heads, sv.need.head_dim):
+                if isinstance(need, KVNeed) and (need.n_kv_heads, need.head_dim, need.v_heads, need.v_dim) != \
+                        (sv.need.n_kv_heads, sv.need.head_dim, sv.need.v_heads, sv.need.v_dim):
                     raise CacheError(f"place {i} cannot read the cache of place {src}: head counts or sizes differ")
                 g = self.groups[sv.group_index]
                 self.views[i] = KVView(g, sv.group_index, g.places.index(src), store=False)
@@ -224,7 +229,7 @@ class Cache:
         for v in self.views:
             if isinstance(v, KVView):
                 keys = min(length, v.need.window) if v.need.window > 0 else length
-                total += 2 * v.need.n_kv_heads * v.need.head_dim * keys * v.k.element_size()
+                total += (v.need.n_kv_heads * v.need.head_dim + v.need.v_heads * v.need.v_dim) * keys * v.k.element_size()
         return total
 
     def __del__(self):

@@ -87,6 +87,8 @@ class Attention(Mixer):
         return 4 * self.heads * self.head_dim * keys
 
     def forward(self, x, step, view):
+        if view.v.shape[1:3] != (self.kv_heads, self.head_dim):
+            raise ValueError("the attention mixer needs values of the keys' head count and head size")
         return self.output(self.attend(self.project(x, step, view), step, view))
 
     def project(self, x, step, view):

@@ -51,10 +51,22 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values per token.  window = 0 keeps every key; window = w keeps the last w."""
+    """Keys and values per token.  window = 0 keeps every key; window = w keeps the last w.  Values
+    may have a head size of their own (value_dim; 0: that of the keys) and a head count of their own
+    (n_value_heads; 0: that of the keys); the attention of this library asks for equal ones."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0
+    n_value_heads: int = 0
+
+    @property
+    def v_dim(self):
+        return self.value_dim or self.head_dim
+
+    @property
+    def v_heads(self):
+        return self.n_value_heads or self.n_kv_heads
 
 
 @dataclass(frozen=True)

@@ -58,7 +58,7 @@ def test_pages_follow_each_sequences_own_length():
 
 def test_layers_of_one_need_share_a_group_and_planes_are_their_own():
     c = make()
-    assert len(c.groups) == 1 and c.groups[0].storage.shape == (3, 2, 16, 2, 16 * 8)
+    assert len(c.groups) == 1 and c.groups[0].k_storage.shape == (3, 16, 2, 16 * 8) and c.groups[0].v_storage.shape == (3, 16, 2, 8 * 16)
     v0, v2 = c.views[0], c.views[2]
     assert isinstance(v0, KVView) and v0.k.data_ptr() != v2.k.data_ptr() and v0.k.data_ptr() != v0.v.data_ptr()
     # key pages are [token][head_dim], value pages are kept transposed
@@ -83,12 +83,23 @@ def test_groups_with_different_needs_have_storage_and_pools_of_their_own():
 
 def test_a_place_may_read_an_earlier_places_cache():
     c = make([KVNeed(2, 8), KVNeed(2, 8), KVNeed(2, 8)], [None, None, 0])
-    assert c.groups[0].storage.shape[0] == 2
+    assert c.groups[0].k_storage.shape[0] == 2
     assert c.views[2].k.data_ptr() == c.views[0].k.data_ptr() and not c.views[2].store
     with pytest.raises(CacheError, match="earlier place"):
         make([KVNeed(2, 8), KVNeed(2, 8)], [1, None])
     with pytest.raises(CacheError, match="differ"):
         make([KVNeed(2, 8), KVNeed(1, 8)], [None, 0])
+    with pytest.raises(CacheError):          # the values' sizes count as the keys' do
+        make([KVNeed(2, 8, value_dim=16), KVNeed(2, 8)], [None, 0])
+
+
+def test_values_with_a_head_size_and_a_head_count_of_their_own():
+    c = make([KVNeed(2, 8, value_dim=20, n_value_heads=1), KVNeed(2, 8)], max_tokens=128)
+    wide = next(g for g in c.groups if g.need.value_dim == 20)
+    assert wide.k_storage.shape == (1, 8, 2, 16 * 8) and wide.v_storage.shape == (1, 8, 1, 20 * 16)
+    v = c.views[0]
+    assert v.k.shape == (8, 2, 16, 8) and v.v.shape == (8, 1, 20, 16)
+    assert len(c.groups) == 2                # another need: storage and pages of its own
 
 
 def test_fixed_size_state_is_per_slot_and_zeroed_when_a_slot_opens():

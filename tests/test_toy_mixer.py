@@ -140,7 +140,7 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype, tol):
     views = eng.cache.views
     assert isinstance(views[0], KVView) and isinstance(views[1], StateView) and isinstance(views[2], KVView)
     assert views[2].k.data_ptr() == views[0].k.data_ptr() and not views[2].store
-    assert eng.cache.groups[0].storage.shape[0] == 1 and views[1].tensor.shape == (4, 48)
+    assert eng.cache.groups[0].k_storage.shape[0] == 1 and views[1].tensor.shape == (4, 48)
     rng = np.random.default_rng(0)
     reqs = [[int(x) for x in rng.integers(0, 97, n)] for n in (70, 9, 33)]
     want = [toy_plain(r, t) for r in reqs]
@@ -263,3 +263,111 @@ def test_a_windowed_attention_layer_beside_a_full_one(tmp_path):
         for s in slots:
             eng.close(s)
         assert eng.cache.pages_in_use() == 0
+
+
+def test_a_mixer_whose_values_have_a_size_and_a_head_count_of_their_own(tmp_path):
+    """The cache keeps keys and values apart, so a mixer may ask for values of another head size and
+    another head count than its keys.  The toy, defined here and written in torch: 4 query heads over
+    2 key heads of size 8, and one value head of size 20 that all query heads share; no rotation.  It
+    writes and reads its pages through the page table by itself."""
+    from burn_lm_amd import registry
+    from burn_lm_amd.engine.loading import load_engine
+    from burn_lm_amd.models.plan import LayerPlan, ModelPlan, Place
+    from burn_lm_amd.parts.base import KVNeed, Mixer, PartSpec, TensorSpec
+    from burn_lm_amd.weights import safetensors_io as st
+    c = dict(architectures=["ToyWideValueLM"], width=40, inner=56, heads=4, kv_heads=2, key_dim=8, value_dim=20, vocab=89,
+             eps=1e-5, max_positions=512)
+    H, G, kd, vd, D = c["heads"], c["kv_heads"], c["key_dim"], c["value_dim"], c["width"]
+
+    class WideValueMixer(Mixer):
+        def tensor_specs(self):
+            n = self.names
+            return {n["q"]: TensorSpec((H * kd, D)), n["k"]: TensorSpec((G * kd, D)), n["v"]: TensorSpec((vd, D)),
+                    n["o"]: TensorSpec((D, H * vd))}
+
+        def cache_need(self):
+            return KVNeed(G, kd, value_dim=vd, n_value_heads=1)
+
+        def bind(self, tensors, rt):
+            self.rt = rt
+            self.q, self.k, self.v, self.o = (tensors[self.names[x]] for x in "qkvo")
+
+        def forward(self, x, step, view):
+            T = x.shape[0]
+            q = self.rt.linear(x, self.q).float().view(T, H, kd)
+            k = self.rt.linear(x, self.k).view(T, G, kd)
+            v = self.rt.linear(x, self.v).view(T, vd)
+            table, pos, page = view.block_table(step).cpu(), step.positions.cpu().tolist(), view.page_size
+            out = torch.zeros(T, H, vd, device=x.device)
+            row = 0
+            for b, n in enumerate(step.host_new):
+                for t in range(row, row + n):
+                    p = int(table[b, pos[t] // page])
+                    view.k[p, :, pos[t] % page] = k[t]
+                    view.v[p, 0, :, pos[t] % page] = v[t]
+                L = pos[row + n - 1] + 1
+                pages = table[b, :(L + page - 1) // page].long().to(x.device)
+                keys = view.k[pages].permute(1, 0, 2, 3).reshape(G, -1, kd)[:, :L].float()       # [G, L, kd]
+                values = view.v[pages][:, 0].permute(1, 0, 2).reshape(vd, -1)[:, :L].float()     # [vd, L]
+                for t in range(row, row + n):
+                    s = torch.einsum("hd,hld->hl", q[t], keys.repeat_interleave(H // G, 0)[:, :pos[t] + 1]) / math.sqrt(kd)
+                    out[t] = torch.softmax(s, -1) @ values[:, :pos[t] + 1].T
+                row += n
+            return self.rt.linear(out.view(T, H * vd).to(self.rt.dtype), self.o)
+
+    def plan(cfg, names=None):
+        norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=cfg["eps"]), dict(weight=n))
+        layer = LayerPlan("pre_norm", mixer=PartSpec("toy_wide_value", {}, dict(q="q", k="k", v="v", o="o")),
+                          feed_forward=PartSpec("swiglu", dict(width=D, inner=cfg["inner"]), dict(gate="gate", up="up", down="down")),
+                          mixer_norm=norm("n1"), ffn_norm=norm("n2"))
+        return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
+                         embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         layers=[layer], order=[Place(0)], final_norm=norm("norm"),
+                         head=PartSpec("linear", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")), positions={})
+
+    registry.register_part("mixer", "toy_wide_value", WideValueMixer)
+    registry.register_architecture(registry.Architecture("ToyWideValueLM", read_config=lambda d: d, plan=plan))
+    g = torch.Generator().manual_seed(8)
+    m = lambda *s: (torch.randn(*s, generator=g) * 0.2).bfloat16()
+    n = lambda: (1 + 0.1 * torch.randn(D, generator=g)).bfloat16()
+    t = {"emb": m(c["vocab"], D), "norm": n(), "n1": n(), "n2": n(), "q": m(H * kd, D), "k": m(G * kd, D), "v": m(vd, D),
+         "o": m(D, H * vd), "gate": m(c["inner"], D), "up": m(c["inner"], D), "down": m(D, c["inner"])}
+    json.dump(c, open(tmp_path / "config.json", "w"))
+    st.write_file(str(tmp_path / "model.safetensors"), t.items())
+    w = {k: v.double().numpy() for k, v in t.items()}
+
+    def plain(tokens):
+        T = len(tokens)
+        h = w["emb"][np.asarray(tokens)][None]
+        x = P.rms_norm(h, w["n1"], c["eps"])
+        q = (x @ w["q"].T).reshape(1, T, H, kd).swapaxes(1, 2)
+        k = (x @ w["k"].T).reshape(1, T, G, kd).swapaxes(1, 2)
+        v = np.repeat((x @ w["v"].T).reshape(1, T, 1, vd).swapaxes(1, 2), G, axis=1)      # the one value head, for every group
+        o = P.scaled_attention(q, k, v, P.hidden_mask(T, T))
+        h = h + o.swapaxes(1, 2).reshape(1, T, -1) @ w["o"].T
+        h = h + P.swiglu_feed_forward(P.rms_norm(h, w["n2"], c["eps"]), w["gate"], w["up"], w["down"])
+        return (P.rms_norm(h, w["norm"], c["eps"]) @ w["emb"].T)[0]
+
+    rng = np.random.default_rng(6)
+    reqs = [[int(x) for x in rng.integers(0, c["vocab"], L)] for L in (100, 17, 70)]
+    want = [plain(r) for r in reqs]
+    err = lambda got, ww: float(np.abs(got.double().cpu().numpy() - ww).max() / np.abs(ww).max())
+    eng = load_engine(str(tmp_path), dtype="float32", max_tokens=512, max_seqs=3)
+    group = eng.cache.groups[0]
+    assert group.k_storage.shape[2:] == (G, 64 * kd) and group.v_storage.shape[2:] == (1, vd * 64)
+    for _ in range(2):                       # twice, so that slots and pages are used again
+        slots = [eng.open() for _ in reqs]
+        cut = [len(r) - 6 for r in reqs]
+        got = eng.step([(s, r[:k], list(range(k))) for s, r, k in zip(slots, reqs, cut)])
+        o = 0
+        for k, ww in zip(cut, want):
+            assert err(got[o:o + k], ww[:k]) <= 2e-5
+            o += k
+        for j in range(6):
+            got = eng.step([(s, [r[k + j]], [0]) for s, r, k in zip(slots, reqs, cut)])
+            for i in range(3):
+                assert err(got[i], want[i][cut[i] + j]) <= 2e-5, (i, j)
+        for s in slots:
+            eng.close(s)
+    assert eng.cache.pages_in_use() == 0
+
