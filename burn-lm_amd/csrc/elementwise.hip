@@ -30,6 +30,45 @@ extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* i
   return 0;
 }
 
+// The same with the token of row t taken on the device where the host does not know it yet:
+// id = (*source)[source_rows[t]] if source_rows[t] >= 0, else ids[t].  `source` is a cell in device
+// memory that holds the address of an int32 array (what a sampler left), so that a recorded launch
+// can read another array at every replay.  An id outside [0, V) gives a row of NaN.
+template <typename TW>
+__global__ void embed_gather_from_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
+                                         const int* __restrict__ source_rows, const int* const* __restrict__ source,
+                                         float* __restrict__ h, int D, int V) {
+  const int t = blockIdx.x;
+  const int r = source_rows[t];
+  const int id = r >= 0 ? (*source)[r] : ids[t];
+  float* out = h + (size_t)t * D;
+  if ((unsigned)id >= (unsigned)V) {
+    for (int d = threadIdx.x; d < D; d += blockDim.x) out[d] = __builtin_nanf("");
+    return;
+  }
+  const TW* row = table + (size_t)id * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) out[d] = to_float(row[d]);
+}
+
+extern "C" int blm_embed_gather_from(const void* table, int table_dtype, const int* ids, const int* source_rows,
+                                     const void* source_cell, float* h, int T, int D, int V, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && D > 0 && V > 0, "embed_gather_from: bad sizes T=%d D=%d V=%d", T, D, V);
+  BLM_REQUIRE(source_rows && source_cell && ((size_t)source_cell & 7) == 0,
+              "embed_gather_from: needs the rows and an 8-byte aligned cell with the tokens' address");
+  dim3 grid(T), block(256);
+  const int* const* cell = (const int* const*)source_cell;
+  if (table_dtype == BLM_F32)
+    hipLaunchKernelGGL(embed_gather_from_kernel<float>, grid, block, 0, stream, (const float*)table, ids, source_rows,
+                       cell, h, D, V);
+  else if (table_dtype == BLM_BF16)
+    hipLaunchKernelGGL(embed_gather_from_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, source_rows,
+                       cell, h, D, V);
+  else
+    return blm_fail("embed_gather_from: unsupported table dtype %d", table_dtype);
+  BLM_LAUNCH_CHECK("embed_gather_from");
+  return 0;
+}
+
 // ---------------------------------------------------------------------------------------
 // residual add + RMS norm
 //   v = h[r] (+ sum over planes p of delta[p][r]);  if write_h: h[r] = v;

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 _lib = None
 _lock = threading.Lock()
 
@@ -23,6 +23,8 @@ class KernelError(RuntimeError):
 
 _SIGNATURES = {
     "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "blm_embed_gather_from": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                              _c_void_p],
     "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p, _c_int,
                         _c_void_p, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "blm_rope_kv_write": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -259,6 +261,24 @@ def embed_gather(table, ids, out_h):
     if out_h.dtype != torch.float32 or table.shape[1] != D:
         raise KernelError("embed_gather: h must be float32 [T, D] with D the table's width")
     _call("blm_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out_h.data_ptr(), T, D, _stream())
+    return out_h
+
+
+def embed_gather_from(table, ids, source_rows, source_cell, out_h):
+    """Like embed_gather, but row t's token is taken on the device where source_rows[t] >= 0: it is
+    element source_rows[t] of the int32 array whose address stands in source_cell (an int64 tensor of
+    one element on the device).  A token outside the vocabulary gives a row of NaN."""
+    _gpu(table, ids, source_rows, source_cell, out_h)
+    T, D = out_h.shape
+    _i32("ids", ids, T)
+    _i32("source_rows", source_rows, T)
+    _contig("table", table); _contig("h", out_h)
+    if out_h.dtype != torch.float32 or table.shape[1] != D:
+        raise KernelError("embed_gather_from: h must be float32 [T, D] with D the table's width")
+    if source_cell.dtype != torch.int64 or source_cell.numel() != 1:
+        raise KernelError("embed_gather_from: the cell is one int64 on the device")
+    _call("blm_embed_gather_from", table.data_ptr(), _code(table), ids.data_ptr(), source_rows.data_ptr(),
+          source_cell.data_ptr(), out_h.data_ptr(), T, D, table.shape[0], _stream())
     return out_h
 
 

@@ -28,6 +28,10 @@ class Step:
     host_slots: List[int] = field(default_factory=list)
     host_new: List[int] = field(default_factory=list)
     host_image: object = None    # the pinned host buffer the index arrays were copied from
+    # (rows int32 [tokens], cell int64 [1]) or None.  Where rows[t] >= 0, token t is not token_ids[t] but
+    # element rows[t] of the int32 array on the device whose address stands in the cell: a token that a
+    # sampler left on the GPU and the host has not read.  Only given to an embedding that has forward_from.
+    token_source: object = None
 
 
 def build_step(entries, cache, device) -> Step:

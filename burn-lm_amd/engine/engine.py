@@ -94,6 +94,8 @@ class Engine:
         step (a sampler's pick) reads them safely, a caller that keeps them longer must copy them."""
         if self.graphs is None:
             return None
+        if picked.device.dtype != torch.int32 or not picked.device.is_contiguous() or picked.device.dim() != 1:
+            raise StepError("step_ahead takes the picked tokens as a contiguous int32 vector on the device")
         n_picked = picked.device.shape[0]
         if not slots or len(rows) != len(slots) or min(rows) < 0 or max(rows) >= n_picked:
             raise StepError("step_ahead needs one row of the picked tokens for every sequence")

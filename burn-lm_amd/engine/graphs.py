@@ -86,9 +86,16 @@ class _Captured:
         self.copied = None
         n = 3 * NT + 4 * B + 1 + G * B * W     # the step's index arrays ...
         self.src_at = n                        # ... and behind them, for run_ahead, where each row's token comes from
-        self.host = torch.zeros(n + B, dtype=torch.int32).pin_memory()
+        self.cell_at = (n + B + 1) // 2 * 2    # ... and the address of the array they come from (8 bytes, aligned)
+        self.host = torch.zeros(self.cell_at + 2, dtype=torch.int32).pin_memory()
         self.host_np = self.host.numpy()
-        self.dev = torch.zeros(n + B, dtype=torch.int32, device=dev)
+        self.host_np[n: n + B] = -1            # no row's token comes from the device
+        self.host_cell = self.host_np[self.cell_at: self.cell_at + 2].view("int64")
+        self.dev = torch.zeros(self.cell_at + 2, dtype=torch.int32, device=dev)
+        self.ahead_rows = 0                    # rows of the host image that the last run_ahead pointed at the device
+        # an embedding that can take tokens from the device does so inside the recorded step; for
+        # another one they are gathered into token_ids by a launch before the replay
+        self.folded = self.decode and hasattr(engine.model.embedding, "forward_from")
         o = 0
 
         def take(k):
@@ -106,6 +113,8 @@ class _Captured:
                          token_seq=token_seq, seq_slots=seq_slots, cu_seqlens=cu, lens_after=after, want_rows=rows,
                          block_tables=tables, max_new=1 if self.decode else T, max_position=span - 1,
                          max_len_after=span, is_decode=self.decode, host_slots=[], host_new=[])
+        if self.folded:
+            self.step.token_source = (self.src_rows, self.dev[self.cell_at: self.cell_at + 2].view(torch.int64))
         self.fill(None, cache)     # all padding: valid contents while capturing
         self.dev.copy_(self.host)
         engine.model.forward(self.step, cache)      # once eagerly at the bucket's size: what the recording meets exists
@@ -141,6 +150,9 @@ class _Captured:
         if self.copied is not None:
             self.copied.synchronize()      # the last copy out of the host image must be over before it changes
         self.fill(entries, cache)
+        if self.ahead_rows:
+            self.host_np[self.src_at: self.src_at + self.ahead_rows] = -1
+            self.ahead_rows = 0
         self.dev.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
@@ -155,10 +167,15 @@ class _Captured:
         n = packed.n
         self.fill(packed, cache)
         self.host_np[self.src_at: self.src_at + n] = rows
+        if self.ahead_rows > n:
+            self.host_np[self.src_at + n: self.src_at + self.ahead_rows] = -1
+        self.ahead_rows = n
+        self.host_cell[0] = tokens_dev.data_ptr()
         self.dev.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
-        torch.index_select(tokens_dev, 0, self.src_rows[:n], out=self.step.token_ids[:n])
+        if not self.folded:
+            torch.index_select(tokens_dev, 0, self.src_rows[:n], out=self.step.token_ids[:n])
         self.graph.replay()
         return self.logits[:n]      # the graph's own buffer: good until the next replay of this shape
 

@@ -96,7 +96,10 @@ class Model:
 
     def forward(self, step, cache):
         """Logits (float32, [wanted rows, vocab]) of one step, or None when no row is wanted."""
-        h = self.embedding.forward(step.token_ids)
+        if step.token_source is None:
+            h = self.embedding.forward(step.token_ids)
+        else:
+            h = self.embedding.forward_from(step.token_ids, *step.token_source)
         delta = None
         for i, place in enumerate(self.plan.order):
             delta = self.blocks[place.layer].forward(h, delta, step, cache.views[i])

@@ -15,7 +15,6 @@ class Embedding(Part):
     """params: vocab, width.  names: weight."""
     graph_safe = True
 
-
     def tensor_specs(self):
         return {self.names["weight"]: TensorSpec((self.params["vocab"], self.params["width"]))}
 
@@ -30,11 +29,17 @@ class Embedding(Part):
         h = torch.empty(ids.shape[0], self.params["width"], dtype=torch.float32, device=ids.device)
         return self.rt.ops.embed_gather(self.table, ids, h)
 
+    def forward_from(self, ids, source_rows, source_cell):
+        """The same where some tokens are still on the device: row t is element source_rows[t] of the
+        array whose address is in source_cell, where source_rows[t] >= 0.  An embedding without this
+        method gets its tokens gathered by a separate launch before the step."""
+        h = torch.empty(ids.shape[0], self.params["width"], dtype=torch.float32, device=ids.device)
+        return self.rt.ops.embed_gather_from(self.table, ids, source_rows, source_cell, h)
+
 
 class LMHead(Part):
     """params: vocab, width.  names: weight (the embedding's name when tied)."""
     graph_safe = True
-
 
     def tensor_specs(self):
         return {self.names["weight"]: TensorSpec((self.params["vocab"], self.params["width"]))}

@@ -42,6 +42,29 @@ def test_embed_gather(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed_gather_with_tokens_left_on_the_device(ops, dtype):
+    """Rows whose source row is >= 0 take their token from the array whose address is in the cell;
+    the cell is changed between two calls, as between two replays; a token outside the table gives NaN."""
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(333, 72, generator=g).to(DT[dtype])
+    ids = dev(torch.tensor([7, 8, 9, 10, 11, 12], dtype=torch.int32))
+    rows = dev(torch.tensor([2, -1, 0, -1, 1, 2], dtype=torch.int32))
+    cell = torch.zeros(1, dtype=torch.int64, device="cuda")
+    h = torch.empty(6, 72, dtype=torch.float32, device="cuda")
+    for left in ([300, 0, 332], [5, 6, 7, 8]):
+        source = dev(torch.tensor(left, dtype=torch.int32))
+        cell.fill_(source.data_ptr())
+        ops.embed_gather_from(dev(table), ids, rows, cell, h)
+        expect = [left[2], 8, left[0], 10, left[1], left[2]]
+        assert torch.equal(h.cpu(), table[torch.tensor(expect)].float())
+    source = dev(torch.tensor([1, 333, -1], dtype=torch.int32))
+    cell.fill_(source.data_ptr())
+    ops.embed_gather_from(dev(table), ids, rows, cell, h)
+    bad = torch.isnan(h).all(1).cpu().tolist()
+    assert bad == [True, False, False, False, True, True] and not torch.isnan(h[1]).any()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("gamma_dtype", ["float32", "bfloat16"])
 def test_add_rmsnorm(ops, dtype, gamma_dtype):
     g = torch.Generator().manual_seed(1)
