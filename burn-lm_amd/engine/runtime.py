@@ -202,9 +202,11 @@ class Runtime:
                                          gated=True, tile=tile)
             # Long prompts: with whole rounds of 256x256 tiles (as many blocks as compute units, or a
             # multiple) and a narrow model the fused kernel is ahead of the library over the whole
-            # prefill (width 2048: 2-4 % at 1,024 and 2,048 rows, 0.5 % at 3,072 and 4,096; behind by
-            # 2-6 % with a partial last round, and at width 3072 behind from 1,536 rows on).
-            if K <= 2048 and M >= 256 and (-(-M // 256) * -(-inner // 128)) % self.compute_units == 0:
+            # prefill (width 2048: 2-4 % at 1,024 and 2,048 rows, 0.5-0.8 % at 3,072 and 4,096; behind by
+            # 2-6 % with a partial last round, and at width 3072 behind from 1,536 rows on).  Beyond
+            # 4,096 rows the library's large tiles are ahead (whole prefill of 8,192 tokens 19.4 ms
+            # against 20.7, of 16,384 tokens 47.9 against 49.0).
+            if K <= 2048 and 256 <= M <= 4096 and (-(-M // 256) * -(-inner // 128)) % self.compute_units == 0:
                 return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
                                      gated=True, tile=(256, 256))
         if fusable and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]:
