@@ -175,12 +175,11 @@ def kernel_rates(engine, batch, context, prefill_tokens):
 
     def rate(name, calls, nbytes=None, flops=None):
         sec = graph_time(calls)
-        r = {"us": round(sec * 1e6, 2)}
+        out[name + "_us"] = round(sec * 1e6, 2)     # flat keys: a record may drop what lies deeper
         if nbytes is not None:
-            r["gbs"] = round(nbytes / sec / 1e9, 1)
+            out[name + "_gbs"] = round(nbytes / sec / 1e9, 1)
         if flops is not None:
-            r["tflops"] = round(flops / sec / 1e12, 1)
-        out[name] = r
+            out[name + "_tflops"] = round(flops / sec / 1e12, 1)
 
     width = model.plan.width
     m0, f0, v0 = blocks[0][0].mixer, blocks[0][0].feed_forward, blocks[0][1]
