@@ -16,7 +16,7 @@ a batch of 8 and a context of 4096 tokens per sequence.  One JSON line is printe
   live requests, as the model's own parts count them) / its time, against 8 TB/s; ``prefill``: a
   prompt of 2,048 tokens through the step function, its flops / time against the dense bf16 peak.
 * ``points``: decode at batch 1 and 64 at the same context, with their roofline fractions;
-  ``workload_512_256``: the workload BASELINE.json names (512-token prompts, 256 generated tokens, at
+  ``workload_512_256``: the benchmark's second workload (512-token prompts, 256 generated tokens, at
   batch 1, 8 and 64) as decoded tokens a second over the whole decode phase.
 * ``measured``: what this machine reaches with a kernel that only reads (GB/s) and one that only
   issues matrix instructions (TFLOP/s), as second denominators; ``kernels``: time and achieved GB/s
@@ -99,7 +99,7 @@ def time_prefill(engine, T, reps=5):
 
 
 def time_workload(engine, batch, prompt_len=512, generated=256):
-    """BASELINE.json's decode workload through the generation loop: decoded tokens a second over the
+    """The workload of 512-token prompts and 256 generated tokens through the generation loop: decoded tokens a second over the
     decode phase of the second of two runs (the first records the graphs)."""
     from burn_lm_amd.engine.generate import generate
     from burn_lm_amd.sampling.sampler import Sampler
