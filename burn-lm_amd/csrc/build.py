@@ -207,12 +207,13 @@ def find_hipcc():
                        "library cannot be built, and there is no fallback path without it")
 
 
-def build(verbose=True, jobs=None):
+def build(verbose=True, jobs=None, with_ref=False):
     """Compile every HIP source and link the kernel library, and compile the host library.  Always
-    compiles; returns the kernel library's path.  The plain C++ references that the kernel tests use
-    are compiled along."""
+    compiles; returns the kernel library's path.  with_ref: the plain C++ references that the kernel
+    tests use are compiled along (a model's first call does not need them)."""
     build_host(verbose=verbose)
-    build_ref(verbose=verbose)
+    if with_ref:
+        build_ref(verbose=verbose)
     hipcc = find_hipcc()
     od = out_dir()
     bdir = os.path.join(od, "_build")
