@@ -100,11 +100,12 @@ def time_prefill(engine, T, reps=5):
 
 def time_workload(engine, batch, prompt_len=512, generated=256):
     """The workload of 512-token prompts and 256 generated tokens through the generation loop: decoded tokens a second over the
-    decode phase of the second of two runs (the first records the graphs)."""
+    decode phase, and prompt tokens a second over the prompt step, of the third of three runs (a shape
+    is recorded as a graph the second time it is met, so the third run replays the prompt step too)."""
     from burn_lm_amd.engine.generate import generate
     from burn_lm_amd.sampling.sampler import Sampler
     prompts = random_prompts(engine, batch, prompt_len, seed=1)
-    for _ in range(2):
+    for _ in range(3):
         _, stats = generate(engine, prompts, Sampler(temperature=0.0), generated, stop_ids=(), batch_size=batch)
     return stats.decode_tokens / stats.decode_seconds, stats.prompt_tokens / stats.prompt_seconds
 
