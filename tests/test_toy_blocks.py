@@ -1,6 +1,7 @@
 """Other arrangements of a layer, defined here in the test and registered without a change to the
 framework's files: a block with four norms around its two parts (a norm before and one after each),
-and a block that has a mixer and no feed-forward at all.  The feed-forward of the first is a toy that
+a block that has a mixer and no feed-forward at all, and a block whose mixer and feed-forward read
+the same normalised rows side by side.  The feed-forward of the first is a toy that
 needs an integer table, which the random-weights mode makes from the toy architecture's own list of
 checkpoint tensors.  The toy is no model of anyone's."""
 import json
@@ -11,7 +12,7 @@ import torch
 
 import plain_llama as P
 
-TOY = dict(architectures=["ToyBlocksLM"], width=96, heads=6, kv_heads=3, head_dim=16, vocab=203, eps=1e-5,
+TOY = dict(architectures=["ToyBlocksLM"], width=96, inner=136, heads=6, kv_heads=3, head_dim=16, vocab=203, eps=1e-5,
            theta=10000.0, max_positions=256)
 
 
@@ -52,6 +53,18 @@ def register_toy():
             f = self.feed_forward.forward(x, step)
             return self.post_ffn_norm.add_norm(f.float().contiguous(), None, write_h=False)
 
+    class ParallelBlock(Block):
+        """y = x + mixer(norm(x)) + ffn(norm(x)): both parts read the same normalised rows; what they
+        give is handed on as two float32 planes, which the next norm's add sums."""
+        roles = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+
+        def forward(self, h, delta, step, view):
+            x = self.norm.add_norm(h, delta)
+            planes = []
+            for d in (self.mixer.forward(x, step, view), self.feed_forward.forward(x, step)):
+                planes += list(d.float()) if d.dim() == 3 else [d.float()]
+            return torch.stack(planes).contiguous()
+
     class MixerOnlyBlock(Block):
         """y = x + mixer(norm(x)): a layer without a feed-forward."""
         roles = {"mixer_norm": "norm", "mixer": "mixer"}
@@ -69,10 +82,13 @@ def register_toy():
                             post_mixer_norm=norm("l0.n2"), pre_ffn_norm=norm("l0.n3"),
                             feed_forward=PartSpec("toy_gather", dict(width=D), dict(table="l0.table", scale="l0.scale")),
                             post_ffn_norm=norm("l0.n4")),
-                  LayerPlan("toy_mixer_only", {"mixer_norm": norm("l1.n1"), "mixer": attn(1)}, position="rope")]
+                  LayerPlan("toy_mixer_only", {"mixer_norm": norm("l1.n1"), "mixer": attn(1)}, position="rope"),
+                  LayerPlan("toy_parallel", position="rope", norm=norm("l2.n1"), mixer=attn(2),
+                            feed_forward=PartSpec("swiglu", dict(width=D, inner=cfg["inner"]),
+                                                  dict(gate="l2.gate", up="l2.up", down="l2.down")))]
         return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
                          embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
-                         layers=layers, order=[Place(0), Place(1)], final_norm=norm("norm"),
+                         layers=layers, order=[Place(0), Place(1), Place(2)], final_norm=norm("norm"),
                          head=PartSpec("linear", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
                          positions={"rope": PartSpec("rope", dict(head_dim=cfg["head_dim"], theta=cfg["theta"],
                                                                   pairing="interleaved", scaling=None))})
@@ -80,10 +96,12 @@ def register_toy():
     def checkpoint_tensors(cfg):
         D, hd = cfg["width"], cfg["head_dim"]
         t = {"emb": ((cfg["vocab"], D), "table"), "norm": ((D,), "norm"), "l0.table": ((D,), IntegerTable(D)),
-             "l0.scale": ((D,), Normal(std=0.5)), "l1.n1": ((D,), "norm")}
+             "l0.scale": ((D,), Normal(std=0.5)), "l1.n1": ((D,), "norm"), "l2.n1": ((D,), "norm"),
+             "l2.gate": ((cfg["inner"], D), "matrix"), "l2.up": ((cfg["inner"], D), "matrix"),
+             "l2.down": ((D, cfg["inner"]), "matrix")}
         for n in ("n1", "n2", "n3", "n4"):
             t[f"l0.{n}"] = ((D,), "norm")
-        for i in (0, 1):
+        for i in (0, 1, 2):
             t.update({f"l{i}.q": ((cfg["heads"] * hd, D), "matrix"), f"l{i}.k": ((cfg["kv_heads"] * hd, D), "matrix"),
                       f"l{i}.v": ((cfg["kv_heads"] * hd, D), "matrix"), f"l{i}.o": ((D, cfg["heads"] * hd), "matrix")})
         return t
@@ -91,6 +109,7 @@ def register_toy():
     registry.register_part("feed_forward", "toy_gather", GatherFeedForward)
     registry.register_part("block", "toy_sandwich", SandwichBlock)
     registry.register_part("block", "toy_mixer_only", MixerOnlyBlock)
+    registry.register_part("block", "toy_parallel", ParallelBlock)
     registry.register_architecture(registry.Architecture("ToyBlocksLM", read_config=lambda d: d, plan=plan,
                                                          checkpoint_tensors=checkpoint_tensors))
 
@@ -107,12 +126,14 @@ def toy_plain(tokens, w):
     x = n(h, "l0.n3")
     h = h + n(x[..., w["l0.table"].astype(np.int64)] * w["l0.scale"], "l0.n4")
     h = h + attn(n(h, "l1.n1"), 1)
+    x = n(h, "l2.n1")
+    h = h + attn(x, 2) + P.swiglu_feed_forward(x, w["l2.gate"], w["l2.up"], w["l2.down"])
     return (n(h, "norm") @ w["emb"].T)[0]
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
-def test_a_block_with_four_norms_and_a_layer_without_a_feed_forward(tmp_path, dtype, tol):
+def test_a_block_with_four_norms_a_layer_without_a_feed_forward_and_a_parallel_block(tmp_path, dtype, tol):
     import burn_lm_amd
     from burn_lm_amd.engine.loading import load_engine
     from burn_lm_amd.weights import safetensors_io as st
@@ -125,8 +146,8 @@ def test_a_block_with_four_norms_and_a_layer_without_a_feed_forward(tmp_path, dt
     w = {k: v.double().numpy() for k, v in stored.items()}
     eng = load_engine(folder, dtype=dtype, max_tokens=1024, max_seqs=4)
     kinds = [type(b).__name__ for b in eng.model.blocks]
-    assert kinds == ["SandwichBlock", "MixerOnlyBlock"] and not hasattr(eng.model.blocks[1], "feed_forward")
-    assert len(eng.model.blocks[0].parts()) == 6 and len(eng.model.blocks[1].parts()) == 2
+    assert kinds == ["SandwichBlock", "MixerOnlyBlock", "ParallelBlock"] and not hasattr(eng.model.blocks[1], "feed_forward")
+    assert [len(b.parts()) for b in eng.model.blocks] == [6, 2, 3]
     rng = np.random.default_rng(3)
     reqs = [[int(x) for x in rng.integers(0, TOY["vocab"], L)] for L in (130, 11, 66)]
     want = [toy_plain(r, w) for r in reqs]
