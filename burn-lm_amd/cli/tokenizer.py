@@ -65,3 +65,39 @@ def for_folder(folder: str, vocab_size: int, special_tokens=None):
         raise ValueError(f"the byte tokenizer needs a vocabulary of at least 256, the model has {vocab_size}; "
                          f"pass token ids instead of text")
     return ByteTokenizer()
+
+
+class StreamingDecoder:
+    """Text of a growing list of tokens, piece by piece.  A token decoded on its own can lose what
+    it shares with its neighbours (a leading space, the bytes of one character spread over two
+    tokens), so a piece is what decoding the last emitted tokens *with* the new ones adds to decoding
+    them alone: two tokens of overlap, as the reference does
+    (crates/burn-lm-llama/src/generation/streaming.rs:10-57).  A piece that would end in half a
+    character is held back until the character is whole."""
+    OVERLAP = 2
+
+    def __init__(self, tokenizer):
+        self.tokenizer = tokenizer
+        self.tokens = []
+        self.emitted = 0
+
+    def push(self, token):
+        """-> the text this token completes ('' if it has to wait for the next one)."""
+        self.tokens.append(token)
+        start = max(0, self.emitted - self.OVERLAP)
+        whole = self.tokenizer.decode(self.tokens[start:])
+        before = self.tokenizer.decode(self.tokens[start:self.emitted])
+        if whole.endswith("\ufffd") or not whole.startswith(before):
+            return ""
+        piece = whole[len(before):]
+        if piece:
+            self.emitted = len(self.tokens)
+        return piece
+
+    def flush(self):
+        """What is still held back when the tokens end (half a character comes out as it decodes)."""
+        start = max(0, self.emitted - self.OVERLAP)
+        whole = self.tokenizer.decode(self.tokens[start:])
+        before = self.tokenizer.decode(self.tokens[start:self.emitted])
+        self.emitted = len(self.tokens)
+        return whole[len(before):] if whole.startswith(before) else ""

@@ -17,6 +17,7 @@ from dataclasses import asdict, dataclass, fields
 from typing import Callable, List, Optional, Sequence
 
 from .engine.generate import ContextLengthExceeded, generate
+from .cli.tokenizer import StreamingDecoder
 from .engine.stats import Stats
 from .sampling.sampler import Sampler
 
@@ -187,18 +188,20 @@ class InferenceServer:
         tok = self._tokenizer()
         ids = tok.encode(text, False, False)  # no BOS/EOS added (nn/llama/inference.rs:35-40)
         stop = set(self.stop_ids())
-        pending: List[int] = []
+        pieces = StreamingDecoder(tok)
 
         def emit(_, t):
             if on_text is None or t in stop:
                 return
-            pending.append(t)
-            s = tok.decode(pending)
-            if s and not s.endswith("�"):
+            s = pieces.push(t)
+            if s:
                 on_text(s)
-                pending.clear()
 
         results, stats = self.generate([ids], on_token=emit, **options)
+        if on_text is not None:
+            rest = pieces.flush()
+            if rest:
+                on_text(rest)
         r = results[0]
         if r.finish_reason == "error":
             if len(ids) > self.engine.max_context:

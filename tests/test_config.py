@@ -190,3 +190,37 @@ def test_command_line_random_models_delete(tmp_path, monkeypatch, capsys):
     main(["random", "llama3.2-1b-test", "--name", "second", "--seed", "3"])
     main(["delete", "all"])
     assert sorted(p.name for p in (tmp_path / "models").iterdir()) == []
+
+
+def test_text_comes_out_piece_by_piece_as_the_whole_would():
+    """The streaming decoder against two tokenizers whose tokens cannot be decoded one by one: bytes
+    (a character of several bytes spans tokens) and a word tokenizer that puts a space between the
+    words of one call and none in front of the first (crates/burn-lm-llama/src/generation/streaming.rs:10-57)."""
+    from burn_lm_amd.cli.tokenizer import ByteTokenizer, StreamingDecoder
+
+    text = "héllo wörld — ça va? 日本語"
+    ids = ByteTokenizer().encode(text)
+    dec = StreamingDecoder(ByteTokenizer())
+    pieces = [dec.push(t) for t in ids]
+    assert "".join(pieces) + dec.flush() == text
+    assert all("�" not in p for p in pieces) and any(p == "" for p in pieces)   # half characters are held back
+
+    class Words:
+        vocab = ["the", "quick", "brown", "fox", ",", "jumps"]
+
+        def decode(self, tokens):
+            out = ""
+            for i, t in enumerate(tokens):
+                w = self.vocab[t]
+                out += w if i == 0 or w == "," else " " + w
+            return out
+
+    ids = [0, 1, 2, 3, 4, 5, 0, 3]
+    dec = StreamingDecoder(Words())
+    pieces = [dec.push(t) for t in ids]
+    assert "".join(pieces) + dec.flush() == Words().decode(ids) == "the quick brown fox, jumps the fox"
+    assert pieces[1] == " quick"          # decoded alone it would have lost its space
+    # tokens that end in the middle of a character at the end of the text come out with the flush
+    dec = StreamingDecoder(ByteTokenizer())
+    cut = ByteTokenizer().encode("aé")[:-1]
+    assert [dec.push(t) for t in cut] == ["a", ""] and dec.flush() == "�"
