@@ -63,10 +63,55 @@ __global__ void __launch_bounds__(MAXT)
   // that all advance through the matrix side by side)
   const int tiles_per_block = (n_tiles + gridDim.x - 1) / gridDim.x;
   const int tile_begin = blockIdx.x * tiles_per_block, tile_end = min(n_tiles, tile_begin + tiles_per_block);
+  // 16 k-steps per wavefront: the weights come in two halves of eight fragments, and each half's
+  // registers are asked for the next tile's weights as soon as the matrix instructions that read them
+  // have been issued, so loads are on their way while the other half is multiplied and while the
+  // block sums its tile.  (All blocks start together; without this they also wait together, and
+  // the memory idles whenever they multiply and sum: gate/up with 16 rows 14.5 us instead of 15.9,
+  // with 8 rows 13.7 instead of 14.3, the head 84-86 instead of 87.5.  No more registers than the
+  // sixteen fragments of one tile.)
+  constexpr bool PIPE = KSTEPS == 16 && KEEP_A;
+  constexpr int HALF = KSTEPS / 2;
+  uint4 wa[PIPE ? HALF : 1], wb[PIPE ? HALF : 1];
+  int woff[PIPE ? KSTEPS : 1];
+  if (PIPE) {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) woff[s] = (step0 + s < k_steps ? step0 + s : k_steps - 1) * 512;
+    const bf16* wt = Wp + ((size_t)min(tile_begin, n_tiles - 1) * k_steps * 64 + lane) * 8;
+#pragma unroll
+    for (int s = 0; s < HALF; ++s) wa[s] = ld16_stream(wt + woff[s]);
+#pragma unroll
+    for (int s = 0; s < HALF; ++s) wb[s] = ld16_stream(wt + woff[HALF + s]);
+  }
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const bf16* wt = Wp + ((size_t)tile * k_steps * 64 + lane) * 8;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     constexpr int CH = KSTEPS < 16 ? KSTEPS : 16;   // weight loads in flight per wavefront
+    if (PIPE) {
+      const bool more = tile + 1 < tile_end;
+      const bf16* wnext = Wp + ((size_t)(tile + 1) * k_steps * 64 + lane) * 8;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < HALF; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
+                                                      __builtin_bit_cast(bf16x8_t, wa[s]), acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) {
+#pragma unroll
+        for (int s = 0; s < HALF; ++s) wa[s] = ld16_stream(wnext + woff[s]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < HALF; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[HALF + s]),
+                                                      __builtin_bit_cast(bf16x8_t, wb[s]), acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) {
+#pragma unroll
+        for (int s = 0; s < HALF; ++s) wb[s] = ld16_stream(wnext + woff[HALF + s]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    } else
 #pragma unroll
     for (int c = 0; c < KSTEPS; c += CH) {
       uint4 w[CH];
