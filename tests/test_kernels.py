@@ -435,6 +435,7 @@ def test_pack_weight_layout(ops):
 @pytest.mark.parametrize("M,N,K", [(1, 1001, 264), (8, 48, 64), (7, 130, 144), (16, 16, 512), (11, 333, 520),
                                    (8, 257, 2048), (3, 40, 8192), (16, 100, 8200), (5, 31, 14336), (9, 77, 4104),
                                    (2, 9000, 264), (8, 8200, 1024), (6, 100, 4096), (4, 52, 600),
+                                   (5, 25000, 1000), (3, 17000, 3080),     # four and five tiles per block, the last block short
                                    (17, 130, 264), (32, 48, 2048), (29, 5000, 2040), (33, 77, 2048), (32, 200, 4096), (20, 1000, 3072), (48, 257, 520),
                                    (47, 16, 64), (49, 300, 1032), (64, 4200, 2048), (61, 40, 136), (35, 20000, 520), (64, 12300, 2048)])
 def test_gemv_mfma(ops, out_dtype, M, N, K):
@@ -494,7 +495,7 @@ def test_gemv_mfma_partial_products_are_summed_by_the_norm(ops, M, N, K, groups)
     assert torch.equal(out2.cpu(), out.cpu()[rows.long()]) and torch.equal(hd2.cpu(), h)
 
 
-@pytest.mark.parametrize("M,I,K", [(8, 176, 64), (3, 384, 144), (16, 8, 520), (5, 1000, 2048), (1, 64, 4104),
+@pytest.mark.parametrize("M,I,K", [(8, 176, 64), (3, 384, 144), (16, 8, 520), (5, 1000, 2048), (1, 64, 4104), (4, 20000, 2048),
                                    (64, 1000, 2048), (20, 176, 1544), (37, 384, 144), (50, 8, 520), (32, 176, 4096)])
 def test_gemv_mfma_gated(ops, M, I, K):
     """The SwiGLU gating in the epilogue of the product that computes gate and up: the packed copy pairs
