@@ -38,8 +38,16 @@ struct Vec8<float> {
 
 #define ATTN_WAVES 4
 #define ATTN_MAX_HD 256
+#define ATTN_STAGE_LDS (64 * 1024)       // most shared memory of the form that stages values, as a kernel gets it without asking
+#define ATTN_STAGE_LDS_BIG (144 * 1024)  // and after blm_attn_paged_init on the device (head sizes up to 128 in four wavefronts)
 
-template <typename TA, bool VEC>
+// STAGE: the values of a chunk of 64 keys go through shared memory.  A value page keeps a head lane's
+// tokens next to each other, so with one lane per key the 64 lanes read 64 neighbouring values per
+// head lane (one line), and write them transposed into a tile of the wavefront's own ([key][lane],
+// rows padded by one float); the weighted sum then reads the tile with one lane per head lane.
+// Without it every lane reads 4 bytes of a line of its own for every key.  The tile is 64 * (hd + 1)
+// floats per wavefront.
+template <typename TA, bool VEC, bool STAGE>
 __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
     attn_paged_kernel(const TA* __restrict__ q, int q_row_stride, TA* __restrict__ out,
                       const int* __restrict__ positions, const int* __restrict__ token_seq,
@@ -55,6 +63,7 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
   const int head = active ? (int)(w - (long long)t * nh) : 0;
   const int b = active ? token_seq[t] : -1;
   float* qs = smem + wave * hd;
+  float* vt = smem + ATTN_WAVES * hd + (size_t)wave * BLM_WAVE * (hd + 1);   // STAGE: this wavefront's tile of values
   if (active && b >= 0) {
     const TA* qrow = q + (size_t)t * q_row_stride + (size_t)head * hd;
     for (int d = lane; d < hd; d += BLM_WAVE) qs[d] = to_float(qrow[d]);
@@ -107,6 +116,25 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
 #pragma unroll
     for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) acc[i] *= corr;
     const int cnt = (j_end - j0 + 1) < BLM_WAVE ? (j_end - j0 + 1) : BLM_WAVE;
+    if (STAGE) {
+      if (valid) {
+        const int page = bt[j / page_size];
+        const TA* vcol = vcache + ((size_t)page * nkv + kvh) * page_size * hd + (j % page_size);
+        float* mine = vt + (size_t)lane * (hd + 1);
+        for (int d = 0; d < hd; ++d) mine[d] = to_float(vcol[(size_t)d * page_size]);
+      }
+      __builtin_amdgcn_wave_barrier();   // the tile is the wavefront's own: its reads follow its writes in order
+      for (int jj = 0; jj < cnt; ++jj) {
+        const float pj = __shfl(p, jj, BLM_WAVE);
+        const float* vrow = vt + (size_t)jj * (hd + 1);
+#pragma unroll
+        for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) {
+          const int d = lane + i * BLM_WAVE;
+          if (d < hd) acc[i] = fmaf(pj, vrow[d], acc[i]);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();   // the next chunk's writes follow these reads
+    } else
     for (int jj = 0; jj < cnt; ++jj) {
       const float pj = __shfl(p, jj, BLM_WAVE);
       const int ja = j0 + jj;
@@ -176,6 +204,25 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
   }
 }
 
+// Once per device, outside any stream capture: lets the form that stages values ask for more shared
+// memory than a kernel gets without asking.  Without it that form serves head sizes up to 62 only.
+#define ATTN_DEVICES 64
+static bool g_attn_big_lds[ATTN_DEVICES];
+extern "C" int blm_attn_paged_init() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  BLM_REQUIRE(e == hipSuccess && dev >= 0, "attn_paged_init: hipGetDevice failed: %s", hipGetErrorString(e));
+  if (dev >= ATTN_DEVICES) return 0;   // such a device keeps the small limit
+  const void* kernels[] = {(const void*)attn_paged_kernel<float, true, true>, (const void*)attn_paged_kernel<float, false, true>,
+                           (const void*)attn_paged_kernel<bf16, true, true>, (const void*)attn_paged_kernel<bf16, false, true>};
+  for (const void* k : kernels) {
+    e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, ATTN_STAGE_LDS_BIG);
+    BLM_REQUIRE(e == hipSuccess, "attn_paged_init: cannot raise the shared memory limit: %s", hipGetErrorString(e));
+  }
+  g_attn_big_lds[dev] = true;
+  return 0;
+}
+
 // part_o: T*nh*n_splits*hd floats, part_ml: T*nh*n_splits*2 floats, arrivals: T*nh ints that are
 // zero before the first call (every call leaves them zero again); all three may be null when
 // n_splits is 1.  Calls that share the arrivals buffer must not overlap in time.
@@ -196,19 +243,27 @@ extern "C" int blm_attn_paged(const void* q, int q_row_stride, void* out, int ac
   const long long blocks = (items + ATTN_WAVES - 1) / ATTN_WAVES;
   BLM_REQUIRE(blocks < 2147483647LL, "attn_paged: too many (token, head) pairs: %lld", items);
   dim3 grid((unsigned)blocks, (unsigned)n_splits), block(ATTN_WAVES * BLM_WAVE);
-  const size_t smem = (size_t)ATTN_WAVES * hd * sizeof(float);
+  // the values' tiles fit the shared memory a kernel gets without asking up to a head size of 62, after
+  // blm_attn_paged_init up to 139; larger heads take the direct form
+  const size_t tiles = (size_t)ATTN_WAVES * BLM_WAVE * (hd + 1) * sizeof(float);
+  int dev = -1;
+  const bool big = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < ATTN_DEVICES && g_attn_big_lds[dev];
+  const bool stage = (size_t)ATTN_WAVES * hd * sizeof(float) + tiles <= (size_t)(big ? ATTN_STAGE_LDS_BIG : ATTN_STAGE_LDS);
+  const size_t smem = (size_t)ATTN_WAVES * hd * sizeof(float) + (stage ? tiles : 0);
   const bool vec = (hd % 8) == 0 && (q_row_stride % 8) == 0;
-#define BLM_ATTN_CASE(TA, V)                                                                        \
-  hipLaunchKernelGGL((attn_paged_kernel<TA, V>), grid, block, smem, stream, (const TA*)q, q_row_stride, \
+#define BLM_ATTN_CASE(TA, V, S)                                                                     \
+  hipLaunchKernelGGL((attn_paged_kernel<TA, V, S>), grid, block, smem, stream, (const TA*)q, q_row_stride, \
                      (TA*)out, positions, token_seq, block_table, table_width, (const TA*)kcache,    \
                      (const TA*)vcache, page_size, T, nh, nkv, hd, scale, window, n_splits, part_o, part_ml, arrivals)
-  if (act_dtype == BLM_F32) {
-    if (vec) BLM_ATTN_CASE(float, true); else BLM_ATTN_CASE(float, false);
-  } else if (act_dtype == BLM_BF16) {
-    if (vec) BLM_ATTN_CASE(bf16, true); else BLM_ATTN_CASE(bf16, false);
-  } else {
-    return blm_fail("attn_paged: unsupported dtype %d", act_dtype);
-  }
+#define BLM_ATTN_PICK(TA)                                                                           \
+  do {                                                                                              \
+    if (stage) { if (vec) BLM_ATTN_CASE(TA, true, true); else BLM_ATTN_CASE(TA, false, true); }     \
+    else { if (vec) BLM_ATTN_CASE(TA, true, false); else BLM_ATTN_CASE(TA, false, false); }         \
+  } while (0)
+  if (act_dtype == BLM_F32) BLM_ATTN_PICK(float);
+  else if (act_dtype == BLM_BF16) BLM_ATTN_PICK(bf16);
+  else return blm_fail("attn_paged: unsupported dtype %d", act_dtype);
+#undef BLM_ATTN_PICK
 #undef BLM_ATTN_CASE
   BLM_LAUNCH_CHECK("attn_paged");
   return 0;

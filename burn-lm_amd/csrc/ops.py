@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 _lib = None
 _lock = threading.Lock()
 
@@ -49,6 +49,7 @@ _SIGNATURES = {
                       _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_gemm_mfma_init": [],
+    "blm_attn_paged_init": [],
     "blm_gemm_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_void_p],
     "blm_gemv_mfma_group_limit": [_c_int],
@@ -545,6 +546,20 @@ def gemm_mfma_init(device=None):
         with torch.cuda.device(index):
             _call("blm_gemm_mfma_init")
         _gemm_ready.add(index)
+
+
+_attn_ready = set()
+
+
+def attn_paged_init(device=None):
+    """Once per device, outside any stream capture: lets attn_paged stage the values of head sizes
+    above 62 (up to 139) through shared memory."""
+    index = torch.device(device or "cuda").index
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _attn_ready:
+        with torch.cuda.device(index):
+            _call("blm_attn_paged_init")
+        _attn_ready.add(index)
 
 
 _static_ready = set()

@@ -59,6 +59,7 @@ class Runtime:
         ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
         ops.static_scratch_init(self.device)   # likewise: the address of the library's own scratch array
         ops.grid_sync(self.device)             # likewise: the counters and the fault word of resident-grid kernels
+        ops.attn_paged_init(self.device)       # likewise: the shared memory of the generic attention's value tiles
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         asked = os.environ.get("BURN_LM_AMD_FUSED_GATE_UP")   # "1": wherever it can run, "0": nowhere, unset: where it is ahead
         self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if asked == "1" else (0, -1)

@@ -182,7 +182,9 @@ def _attn_ref(q, keys, values, pos, scale, window, n_rep):
                                                (3, 1, 200, 0), (4, 2, 32, 37)])
 def test_attn_paged(ops, dtype, nh, nkv, hd, window, splits):
     """The generic kernel, whole key ranges and ranges cut into pieces that are merged by the last
-    wavefront to finish (more pieces than some sequences have chunks of keys: empty pieces)."""
+    wavefront to finish (more pieces than some sequences have chunks of keys: empty pieces).  Head
+    sizes up to 128 run the form that stages values through shared memory, 200 the direct one."""
+    ops.attn_paged_init()
     g = torch.Generator().manual_seed(4)
     page, n_pages = 16, 40
     lens = [150, 1, 70]          # cached length of three sequences after this step
