@@ -47,7 +47,7 @@ struct Vec8<float> {
 // rows padded by one float); the weighted sum then reads the tile with one lane per head lane.
 // Without it every lane reads 4 bytes of a line of its own for every key.  The tile is 64 * (hd + 1)
 // floats per wavefront.
-template <typename TA, bool VEC, bool STAGE>
+template <typename TA, bool VEC, bool STAGE, bool SHARE>
 __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
     attn_paged_kernel(const TA* __restrict__ q, int q_row_stride, TA* __restrict__ out,
                       const int* __restrict__ positions, const int* __restrict__ token_seq,
@@ -55,6 +55,8 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
                       const TA* __restrict__ kcache, const TA* __restrict__ vcache, int page_size,
                       int T, int nh, int nkv, int hd, float scale, int window, int n_splits, float* part_o,
                       float* part_ml, int* arrivals) {
+  static_assert(STAGE || !SHARE, "shared tiles are staged tiles");
+  constexpr bool share = SHARE;
   extern __shared__ float smem[];
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const long long w = (long long)blockIdx.x * ATTN_WAVES + wave;
@@ -63,7 +65,11 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
   const int head = active ? (int)(w - (long long)t * nh) : 0;
   const int b = active ? token_seq[t] : -1;
   float* qs = smem + wave * hd;
-  float* vt = smem + ATTN_WAVES * hd + (size_t)wave * BLM_WAVE * (hd + 1);   // STAGE: this wavefront's tile of values
+  // STAGE: this wavefront's tile of values; with `share` (the block's wavefronts are heads of one group
+  // and work on the same token: groups of a multiple of four heads) one tile of keys and one of values
+  // for the whole block, filled by all its threads, so the group's keys and values are read once
+  float* kt = smem + ATTN_WAVES * hd;
+  float* vt = share ? kt + (size_t)BLM_WAVE * (hd + 1) : kt + (size_t)wave * BLM_WAVE * (hd + 1);
   if (active && b >= 0) {
     const TA* qrow = q + (size_t)t * q_row_stride + (size_t)head * hd;
     for (int d = lane; d < hd; d += BLM_WAVE) qs[d] = to_float(qrow[d]);
@@ -93,7 +99,32 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
     const int j = j0 + lane;
     const bool valid = j <= j_end;
     float s = -INFINITY;
-    if (valid) {
+    if constexpr (SHARE) {
+      __syncthreads();   // nobody reads the last chunk's tiles any more
+      {   // keys: four threads per key, neighbouring threads neighbouring lanes of the head
+        const int key = threadIdx.x >> 2, jk = j0 + key;
+        if (jk <= j_end) {
+          const int page = bt[jk / page_size];
+          const TA* krow = kcache + (((size_t)page * nkv + kvh) * page_size + (jk % page_size)) * hd;
+          for (int d = threadIdx.x & 3; d < hd; d += 4) kt[(size_t)key * (hd + 1) + d] = to_float(krow[d]);
+        }
+      }
+      {   // values: a wavefront reads the 64 keys of one head lane, which are neighbours in the page
+        const int jk = j0 + lane;
+        if (jk <= j_end) {
+          const int page = bt[jk / page_size];
+          const TA* vcol = vcache + ((size_t)page * nkv + kvh) * page_size * hd + (jk % page_size);
+          for (int d = wave; d < hd; d += ATTN_WAVES) vt[(size_t)lane * (hd + 1) + d] = to_float(vcol[(size_t)d * page_size]);
+        }
+      }
+      __syncthreads();
+      if (valid) {
+        const float* krow = kt + (size_t)lane * (hd + 1);
+        float dot = 0.f;
+        for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], krow[d], dot);
+        s = dot * scale;
+      }
+    } else if (valid) {
       const int page = bt[j / page_size];
       const TA* krow = kcache + (((size_t)page * nkv + kvh) * page_size + (j % page_size)) * hd;
       float dot = 0.f;
@@ -117,7 +148,7 @@ __global__ void __launch_bounds__(ATTN_WAVES* BLM_WAVE)
     for (int i = 0; i < ATTN_MAX_HD / BLM_WAVE; ++i) acc[i] *= corr;
     const int cnt = (j_end - j0 + 1) < BLM_WAVE ? (j_end - j0 + 1) : BLM_WAVE;
     if (STAGE) {
-      if (valid) {
+      if (valid && !share) {
         const int page = bt[j / page_size];
         const TA* vcol = vcache + ((size_t)page * nkv + kvh) * page_size * hd + (j % page_size);
         float* mine = vt + (size_t)lane * (hd + 1);
@@ -213,8 +244,10 @@ extern "C" int blm_attn_paged_init() {
   hipError_t e = hipGetDevice(&dev);
   BLM_REQUIRE(e == hipSuccess && dev >= 0, "attn_paged_init: hipGetDevice failed: %s", hipGetErrorString(e));
   if (dev >= ATTN_DEVICES) return 0;   // such a device keeps the small limit
-  const void* kernels[] = {(const void*)attn_paged_kernel<float, true, true>, (const void*)attn_paged_kernel<float, false, true>,
-                           (const void*)attn_paged_kernel<bf16, true, true>, (const void*)attn_paged_kernel<bf16, false, true>};
+  const void* kernels[] = {(const void*)attn_paged_kernel<float, true, true, false>, (const void*)attn_paged_kernel<float, false, true, false>,
+                           (const void*)attn_paged_kernel<bf16, true, true, false>,  (const void*)attn_paged_kernel<bf16, false, true, false>,
+                           (const void*)attn_paged_kernel<float, true, true, true>,  (const void*)attn_paged_kernel<float, false, true, true>,
+                           (const void*)attn_paged_kernel<bf16, true, true, true>,   (const void*)attn_paged_kernel<bf16, false, true, true>};
   for (const void* k : kernels) {
     e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, ATTN_STAGE_LDS_BIG);
     BLM_REQUIRE(e == hipSuccess, "attn_paged_init: cannot raise the shared memory limit: %s", hipGetErrorString(e));
@@ -245,20 +278,26 @@ extern "C" int blm_attn_paged(const void* q, int q_row_stride, void* out, int ac
   dim3 grid((unsigned)blocks, (unsigned)n_splits), block(ATTN_WAVES * BLM_WAVE);
   // the values' tiles fit the shared memory a kernel gets without asking up to a head size of 62, after
   // blm_attn_paged_init up to 139; larger heads take the direct form
-  const size_t tiles = (size_t)ATTN_WAVES * BLM_WAVE * (hd + 1) * sizeof(float);
+  // heads of one group in one block: the group's keys and values are staged once for all of them.  Only
+  // where blocks are plentiful (prompts): the block then meets twice per chunk, which a decode step's few
+  // blocks cannot hide (float32 at the 1B shape: prefill of 2,048 tokens 120 ms against 164, but a
+  // decode step of batch 8 4.7 ms against 4.3).
+  const int share = ((nh / nkv) % ATTN_WAVES == 0 && blocks >= 2048) ? 1 : 0;
+  const size_t tiles = (size_t)(share ? 2 : ATTN_WAVES) * BLM_WAVE * (hd + 1) * sizeof(float);
   int dev = -1;
   const bool big = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < ATTN_DEVICES && g_attn_big_lds[dev];
   const bool stage = (size_t)ATTN_WAVES * hd * sizeof(float) + tiles <= (size_t)(big ? ATTN_STAGE_LDS_BIG : ATTN_STAGE_LDS);
   const size_t smem = (size_t)ATTN_WAVES * hd * sizeof(float) + (stage ? tiles : 0);
   const bool vec = (hd % 8) == 0 && (q_row_stride % 8) == 0;
-#define BLM_ATTN_CASE(TA, V, S)                                                                     \
-  hipLaunchKernelGGL((attn_paged_kernel<TA, V, S>), grid, block, smem, stream, (const TA*)q, q_row_stride, \
+#define BLM_ATTN_CASE(TA, V, S, H)                                                                  \
+  hipLaunchKernelGGL((attn_paged_kernel<TA, V, S, H>), grid, block, smem, stream, (const TA*)q, q_row_stride, \
                      (TA*)out, positions, token_seq, block_table, table_width, (const TA*)kcache,    \
                      (const TA*)vcache, page_size, T, nh, nkv, hd, scale, window, n_splits, part_o, part_ml, arrivals)
 #define BLM_ATTN_PICK(TA)                                                                           \
   do {                                                                                              \
-    if (stage) { if (vec) BLM_ATTN_CASE(TA, true, true); else BLM_ATTN_CASE(TA, false, true); }     \
-    else { if (vec) BLM_ATTN_CASE(TA, true, false); else BLM_ATTN_CASE(TA, false, false); }         \
+    if (stage && share) { if (vec) BLM_ATTN_CASE(TA, true, true, true); else BLM_ATTN_CASE(TA, false, true, true); } \
+    else if (stage) { if (vec) BLM_ATTN_CASE(TA, true, true, false); else BLM_ATTN_CASE(TA, false, true, false); }   \
+    else { if (vec) BLM_ATTN_CASE(TA, true, false, false); else BLM_ATTN_CASE(TA, false, false, false); }            \
   } while (0)
   if (act_dtype == BLM_F32) BLM_ATTN_PICK(float);
   else if (act_dtype == BLM_BF16) BLM_ATTN_PICK(bf16);

@@ -179,11 +179,12 @@ def _attn_ref(q, keys, values, pos, scale, window, n_rep):
 @pytest.mark.parametrize("splits", [1, 2, 5])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (6, 1, 24, 0), (5, 5, 64, 0), (8, 2, 128, 0),
-                                               (3, 1, 200, 0), (4, 2, 32, 37)])
+                                               (3, 1, 200, 0), (4, 2, 32, 37), (8, 1, 48, 21), (4, 1, 64, 0)])
 def test_attn_paged(ops, dtype, nh, nkv, hd, window, splits):
     """The generic kernel, whole key ranges and ranges cut into pieces that are merged by the last
     wavefront to finish (more pieces than some sequences have chunks of keys: empty pieces).  Head
-    sizes up to 128 run the form that stages values through shared memory, 200 the direct one."""
+    sizes up to 128 run the form that stages values through shared memory (groups of four and eight
+    heads share one tile of keys and one of values per block), 200 the direct one."""
     ops.attn_paged_init()
     g = torch.Generator().manual_seed(4)
     page, n_pages = 16, 40
@@ -229,6 +230,51 @@ def test_attn_paged(ops, dtype, nh, nkv, hd, window, splits):
         want = _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[b], values[b], positions[t], scale, window, nh // nkv)
         close(got[t], want, EPS[dtype] * 2)
     assert bool((got[T - 1] == 0).all()), "a padding token gives zeros"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,window", [(8, 2, 32, 0), (4, 1, 64, 300)])
+def test_attn_paged_prompt_of_many_tokens(ops, dtype, nh, nkv, hd, window):
+    """A prompt long enough that the generic kernel has blocks in plenty: the four heads of a group then
+    share one tile of keys and one of values per block.  Two sequences in one step, pages scattered."""
+    ops.attn_paged_init()
+    g = torch.Generator().manual_seed(9)
+    page, lens = 16, [2200 if nh == 4 else 1100, 130]
+    n_pages = sum((L + page - 1) // page for L in lens) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.full((2, (max(lens) + page - 1) // page), -1, dtype=torch.int32)
+    kc = torch.full((n_pages, nkv, page, hd), float("nan"))
+    vc = torch.full((n_pages, nkv, hd, page), float("nan"))
+    keys, values, positions, token_seq = [], [], [], []
+    for b, L in enumerate(lens):
+        kb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
+        vb = torch.randn(L, nkv, hd, generator=g).to(DT[dtype])
+        kb[7] *= 5.0       # an early key that late queries must find (or must not, behind a window)
+        keys.append(kb); values.append(vb)
+        for i in range((L + page - 1) // page):
+            pg = perm.pop()
+            table[b, i] = pg
+            n = min(page, L - i * page)
+            kc[pg, :, :n] = kb[i * page: i * page + n].transpose(0, 1).float()
+            vc[pg, :, :, :n] = vb[i * page: i * page + n].permute(1, 2, 0).float()
+        positions += list(range(L)); token_seq += [b] * L
+    T = len(positions)
+    assert T * nh // 4 >= 2048
+    stride = (nh + 2 * nkv) * hd
+    qkv = torch.randn(T, stride, generator=g).to(DT[dtype])
+    out = torch.full((T, nh * hd), 7.0, dtype=DT[dtype], device="cuda")
+    scale = 1.0 / math.sqrt(hd)
+    ops.attn_paged(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
+                   dev(torch.tensor(token_seq, dtype=torch.int32)), dev(table), dev(kc.to(DT[dtype])),
+                   dev(vc.to(DT[dtype])), page, nh, nkv, hd, scale, window, 1)
+    got = out.cpu().double().reshape(T, nh, hd)
+    assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
+    rng = torch.Generator().manual_seed(1)
+    picks = sorted(set(torch.randint(0, T, (60,), generator=rng).tolist()) | {0, 63, 64, 65, lens[0] - 1, lens[0], T - 1})
+    for t in picks:
+        b = token_seq[t]
+        want = _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[b], values[b], positions[t], scale, window, nh // nkv)
+        close(got[t], want, EPS[dtype] * 2)
 
 
 def _paged_case(g, lens, nkv, hd, page=64, n_pages=40, far_key=None):
