@@ -833,6 +833,39 @@ def test_generation_that_runs_ahead_of_the_host_in_bfloat16(folders, name):
         assert rel_err(got, P.transformer_forward([p], plain)[0, -1]) <= TOL["bfloat16"]
 
 
+def test_run_ahead_with_an_embedding_that_cannot_take_tokens_from_the_device(folders):
+    """An embedding part without forward_from (here: the framework's own with the method hidden) gets the
+    picked tokens gathered into the step's token ids by a launch in front of the replay; generation
+    gives the same tokens as the loop that reads every token first."""
+    from burn_lm_amd.engine.generate import generate
+    from burn_lm_amd.parts.embedding import Embedding
+    from burn_lm_amd.sampling.sampler import Sampler
+    cfg, seed = TINIES["B"]
+
+    class PlainEmbedding(Embedding):
+        def __getattribute__(self, name):
+            if name == "forward_from":
+                raise AttributeError(name)
+            return super().__getattribute__(name)
+
+    eng = load(folders["B"], "bfloat16", max_tokens=2048, max_seqs=4)
+    eng.model.embedding.__class__ = PlainEmbedding
+    assert not hasattr(eng.model.embedding, "forward_from")
+    prompts = [random_tokens(40 + i, cfg["vocab_size"], n) for i, n in enumerate([9, 33, 2])]
+
+    class Waiting:
+        def __init__(self, e):
+            self.open, self.close, self.step, self.length = e.open, e.close, e.step, e.length
+            self.max_context, self.cache = e.max_context, e.cache
+
+    for _ in range(2):
+        ahead, _ = generate(eng, prompts, Sampler(0.0), 20, stop_ids=[], batch_size=4)
+        waited, _ = generate(Waiting(eng), prompts, Sampler(0.0), 20, stop_ids=[], batch_size=4)
+        assert [r.tokens for r in ahead] == [r.tokens for r in waited]
+    assert eng.graphs.replays > 20
+    assert all(not c.folded for c in eng.graphs.captured.values())
+
+
 def test_recorded_shapes_are_limited_and_the_oldest_goes(folders, monkeypatch):
     """A shape is recorded at its second sight; with room for two recorded shapes a third one evicts
     the shape replayed longest ago, and every step still gives the plain logits."""
