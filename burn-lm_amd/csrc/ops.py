@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 _lib = None
 _lock = threading.Lock()
 
@@ -49,6 +49,9 @@ _SIGNATURES = {
                       _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_gemm_mfma_init": [],
+    "blm_gemm_rows_init": [],
+    "blm_gemm_rows": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                      _c_int, _c_void_p],
     "blm_attn_paged_init": [],
     "blm_gemm_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_void_p],
@@ -602,6 +605,46 @@ def gemm_mfma(a, w, out, gated=False, tile=(128, 128)):
         raise KernelError(f"gemm_mfma: tile {tile} is not one of {sorted(GEMM_TILES)}")
     _call("blm_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0), w.stride(0),
           out.stride(-2), 1 if gated else 0, groups, GEMM_TILES[tile], _stream())
+    return out
+
+
+_rows_ready = set()
+
+
+def gemm_rows_init(device=None):
+    """Once per device, outside any stream capture, before the first gemm_rows (its rings of stages
+    take more shared memory than a kernel gets without asking)."""
+    index = torch.device(device or "cuda").index
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _rows_ready:
+        with torch.cuda.device(index):
+            _call("blm_gemm_rows_init")
+        _rows_ready.add(index)
+
+
+def gemm_rows(a, w, out, gated=False, columns=64):
+    """bfloat16 product for up to 64 rows whose loads never stop for a barrier: out = a[M, K] @ w[N, K]^T,
+    w as the checkpoint stores it.  out: bfloat16 or float32 [M, N], or float32 [groups, M, N] partial
+    products over that many groups of K (the reader sums them).  gated=True: w is [gate rows; up rows]
+    ([2I, K]) and out is [M, I] = silu(a gate^T) * (a up^T).  columns: 64 or (without gating) 32 columns
+    of out (of gate and up together when gated) per block."""
+    _gpu(a, w, out)
+    gemm_rows_init(a.device)
+    groups = 1
+    if out.dim() == 3:
+        groups = out.shape[0]
+        if out.dtype != torch.float32 or not out.is_contiguous():
+            raise KernelError("gemm_rows: partial outputs must be contiguous float32 [groups, M, N]")
+    M, N = out.shape[-2], out.shape[-1]
+    K = a.shape[1]
+    if a.shape[0] != M or w.dim() != 2 or w.shape != (N * (2 if gated else 1), K):
+        raise KernelError(f"gemm_rows: shapes a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)} do not fit")
+    if a.stride(1) != 1 or w.stride(1) != 1 or out.stride(-1) != 1:
+        raise KernelError("gemm_rows: a, w and out need unit stride along their rows")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("gemm_rows: operands must be bfloat16")
+    _call("blm_gemm_rows", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0), w.stride(0),
+          out.stride(-2), 1 if gated else 0, groups, int(columns), _stream())
     return out
 
 

@@ -5,7 +5,11 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
   reduced-precision matrix mode), whatever the activation dtype.  This is the whole float32 path
   and also what keeps a tensor that a checkpoint stores in 32 bits exact in a bfloat16 run.
 * bfloat16 weights, up to 64 rows (decode): the hand-written skinny kernel on the matrix cores that
-  streams the weight once (where the width fits its registers: see ops.gemv_mfma_group_limit).
+  streams the weight once (where the width fits its registers: see ops.gemv_mfma_group_limit).  From
+  17 rows on, the products that come as partial planes (output and down projection) and, from 33 rows
+  on, the gated product run on the kernel whose wavefronts each stream their own stages of K through
+  shared memory (ops.gemm_rows): with that many rows the activations cost as much traffic as the
+  weights, and its loads never stop for a barrier (see rows_plan and gated_linear).
 * bfloat16 weights, 65 rows and more, narrow output and long K (the down projection of short
   prompts): partial planes from the hand-written matrix-core kernel (see mid_k_groups).
 * bfloat16 weights, many rows (prefill): the library product (hipBLASLt through torch), as the
@@ -60,6 +64,7 @@ class Runtime:
         ops.static_scratch_init(self.device)   # likewise: the address of the library's own scratch array
         ops.grid_sync(self.device)             # likewise: the counters and the fault word of resident-grid kernels
         ops.attn_paged_init(self.device)       # likewise: the shared memory of the generic attention's value tiles
+        ops.gemm_rows_init(self.device)        # likewise: the rings of stages of the product for 17 to 64 rows
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         asked = os.environ.get("BURN_LM_AMD_FUSED_GATE_UP")   # "1": wherever it can run, "0": nowhere, unset: where it is ahead
         self.fused_gate_up_rows = FUSED_GATE_UP_ROWS if asked == "1" else (0, -1)
@@ -74,6 +79,8 @@ class Runtime:
         # three kernels.  Off unless asked for: measured 36-53 us against 24-29 us for the three kernels (a
         # hand-over between blocks through device-wide counters costs more than a kernel boundary here).
         self.resident_decode = os.environ.get("BURN_LM_AMD_RESIDENT_DECODE") == "1"
+        # "0": 17 to 64 rows stay on the packed skinny kernels (for measurements)
+        self.rows_ring = os.environ.get("BURN_LM_AMD_ROWS_RING") != "0"
 
     def check_fault(self):
         ops.check_fault(self.device)
@@ -108,6 +115,20 @@ class Runtime:
         while g < 64 and (steps + g - 1) // g * 32 > limit:
             g *= 2
         return g
+
+    def rows_plan(self, N, K):
+        """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial
+        planes (ops.gemm_rows).  A group spans about 2048 of K (measured at the 1B, 3B and 8B layer
+        shapes: shorter groups write more planes than they gain, longer ones leave compute units
+        idle); 32 columns per block where that gives at most one block per compute unit, else 64;
+        and a short K is cut further, down to 512, until three quarters of the units have a block."""
+        groups = 1
+        while groups < 8 and K // (groups * 2) >= 2048:
+            groups *= 2
+        columns = 32 if -(-N // 32) * groups <= self.compute_units else 64
+        while groups < 8 and K // (groups * 2) >= 512 and -(-N // columns) * groups * 4 < self.compute_units * 3:
+            groups *= 2
+        return groups, columns
 
     def mid_k_groups(self, M, N, K):
         """Short prompts, narrow output, long K (the down projection): the product as partial planes
@@ -148,6 +169,14 @@ class Runtime:
             if groups:
                 return ops.gemm_mfma(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device),
                                      tile=(128, 64, 6))
+        if (partials and out is None and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and aligned
+                and (M > 32 or K <= 4096) and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()):
+            # 17 to 64 rows as partial planes (measured against the packed skinny kernel at the 1B, 3B and 8B
+            # shapes: output projection 15-35 % faster at every row count, down projection 25-40 % at K = 8192 of
+            # the 1B width, equal to 10 % at the wider ones from 33 rows on and up to 10 % behind below: left there)
+            groups, columns = self.rows_plan(N, K)
+            if groups > 1:
+                return ops.gemm_rows(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), columns=columns)
         if packed is not None and M <= MFMA_SKINNY_MAX_ROWS and aligned:
             if partials and out is None:
                 groups = self.k_groups(N, K, M)
@@ -181,14 +210,20 @@ class Runtime:
         it); otherwise the product is followed by the gating kernel."""
         M, K = x.shape
         inner = w.shape[0] // 2
+        plain = w.w if isinstance(w, LinearWeight) else w
+        fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
+                   and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
+        if fusable and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and (
+                M > 32 or (K > 2048 and -(-inner // 32) <= self.compute_units)):
+            # 33 to 64 rows (measured against the packed skinny kernel: 4-15 % faster at the 1B and 3B shapes, and
+            # at wider ones in place of the library's product, which the packed kernel's registers leave them to);
+            # from 17 rows on where K is above 2048 and the blocks come in one round (3B: 10-15 %)
+            return ops.gemm_rows(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True)
         if (isinstance(w, LinearWeight) and w.packed is not None and w.gated and x.dtype == torch.bfloat16
                 and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
             return ops.gemv_mfma(x, w.packed, out, K, gated=True)
-        plain = w.w if isinstance(w, LinearWeight) else w
-        fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
-                   and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
         if fusable and self.fused_gate_up_measured:
             # Short prompts: when all tiles of the product run at once (one block per compute unit,
             # most of the units busy), the fused kernel with a deep ring of stages streams the

@@ -561,6 +561,75 @@ def test_gemv_mfma_gated(ops, M, I, K):
     assert float((torch.nn.functional.silu(up) * gate - want).abs().max() / want.abs().max()) > 0.1
 
 
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("M,N,K,columns", [(64, 128, 64, 64), (33, 200, 136, 32), (17, 72, 1000, 64), (32, 100, 264, 64), (20, 264, 520, 32),
+                                           (50, 96, 4104, 64), (1, 40, 72, 32), (48, 3072, 2048, 32), (64, 1000, 3080, 64)])
+def test_gemm_rows(ops, out_dtype, M, N, K, columns):
+    """The product for 17 to 64 rows whose wavefronts each stream their own stages of K: both stagings of
+    the rows (32 and 64), both widths of a block, tails in N, K and M, more and fewer stages than the
+    rings hold."""
+    g = torch.Generator().manual_seed(26)
+    A = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(N, K, generator=g) * 0.1).bfloat16()
+    W[N // 2, K - 8:] = 5.0   # one term that a wrong piece order or a lost tail cannot hide
+    out = torch.full((M, N), 7.0, dtype=DT[out_dtype], device="cuda")
+    ops.gemm_rows(dev(A), dev(W), out, columns=columns)
+    want = A.double() @ W.double().T
+    err = ((out.double().cpu() - want).abs() / (want.abs() + want.abs().mean())).max()
+    assert float(err) <= (2e-5 if out_dtype == "float32" else 8e-3), f"error {float(err):.3g}"
+    # rows of wider buffers, and an output with a row stride
+    wide = torch.randn(M, K + 24, generator=g).bfloat16()
+    wwide = (torch.randn(N, K + 16, generator=g) * 0.1).bfloat16()
+    big = torch.zeros(M, N + 5, dtype=DT[out_dtype], device="cuda")
+    ops.gemm_rows(dev(wide)[:, 8:K + 8], dev(wwide)[:, :K], big[:, :N], columns=columns)
+    close(big[:, :N], wide[:, 8:K + 8].double() @ wwide[:, :K].double().T, EPS[out_dtype] * 3)
+    assert bool((big[:, N:] == 0).all())
+
+
+@pytest.mark.parametrize("M,N,K,groups,columns", [(64, 2048, 8192, 4, 32), (24, 100, 8200, 8, 64), (40, 48, 3000, 2, 32), (33, 64, 14336, 4, 64),
+                                                  (17, 200, 1096, 3, 32)])
+def test_gemm_rows_partial_products_sum_to_the_product(ops, M, N, K, groups, columns):
+    g = torch.Generator().manual_seed(27)
+    A = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    planes = torch.full((groups, M, N), 7.0, dtype=torch.float32, device="cuda")
+    ops.gemm_rows(dev(A), dev(W), planes, columns=columns)
+    close(planes.double().sum(0), A.double() @ W.double().T, 1e-5)
+    per = ((K + groups - 1) // groups + 63) // 64 * 64          # a group's span: K / groups rounded up to whole stages of 64
+    close(planes[0], A[:, :per].double() @ W[:, :per].double().T, 1e-5)
+    close(planes[groups - 1], A[:, (groups - 1) * per:].double() @ W[:, (groups - 1) * per:].double().T, 1e-5)
+
+
+@pytest.mark.parametrize("M,I,K", [(64, 1000, 2048), (20, 176, 1544), (37, 384, 144), (50, 8, 520), (32, 176, 4096), (33, 100, 3080)])
+def test_gemm_rows_gated(ops, M, I, K):
+    """The SwiGLU gating where the partial tiles of a block meet: w is [gate rows; up rows] as the checkpoint
+    has them, a block takes 32 gate columns and the matching up columns."""
+    g = torch.Generator().manual_seed(28)
+    A = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(2 * I, K, generator=g) * (2.0 / K ** 0.5)).bfloat16()
+    out = torch.full((M, I), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_rows(dev(A), dev(W), out, gated=True)
+    gate, up = A.double() @ W[:I].double().T, A.double() @ W[I:].double().T
+    want = torch.nn.functional.silu(gate) * up
+    close(out, want, EPS["bfloat16"] * 1.5)
+    assert float((torch.nn.functional.silu(up) * gate - want).abs().max() / want.abs().max()) > 0.1
+
+
+def test_gemm_rows_refuses_what_it_cannot_do(ops):
+    from burn_lm_amd.csrc.ops import KernelError
+    a, w = dev(torch.zeros(65, 64).bfloat16()), dev(torch.zeros(8, 64).bfloat16())
+    with pytest.raises(KernelError, match="M <= 64"):
+        ops.gemm_rows(a, w, torch.zeros(65, 8, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(KernelError, match="32 without gating"):
+        ops.gemm_rows(a[:8], w, torch.zeros(8, 4, dtype=torch.bfloat16, device="cuda"), gated=True, columns=32)
+    with pytest.raises(KernelError, match="32 without gating"):
+        ops.gemm_rows(a[:8], w, torch.zeros(8, 8, dtype=torch.bfloat16, device="cuda"), columns=48)
+    with pytest.raises(KernelError, match="float32"):
+        ops.gemm_rows(a[:8], w, torch.zeros(2, 8, 8, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(KernelError, match="do not fit"):
+        ops.gemm_rows(a[:8], w, torch.zeros(8, 9, dtype=torch.bfloat16, device="cuda"))
+
+
 def test_gemv_mfma_refuses_what_it_cannot_do(ops):
     from burn_lm_amd.csrc.ops import KernelError
     assert not ops.gemv_mfma_supported(65, 64, 64) and not ops.gemv_mfma_supported(4, 64, 60)
