@@ -136,7 +136,10 @@ def machine_rates(device):
     del buf
     flops = ops.probe_mfma(iters=2048, blocks=2048, device=device)
     mfma = flops / event_time(lambda: ops.probe_mfma(iters=2048, blocks=2048, device=device)) / 1e12
-    return {"read_gbs": round(read, 1), "mfma_bf16_tflops": round(mfma, 1)}
+    # the same on random operands that change with every instruction, as a product of real data has them:
+    # the clock follows the power the multipliers draw
+    rand = flops / event_time(lambda: ops.probe_mfma(iters=2048, blocks=2048, device=device, random_operands=True)) / 1e12
+    return {"read_gbs": round(read, 1), "mfma_bf16_tflops": round(mfma, 1), "mfma_bf16_random_tflops": round(rand, 1)}
 
 
 def kernel_rates(engine, batch, context, prefill_tokens):

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 _lib = None
 _lock = threading.Lock()
 
@@ -66,7 +66,7 @@ _SIGNATURES = {
                        _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                        _c_int, _c_void_p],
     "blm_probe_read": [_c_void_p, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p],
-    "blm_probe_mfma": [_c_int, _c_int, _c_void_p, _c_void_p],
+    "blm_probe_mfma": [_c_int, _c_int, _c_int, _c_void_p, _c_void_p],
     "blm_static_scratch_init": [],
     "blm_argmax_static": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "blm_sample": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p, _c_void_p,
@@ -733,10 +733,11 @@ def probe_read(buffer, blocks=2048):
     return n
 
 
-def probe_mfma(iters=4096, blocks=2048, device="cuda"):
-    """Launches the matrix-instruction measuring kernel; returns the floating-point operations it does."""
+def probe_mfma(iters=4096, blocks=2048, device="cuda", random_operands=False):
+    """Launches the matrix-instruction measuring kernel (on the same small operands every time, or on
+    random ones that change with every instruction); returns the floating-point operations it does."""
     sink = _probe_sink(torch.device(device))
-    _call("blm_probe_mfma", int(iters), int(blocks), sink.data_ptr(), _stream())
+    _call("blm_probe_mfma", int(iters), int(blocks), 1 if random_operands else 0, sink.data_ptr(), _stream())
     return blocks * 4 * iters * 4 * 2 * 32 * 32 * 16
 
 

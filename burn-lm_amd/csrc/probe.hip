@@ -5,7 +5,10 @@
 //                flight per lane, and keeps an exclusive-or of what it read (stored only if it equals a
 //                value it cannot have, so the loads are not optimised away and nothing is written).
 //   probe_mfma : every wavefront issues `iters` rounds of four independent 32x32x16 bf16 matrix
-//                instructions on registers (4 * 32768 multiply-adds per round per wavefront).
+//                instructions on registers (4 * 32768 multiply-adds per round per wavefront), either on
+//                the same few small values every time, or on random operands that change with every
+//                instruction: the rate differs, since the clock follows the power the multipliers
+//                draw (measured: 2.2 against 1.8 PFLOP/s), and a product of real data is the second case.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 pb_bf16x8;
@@ -30,19 +33,37 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const uint4* __restrict
   if (acc == 0x12345678u) sink[0] = acc;
 }
 
+__device__ __forceinline__ unsigned probe_hash(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+
+template <bool RANDOM>
 __global__ void __launch_bounds__(256) probe_mfma_kernel(int iters, float* __restrict__ sink) {
-  pb_bf16x8 a, b;
+  pb_bf16x8 a[4], b[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    a[i] = (__bf16)(0.001f * (float)((threadIdx.x + i) & 7));
-    b[i] = (__bf16)(0.002f * (float)((threadIdx.x * 3 + i) & 7));
-  }
+  for (int f = 0; f < 4; ++f)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (RANDOM) {
+        // uniform in [-2, 2) and in [-0.04, 0.04): activations and weights of a layer, roughly
+        const unsigned h = probe_hash(threadIdx.x * 64 + f * 8 + i + blockIdx.x * 7919u), g = probe_hash(h + 1);
+        a[f][i] = (__bf16)(((int)(h & 0xffff) - 32768) / 16384.0f);
+        b[f][i] = (__bf16)(((int)(g & 0xffff) - 32768) / 16384.0f * 0.02f);
+      } else {
+        a[f][i] = (__bf16)(0.001f * (float)((threadIdx.x + i) & 7));
+        b[f][i] = (__bf16)(0.002f * (float)((threadIdx.x * 3 + i) & 7));
+      }
+    }
   pb_f32x16 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
-  for (int it = 0; it < iters; ++it) {
-    c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
-    c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
-    c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
-    c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+  for (int it = 0; it < iters; it += 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u], b[u], c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(u + 1) & 3], b[u], c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(u + 2) & 3], b[(u + 1) & 3], c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(u + 3) & 3], b[(u + 2) & 3], c3, 0, 0, 0);
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -60,10 +81,13 @@ extern "C" int blm_probe_read(const void* x, long long bytes, void* sink, int bl
   return 0;
 }
 
-// blocks x 4 wavefronts, `iters` rounds each: flops = blocks * 4 * iters * 4 * 2 * 32 * 32 * 16.
-extern "C" int blm_probe_mfma(int iters, int blocks, void* sink, hipStream_t stream) {
-  BLM_REQUIRE(sink != nullptr && iters >= 1 && blocks >= 1 && blocks <= 65535, "probe_mfma: bad arguments (iters=%d blocks=%d)", iters, blocks);
-  hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(256), 0, stream, iters, (float*)sink);
+// blocks x 4 wavefronts, `iters` rounds (a multiple of 4) each: flops = blocks * 4 * iters * 4 * 2 * 32 * 32 * 16.
+// random_operands: operands that differ from instruction to instruction instead of the same small values.
+extern "C" int blm_probe_mfma(int iters, int blocks, int random_operands, void* sink, hipStream_t stream) {
+  BLM_REQUIRE(sink != nullptr && iters >= 4 && iters % 4 == 0 && blocks >= 1 && blocks <= 65535,
+              "probe_mfma: bad arguments (iters=%d, a multiple of 4; blocks=%d)", iters, blocks);
+  if (random_operands) hipLaunchKernelGGL(probe_mfma_kernel<true>, dim3(blocks), dim3(256), 0, stream, iters, (float*)sink);
+  else hipLaunchKernelGGL(probe_mfma_kernel<false>, dim3(blocks), dim3(256), 0, stream, iters, (float*)sink);
   BLM_LAUNCH_CHECK("probe_mfma");
   return 0;
 }
