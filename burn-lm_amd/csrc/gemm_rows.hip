@@ -18,6 +18,9 @@
 // gate columns and the matching up columns, and C[M, N] = silu(gate) * up.
 // k_groups > 1: K is cut into groups, C is float [k_groups, M, ldc] with one partial product each
 // (summed by the reader), so that a narrow output still fills the chip.
+// mode 2: W is the q/k/v projection; where the partial tiles meet, queries and keys are rotated by
+// their positions (partners in adjacent columns), queries go to C, keys and values to their pages
+// of the cache, as gemv_qkv_rope.hip does for up to 16 rows.
 #include <type_traits>
 
 #include "common.h"
@@ -47,10 +50,22 @@ __device__ __forceinline__ void gr_dma16_lanes(const char* address, const void* 
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(address) : "memory");
 }
 
+// what mode 2 needs beside the product: positions and sequences of the rows, the pages, the table of
+// cosines and sines, the cache planes (keys [pages, nkv, page, hd], values [pages, nkv, hd, page])
+struct GrRope {
+  const int* positions;
+  const int* token_seq;
+  const int* block_table;
+  const float2* cos_sin;
+  bf16* kcache;
+  bf16* vcache;
+  int table_width, page_size, nh, nkv, hd, store;
+};
+
 template <int BM, int BN, int BK, int R, int MODE, typename TC>
 __global__ void __launch_bounds__(256)
     gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, TC* __restrict__ C, int M, int N, int K, int lda,
-                     int ldw, int ldc, int k_per_group) {
+                     int ldw, int ldc, int k_per_group, GrRope rope) {
   constexpr int NW = 4;
   static_assert(BM == 32 || BM == 64, "rows");
   constexpr int TM = BM / 32, TN = BN / 32;
@@ -69,6 +84,7 @@ __global__ void __launch_bounds__(256)
   const int wave = __builtin_amdgcn_readfirstlane(tid / BLM_WAVE);   // known to be the same in all lanes
   const int l32 = lane & 31, lh = lane >> 5;
   const int n0 = blockIdx.x * (MODE == 1 ? BN / 2 : BN);   // first output column
+  if (MODE == 2 && !rope.store && n0 >= rope.nh * rope.hd) return;   // keys and values belong to another layer's cache
   const int k_begin = blockIdx.y * k_per_group, k_end = min(K, k_begin + k_per_group);
   C += (size_t)blockIdx.y * M * ldc;
   bf16* ring = reinterpret_cast<bf16*>(gr_smem) + (size_t)wave * R * SLOT;
@@ -215,6 +231,38 @@ __global__ void __launch_bounds__(256)
       }
     }
     const int n = n0 + c0;
+    if constexpr (MODE == 2) {
+      const int pos = rope.positions[row], b = rope.token_seq[row];
+      int page = -1;
+      if (b >= 0 && rope.store) page = rope.block_table[(size_t)b * rope.table_width + pos / rope.page_size];
+      const int slot = pos % rope.page_size, hd = rope.hd;
+#pragma unroll
+      for (int c = 0; c < CPT; c += 2) {
+        const int nn = n + c;   // even; its partner nn + 1 is in the same head (head sizes are even)
+        if (nn >= N) break;
+        const int head = nn / hd, d = nn - head * hd;
+        float y0 = v[c], y1 = v[c + 1];   // value heads are stored as they are
+        if (head < rope.nh + rope.nkv) {
+          const float2 cs = rope.cos_sin[(size_t)pos * (hd / 2) + (d >> 1)];
+          y0 = v[c] * cs.x - v[c + 1] * cs.y;
+          y1 = v[c] * cs.y + v[c + 1] * cs.x;
+        }
+        if (head < rope.nh) {
+          *reinterpret_cast<uint32_t*>(C + (size_t)row * ldc + nn) = f32x2_to_bf16x2_bits(y0, y1);
+        } else if (page >= 0) {
+          if (head < rope.nh + rope.nkv) {
+            *reinterpret_cast<uint32_t*>(rope.kcache + (((size_t)page * rope.nkv + (head - rope.nh)) * rope.page_size + slot) * hd + d) =
+                f32x2_to_bf16x2_bits(y0, y1);
+          } else {
+            bf16* vp = rope.vcache + ((size_t)page * rope.nkv + (head - rope.nh - rope.nkv)) * hd * rope.page_size +
+                       (size_t)d * rope.page_size + slot;
+            vp[0] = from_float<bf16>(y0);
+            vp[rope.page_size] = from_float<bf16>(y1);
+          }
+        }
+      }
+      return;
+    }
     TC* dst = C + (size_t)row * ldc + n;
     constexpr int PER = sizeof(TC) == 2 ? 8 : 4;   // elements per 16-byte store
     if constexpr (CPT >= PER) {
@@ -251,14 +299,14 @@ static int gr_prepare() {
 
 template <int BM, int BN, int BK, int R, int MODE, typename TC>
 static int gr_launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc, int k_groups,
-                     hipStream_t stream) {
+                     hipStream_t stream, GrRope rope = GrRope{}) {
   constexpr size_t smem = (size_t)4 * R * (BM + BN) * BK * sizeof(bf16);
   static_assert(smem >= (size_t)4 * BM * (BN + 4) * sizeof(float), "the partial tiles fit where the ring was");
   const int n_tiles = (N + (MODE == 1 ? BN / 2 : BN) - 1) / (MODE == 1 ? BN / 2 : BN);
   const int k_per_group = ((K + k_groups - 1) / k_groups + BK - 1) / BK * BK;
   dim3 grid((unsigned)n_tiles, (unsigned)k_groups), block(256);
   hipLaunchKernelGGL((gemm_rows_kernel<BM, BN, BK, R, MODE, TC>), grid, block, smem, stream, (const bf16*)A, (const bf16*)W, (TC*)C, M,
-                     N, K, lda, ldw, ldc, k_per_group);
+                     N, K, lda, ldw, ldc, k_per_group, rope);
   BLM_LAUNCH_CHECK("gemm_rows");
   return 0;
 }
@@ -271,6 +319,7 @@ extern "C" int blm_gemm_rows_init() {
   GR_PREP(64, 64, 2, 0) GR_PREP(64, 32, 3, 0) GR_PREP(32, 64, 3, 0) GR_PREP(32, 32, 5, 0)
   GR_PREP(64, 64, 2, 1) GR_PREP(32, 64, 3, 1)
 #undef GR_PREP
+  if (gr_prepare<64, 32, 64, 3, 2, bf16>() || gr_prepare<32, 32, 64, 5, 2, bf16>()) return 1;
   return 0;
 }
 
@@ -306,4 +355,29 @@ extern "C" int blm_gemm_rows(const void* A, const void* W, void* C, int c_dtype,
   if (M > 32) GR_GO(64, 32, 3, 0);
   GR_GO(32, 32, 5, 0);
 #undef GR_GO
+}
+
+// The q/k/v projection of 17 to 64 rows with the rotation and the cache write where the partial tiles meet
+// (32 columns per block).  W: W_qkv [(nh + 2 nkv) * hd, K] with rotary partners in adjacent rows; qkv_out:
+// [M, ldq] bf16, of which only the first nh * hd columns (the rotated queries) are written; key plane
+// [pages, nkv, page, hd], value plane [pages, nkv, hd, page].  store = 0: keys and values are neither
+// computed nor written.
+extern "C" int blm_gemm_rows_qkv_rope(const void* A, const void* W, void* qkv_out, const int* positions, const int* token_seq,
+                                      const int* block_table, int table_width, const float* cos_sin, void* kcache, void* vcache,
+                                      int page_size, int M, int K, int lda, int ldw, int ldq, int nh, int nkv, int hd, int store,
+                                      hipStream_t stream) {
+  BLM_REQUIRE(M >= 1 && M <= 64 && K >= 8 && K % 8 == 0 && hd >= 2 && hd % 2 == 0,
+              "gemm_rows_qkv_rope: M=%d K=%d head_dim=%d not supported (M <= 64, K a multiple of 8, an even head size)", M, K, hd);
+  BLM_REQUIRE(nh > 0 && nkv > 0 && page_size > 0 && table_width > 0, "gemm_rows_qkv_rope: bad geometry");
+  BLM_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldq >= nh * hd && ldq % 2 == 0,
+              "gemm_rows_qkv_rope: bad strides lda=%d ldw=%d ldq=%d", lda, ldw, ldq);
+  BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)qkv_out % 4) == 0 && ((uintptr_t)kcache % 4) == 0,
+              "gemm_rows_qkv_rope: operands must be 16-byte aligned (outputs 4-byte)");
+  const int N = (nh + 2 * nkv) * hd;
+  BLM_REQUIRE((size_t)64 * lda * 2 < ((size_t)1 << 32) && (size_t)N * ldw * 2 < ((size_t)1 << 32),
+              "gemm_rows_qkv_rope: matrices of 4 GiB and more are not supported");
+  const GrRope rope{positions, token_seq, block_table, (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache,
+                    table_width, page_size, nh, nkv, hd, store};
+  if (M > 32) return gr_launch<64, 32, 64, 3, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
+  return gr_launch<32, 32, 64, 5, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
 }

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 _lib = None
 _lock = threading.Lock()
 
@@ -60,6 +60,9 @@ _SIGNATURES = {
     "blm_gemv_qkv_rope": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
+    "blm_gemm_rows_qkv_rope": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                               _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                               _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_decode_ffn_supported": [_c_int, _c_int, _c_int, _c_int],
     "blm_decode_ffn": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_float, _c_void_p,
@@ -679,6 +682,35 @@ def gemv_qkv_rope(x, packed, qkv_out, positions, token_seq, block_table, cos_sin
     _call("blm_gemv_qkv_rope", x.data_ptr(), packed.data_ptr(), qkv_out.data_ptr(), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], cos_sin.data_ptr(), kcache.data_ptr(),
           vcache.data_ptr(), page_size, M, K, x.stride(0), qkv_out.stride(0), nh, nkv, hd, pairing,
+          1 if write_kv else 0, _stream())
+    return qkv_out
+
+
+def gemm_rows_qkv_rope(x, w, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,
+                       nh, nkv, hd, write_kv=True):
+    """17 to 64 rows: x [M, K] @ W_qkv^T (w [(nh + 2 nkv) * hd, K] as bound, rotary partners in adjacent
+    rows), rotary encoding of q and k on the float results, q into qkv_out[:, :nh*hd], k and v into
+    their cache pages, in one kernel (the product of gemm_rows)."""
+    _gpu(x, w, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache)
+    gemm_rows_init(x.device)
+    M, K = x.shape
+    N = (nh + 2 * nkv) * hd
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or qkv_out.dtype != torch.bfloat16:
+        raise KernelError("gemm_rows_qkv_rope: operands must be bfloat16")
+    if w.dim() != 2 or w.shape != (N, K) or w.stride(1) != 1:
+        raise KernelError(f"gemm_rows_qkv_rope: the weights must be [{N}, {K}] with unit stride along rows, got {tuple(w.shape)}")
+    if qkv_out.shape[0] != M or qkv_out.stride(1) != 1 or qkv_out.shape[1] < nh * hd or x.stride(1) != 1:
+        raise KernelError("gemm_rows_qkv_rope: qkv_out must be [M, >= heads*head_dim] with unit stride along rows")
+    _i32("positions", positions, M); _i32("token_seq", token_seq, M); _i32("block_table", block_table)
+    if cos_sin.dtype != torch.float32 or cos_sin.shape[1:] != (hd // 2, 2) or not cos_sin.is_contiguous():
+        raise KernelError("gemm_rows_qkv_rope: cos_sin must be contiguous float32 [positions, head_dim/2, 2]")
+    if kcache.dtype != torch.bfloat16:
+        raise KernelError("gemm_rows_qkv_rope: the cache must be bfloat16")
+    _contig("kcache", kcache); _contig("vcache", vcache)
+    _check_planes("gemm_rows_qkv_rope", kcache, vcache, nkv, page_size, hd)
+    _call("blm_gemm_rows_qkv_rope", x.data_ptr(), w.data_ptr(), qkv_out.data_ptr(), positions.data_ptr(),
+          token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], cos_sin.data_ptr(), kcache.data_ptr(),
+          vcache.data_ptr(), page_size, M, K, x.stride(0), w.stride(0), qkv_out.stride(0), nh, nkv, hd,
           1 if write_kv else 0, _stream())
     return qkv_out
 

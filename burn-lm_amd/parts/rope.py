@@ -95,6 +95,21 @@ class RotaryEncoding(PositionEncoding):
         rt = self.rt
         packed = getattr(w_qkv, "packed", None)
         M, K = x.shape
+        raw = getattr(w_qkv, "w", None)
+        if (16 < M <= 64 and (M > 32 or K > 2048) and self.pairing == PAIRING["interleaved"] and getattr(rt, "rows_ring", False)
+                and raw is not None
+                and x.dtype == raw.dtype == view.k.dtype == torch.bfloat16 and head_dim % 2 == 0 and K % 8 == 0
+                and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and raw.is_contiguous()):
+            # 33 to 64 rows, and 17 to 32 where K is above 2048: the product whose wavefronts stream their own stages
+            # of K, rotation and cache write where its partial tiles meet (measured over whole decode steps against
+            # the packed kernel with two to four row tiles, and against the library's product and the rotation kernel
+            # where that kernel's registers do not take the width: 1.4 % faster at batch 64 of the 1B shape and 1.3 %
+            # slower at batch 17-32, hence the rule; 2-6 % faster at every batch from 17 to 64 of the 3B and 8B shapes)
+            if step.max_position >= self.n_positions:
+                raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
+            qkv = torch.empty(M, (heads + 2 * kv_heads) * head_dim, dtype=torch.bfloat16, device=x.device)
+            return rt.ops.gemm_rows_qkv_rope(x, raw, qkv, step.positions, step.token_seq, view.block_table(step), self.table,
+                                             view.k, view.v, view.page_size, heads, kv_heads, head_dim, write_kv=view.store)
         if (packed is not None and not getattr(w_qkv, "gated", False) and x.dtype == torch.bfloat16
                 and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing) and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0 and view.k.dtype == torch.bfloat16):

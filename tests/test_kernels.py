@@ -808,7 +808,7 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     """The fused decode projection: equals the product, the rotation of its float result and the
     cache write done one after the other (in float64), for both pairings, with a padding row and
     scrambled pages; nothing else in the cache is touched."""
-    from burn_lm_amd.parts.rope import PAIRING, rope_frequencies
+    from burn_lm_amd.parts.rope import PAIRING
     # adjacent pairs sit in one 16-column tile: any head size in steps of 16; pairs half a head apart
     # need two whole tiles per half: steps of 32
     # and from 17 rows on only adjacent pairs, with K up to 4096 for 32 rows and up to 2048 beyond
@@ -816,6 +816,28 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     assert ops.gemv_qkv_rope_supported(M, K, hd, PAIRING[pairing]) == takes
     if not takes:
         return
+
+    def run(x, W, out, positions, token_seq, perm, cs, kd, vd, page, write_kv):
+        ops.gemv_qkv_rope(x, ops.pack_weight(W), out, positions, token_seq, perm, cs, kd, vd, page, nh, nkv, hd, PAIRING[pairing],
+                          write_kv=write_kv)
+
+    _check_qkv_rope(run, pairing, M, K, nh, nkv, hd)
+
+
+@pytest.mark.parametrize("M,K,nh,nkv,hd", [(33, 2048, 4, 2, 64), (64, 520, 3, 1, 48), (20, 4096, 2, 1, 64), (17, 264, 30, 2, 128),
+                                           (48, 2056, 2, 1, 32), (64, 3072, 3, 1, 128), (40, 4104, 2, 2, 80), (32, 72, 1, 1, 6)])
+def test_gemm_rows_qkv_rope(ops, M, K, nh, nkv, hd):
+    """The same for 17 to 64 rows on the product whose wavefronts stream their own stages of K: any K,
+    head sizes that put two heads into a block's 32 columns or a head across several blocks."""
+
+    def run(x, W, out, positions, token_seq, perm, cs, kd, vd, page, write_kv):
+        ops.gemm_rows_qkv_rope(x, W, out, positions, token_seq, perm, cs, kd, vd, page, nh, nkv, hd, write_kv=write_kv)
+
+    _check_qkv_rope(run, "interleaved", M, K, nh, nkv, hd)
+
+
+def _check_qkv_rope(run, pairing, M, K, nh, nkv, hd):
+    from burn_lm_amd.parts.rope import rope_frequencies
     g = torch.Generator().manual_seed(19)
     page, n_pages = 64, (16 if M <= 16 else 64)       # four pages for every sequence
     N = (nh + 2 * nkv) * hd
@@ -835,8 +857,7 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     v = torch.full((n_pages * 4, nkv, hd, page), 99.0).bfloat16()
     kd, vd = dev(k), dev(v)
     out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
-    ops.gemv_qkv_rope(dev(x), ops.pack_weight(dev(W)), out, dev(positions), dev(token_seq), dev(perm), dev(cs), kd, vd,
-                      page, nh, nkv, hd, PAIRING[pairing])
+    run(dev(x), dev(W), out, dev(positions), dev(token_seq), dev(perm), dev(cs), kd, vd, page, True)
     qkv = x.double() @ W.double().T
     q_ref = _rope_ref(qkv[:, : nh * hd].reshape(M, nh, hd), positions, freqs, pairing)
     k_ref = _rope_ref(qkv[:, nh * hd: (nh + nkv) * hd].reshape(M, nkv, hd), positions, freqs, pairing)
@@ -858,8 +879,7 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
     # a place that reads another's cache: queries only
     kd2 = dev(k)
     out2 = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
-    ops.gemv_qkv_rope(dev(x), ops.pack_weight(dev(W)), out2, dev(positions), dev(token_seq), dev(perm), dev(cs), kd2, dev(v),
-                      page, nh, nkv, hd, PAIRING[pairing], write_kv=False)
+    run(dev(x), dev(W), out2, dev(positions), dev(token_seq), dev(perm), dev(cs), kd2, dev(v), page, False)
     assert torch.equal(out2.cpu(), out.cpu()) and bool((kd2.cpu() == 99).all())
 
 
