@@ -38,6 +38,21 @@ MFMA_SKINNY_MAX_ROWS = 64
 FUSED_GATE_UP_ROWS = (192, 4096)
 
 
+def rows_plan(N, K, compute_units):
+    """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial
+    planes (ops.gemm_rows).  A group spans about 2048 of K (measured at the 1B, 3B and 8B layer
+    shapes: shorter groups write more planes than they gain, longer ones leave compute units
+    idle); 32 columns per block where that gives at most one block per compute unit, else 64;
+    and a short K is cut further, down to 512, until three quarters of the units have a block."""
+    groups = 1
+    while groups < 8 and K // (groups * 2) >= 2048:
+        groups *= 2
+    columns = 32 if -(-N // 32) * groups <= compute_units else 64
+    while groups < 8 and K // (groups * 2) >= 512 and -(-N // columns) * groups * 4 < compute_units * 3:
+        groups *= 2
+    return groups, columns
+
+
 class LinearWeight:
     """A bound weight matrix [N, K] and, for bfloat16, its copy packed for the skinny product."""
 
@@ -117,18 +132,8 @@ class Runtime:
         return g
 
     def rows_plan(self, N, K):
-        """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial
-        planes (ops.gemm_rows).  A group spans about 2048 of K (measured at the 1B, 3B and 8B layer
-        shapes: shorter groups write more planes than they gain, longer ones leave compute units
-        idle); 32 columns per block where that gives at most one block per compute unit, else 64;
-        and a short K is cut further, down to 512, until three quarters of the units have a block."""
-        groups = 1
-        while groups < 8 and K // (groups * 2) >= 2048:
-            groups *= 2
-        columns = 32 if -(-N // 32) * groups <= self.compute_units else 64
-        while groups < 8 and K // (groups * 2) >= 512 and -(-N // columns) * groups * 4 < self.compute_units * 3:
-            groups *= 2
-        return groups, columns
+        """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial planes."""
+        return rows_plan(N, K, self.compute_units)
 
     def mid_k_groups(self, M, N, K):
         """Short prompts, narrow output, long K (the down projection): the product as partial planes

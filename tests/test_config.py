@@ -224,3 +224,19 @@ def test_text_comes_out_piece_by_piece_as_the_whole_would():
     dec = StreamingDecoder(ByteTokenizer())
     cut = ByteTokenizer().encode("aé")[:-1]
     assert [dec.push(t) for t in cut] == ["a", ""] and dec.flush() == "�"
+
+
+def test_how_a_product_of_17_to_64_rows_is_cut():
+    """Groups of about 2048 of K, 32 columns per block where that is one round of blocks on 256 compute
+    units, a short K cut further until most units have a block; a tiny product is not cut at all (it
+    then stays with the packed kernel)."""
+    from burn_lm_amd.engine.runtime import rows_plan
+    shapes = {"1b o": (2048, 2048), "1b down": (2048, 8192), "3b o": (3072, 3072), "3b down": (3072, 8192),
+              "8b o": (4096, 4096), "8b down": (4096, 14336), "tiny": (72, 136), "narrow": (64, 1200)}
+    got = {k: rows_plan(n, kk, 256) for k, (n, kk) in shapes.items()}
+    assert got == {"1b o": (4, 32), "1b down": (4, 32), "3b o": (2, 32), "3b down": (4, 64), "8b o": (2, 32),
+                   "8b down": (4, 64), "tiny": (1, 32), "narrow": (2, 32)}
+    for n, kk in shapes.values():
+        groups, columns = rows_plan(n, kk, 256)
+        assert groups == 1 or kk // groups >= 512
+        assert columns in (32, 64)
