@@ -241,6 +241,17 @@ class Runtime:
                 if self.compute_units // 4 <= blocks <= self.compute_units:
                     return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
                                          gated=True, tile=tile)
+            # 256x128 tiles that make one round on at least three quarters of the compute units, with rows
+            # that fill their tiles to 85 % and more: measured against the library's product and the gating
+            # kernel 11-16 % faster with a full round (512 rows of an inner size of 8192 at widths 2048 and
+            # 3072; 900 and 1,024 rows of an inner size of 4096), 6 % with three quarters of one (700 and 768
+            # rows, inner 4096); rows that fill their tiles less (320, 520, 600) are equal or 5 % behind, and
+            # one and a half rounds and more 15-30 % behind.
+            m256 = -(-M // 256)
+            blocks = m256 * -(-inner // 64)
+            if M > 256 and M * 20 >= m256 * 256 * 17 and self.compute_units * 3 // 4 <= blocks <= self.compute_units:
+                return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
+                                     gated=True, tile=(256, 128))
             # Long prompts: with whole rounds of 256x256 tiles (as many blocks as compute units, or a
             # multiple) and a narrow model the fused kernel is ahead of the library over the whole
             # prefill (width 2048: 2-4 % at 1,024 and 2,048 rows, 0.5-0.8 % at 3,072 and 4,096; behind by

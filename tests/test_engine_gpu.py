@@ -358,9 +358,10 @@ def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
                                                            real(*a, **k))[1])
     eng = load(folder, "bfloat16", max_tokens=4096, graphs=False)
     # 70 rows: 128 blocks of the 128x64 tile; 100 + 150 rows: 256 of them; 300 + 90: 512, so the 128x128
-    # tile with 256; 700 rows: the library (96 tiles of 256x256 are no whole round); 2,000 rows: 256 such tiles
-    for lengths, tile in (([70], (128, 64, 6)), ([100, 150], (128, 64, 6)), ([300, 90], (128, 128, 4)), ([700], None),
-                          ([1500, 500], (256, 256))):
+    # tile with 256; 700 rows: 192 tiles of 256x128, one round on three quarters of the units; 600 rows fill
+    # such tiles too little: the library; 2,000 rows: 256 tiles of 256x256
+    for lengths, tile in (([70], (128, 64, 6)), ([100, 150], (128, 64, 6)), ([300, 90], (128, 128, 4)), ([700], (256, 128)),
+                          ([600], None), ([1500, 500], (256, 256))):
         reqs = [random_tokens(300 + i + sum(lengths), 300, n) for i, n in enumerate(lengths)]
         want = [P.transformer_forward([r], plain)[0] for r in reqs]
         slots = [eng.open() for _ in reqs]
