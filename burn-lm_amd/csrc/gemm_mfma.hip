@@ -6,10 +6,10 @@
 // tiles are staged the same way: 16 bytes per lane from global memory straight into a ring of NS
 // shared-memory buffers (no registers in between), NS - 1 stages ahead of the multiplications: a
 // load takes longer than a stage's multiplications, and one or two wavefronts per SIMD have little
-// else to hide it behind.  (The loads are inline assembly, see gm_dma16.)  The pieces of a staged row are permuted so that a fragment read meets every
-// bank once.  A wavefront owns its part of the tile as 32x32 accumulators of the 32x32x16
-// instruction; per k-step of 16 it reads one fragment per 32 rows and per 32 columns and
-// multiplies every pair.
+// else to hide it behind.  (The loads are inline assembly, see blm_dma16 in common.h.)  The pieces of
+// a staged row are permuted so that a fragment read meets every bank once.  A wavefront owns its
+// part of the tile as 32x32 accumulators of the 32x32x16 instruction; per k-step of 16 it reads one
+// fragment per 32 rows and per 32 columns and multiplies every pair.
 //
 // mode 1: W holds gate rows [0, I) and up rows [I, 2I) of a gated feed-forward; a block takes
 // BN / 2 gate columns and the matching up columns, each wavefront both halves of its pairs, and
@@ -31,27 +31,11 @@ __device__ __align__(16) const uint32_t gm_zero_piece[4] = {0u, 0u, 0u, 0u};
 #define GM_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 #define GM_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
 
-typedef __attribute__((address_space(3))) void* gm_lds_ptr;
 
 // scheduling hints: the next `n` instructions of a kind, in the order the hints are given
 #define GM_SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
 #define GM_SCHED_VMEM(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
 #define GM_SCHED_DSREAD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
-
-// One direct load of 16 bytes per lane from global memory (uniform base + per-lane byte offset, or a
-// full address per lane) into shared memory at lds (uniform) + 16 * lane.  Written as assembly: when the
-// compiler knows of such a load it waits for every outstanding one in front of the next read of shared
-// memory, whatever buffer that read goes to, so that a ring of three and more stages never had more
-// than one in flight; the waits are the kernel's own (GM_WAIT_VM; loads complete in order).  m0 holds
-// the address in shared memory; nothing else in this kernel reads m0.
-__device__ __forceinline__ void gm_dma16(const char* base, uint32_t lane_offset, const void* lds) {
-  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(gm_lds_ptr)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base));
-}
-__device__ __forceinline__ void gm_dma16_lanes(const char* address, const void* lds) {
-  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(gm_lds_ptr)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(address));
-}
 
 // x * sigmoid(x) with the hardware's exponential and reciprocal (each within an ulp; the result is
 // rounded to bf16 afterwards): 128 of these per lane would otherwise cost as much as 6 % of a tile
@@ -134,10 +118,10 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
     const char* bb = b_base + (size_t)k0 * 2;
 #pragma unroll
     for (int i = 0; i < A_LD; ++i)
-      gm_dma16(ab, a_off[i], As + (buf * BM + (wave * A_LD + i) * RPL) * BK);
+      blm_dma16(ab, a_off[i], As + (buf * BM + (wave * A_LD + i) * RPL) * BK);
 #pragma unroll
     for (int i = 0; i < B_LD; ++i)
-      gm_dma16(bb, b_off[i], Bs + (buf * BN + (wave * B_LD + i) * RPL) * BK);
+      blm_dma16(bb, b_off[i], Bs + (buf * BN + (wave * B_LD + i) * RPL) * BK);
   };
   auto fetch = [&](int k0, int buf) {
     if (k0 + BK <= k_end) {
@@ -152,13 +136,13 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
     for (int i = 0; i < A_LD; ++i) {
       const int r = (wave * A_LD + i) * RPL + st_row;
       const bool in = k0 + (st_slot ^ ((r / RPB) % P)) * 8 < k_end;
-      gm_dma16_lanes(in ? ab + a_off[i] : zero_piece, As + (buf * BM + (wave * A_LD + i) * RPL) * BK);
+      blm_dma16_lanes(in ? ab + a_off[i] : zero_piece, As + (buf * BM + (wave * A_LD + i) * RPL) * BK);
     }
 #pragma unroll
     for (int i = 0; i < B_LD; ++i) {
       const int r = (wave * B_LD + i) * RPL + st_row;
       const bool in = k0 + (st_slot ^ ((r / RPB) % P)) * 8 < k_end;
-      gm_dma16_lanes(in ? bb + b_off[i] : zero_piece, Bs + (buf * BN + (wave * B_LD + i) * RPL) * BK);
+      blm_dma16_lanes(in ? bb + b_off[i] : zero_piece, Bs + (buf * BN + (wave * B_LD + i) * RPL) * BK);
     }
   };
 

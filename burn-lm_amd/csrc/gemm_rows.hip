@@ -27,28 +27,11 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 gr_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float gr_f32x16;
-typedef __attribute__((address_space(3))) void* gr_lds_ptr;
 
 __device__ __align__(16) const uint32_t gr_zero_piece[4] = {0u, 0u, 0u, 0u};
 
 #define GR_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 #define GR_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
-
-// One direct load of 16 bytes per lane from global memory (uniform base + per-lane byte offset) into
-// shared memory at lds (uniform) + 16 * lane.  Written as assembly because the compiler, when it knows
-// of such a load, waits for every outstanding one in front of the next read of shared memory, whatever
-// slot that read goes to; here the waits are written out (loads complete in order).  m0 holds the
-// address in shared memory; nothing else in these kernels reads m0.
-__device__ __forceinline__ void gr_dma16(const char* base, uint32_t lane_offset, const void* lds) {
-  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(gr_lds_ptr)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base)
-               : "memory");
-}
-// the same with a full address per lane
-__device__ __forceinline__ void gr_dma16_lanes(const char* address, const void* lds) {
-  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(gr_lds_ptr)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(address) : "memory");
-}
 
 // what mode 2 needs beside the product: positions and sequences of the rows, the pages, the table of
 // cosines and sines, the cache planes (keys [pages, nkv, page, hd], values [pages, nkv, hd, page])
@@ -115,9 +98,9 @@ __global__ void __launch_bounds__(256)
     const char* bb = b_base + (size_t)k0 * 2;
     if (k0 + BK <= k_end) {
 #pragma unroll
-      for (int i = 0; i < A_LD; ++i) gr_dma16(ab, a_off[i], s + i * RPL * BK);
+      for (int i = 0; i < A_LD; ++i) blm_dma16(ab, a_off[i], s + i * RPL * BK);
 #pragma unroll
-      for (int i = 0; i < B_LD; ++i) gr_dma16(bb, b_off[i], s + (BM + i * RPL) * BK);
+      for (int i = 0; i < B_LD; ++i) blm_dma16(bb, b_off[i], s + (BM + i * RPL) * BK);
     } else {
       // the last stage of a K that is no multiple of BK: pieces beyond the end come from a zero constant
       const char* zero_piece = reinterpret_cast<const char*>(gr_zero_piece);
@@ -125,13 +108,13 @@ __global__ void __launch_bounds__(256)
       for (int i = 0; i < A_LD; ++i) {
         const int r = i * RPL + st_row;
         const bool in = k0 + (st_slot ^ ((r / RPB) % P)) * 8 < k_end;
-        gr_dma16_lanes(in ? ab + a_off[i] : zero_piece, s + i * RPL * BK);
+        blm_dma16_lanes(in ? ab + a_off[i] : zero_piece, s + i * RPL * BK);
       }
 #pragma unroll
       for (int i = 0; i < B_LD; ++i) {
         const int r = i * RPL + st_row;
         const bool in = k0 + (st_slot ^ ((r / RPB) % P)) * 8 < k_end;
-        gr_dma16_lanes(in ? bb + b_off[i] : zero_piece, s + (BM + i * RPL) * BK);
+        blm_dma16_lanes(in ? bb + b_off[i] : zero_piece, s + (BM + i * RPL) * BK);
       }
     }
   };
