@@ -451,6 +451,20 @@ def test_float32_product_is_true_32_bit(ops):
     assert torch.equal(out.cpu(), torch.full((150, 70), 16.0 + 2.0 ** -16))
 
 
+@pytest.mark.parametrize("M", [8, 17, 64])
+def test_float32_product_keeps_its_accuracy_over_a_long_sum(ops, M):
+    """8,200 terms of one sign: a single accumulator that takes them one after the other is off by
+    5e-6 of the result at the end (measured), sums in two levels or across lanes by a tenth of that."""
+    g = torch.Generator().manual_seed(12)
+    N, K = 200, 8200
+    A = torch.randn(M, K, generator=g).abs()
+    W = torch.randn(N, K, generator=g).abs() * 0.05
+    out = torch.empty(M, N, device="cuda")
+    (ops.gemv_skinny if M <= 8 else ops.gemm_tiled)(dev(A), dev(W), out)
+    want = A.double() @ W.double().T
+    assert float((out.cpu().double() - want).abs().max() / want.abs().max()) < 1e-6
+
+
 @pytest.mark.parametrize("dtype,out_dtype", [("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")])
 @pytest.mark.parametrize("M", [1, 2, 3, 5, 8])
 def test_gemv_skinny(ops, dtype, out_dtype, M):
