@@ -45,6 +45,8 @@ struct GrRope {
   int table_width, page_size, nh, nkv, hd, store;
 };
 
+#define GR_MAX_ROWS 256   // four blocks of 64 rows
+
 template <int BM, int BN, int BK, int R, int MODE, typename TC>
 __global__ void __launch_bounds__(256)
     gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, TC* __restrict__ C, int M, int N, int K, int lda,
@@ -69,7 +71,15 @@ __global__ void __launch_bounds__(256)
   const int n0 = blockIdx.x * (MODE == 1 ? BN / 2 : BN);   // first output column
   if (MODE == 2 && !rope.store && n0 >= rope.nh * rope.hd) return;   // keys and values belong to another layer's cache
   const int k_begin = blockIdx.y * k_per_group, k_end = min(K, k_begin + k_per_group);
-  C += (size_t)blockIdx.y * M * ldc;
+  // more rows than one block stages: blockIdx.z counts blocks of BM rows, each a product of its own
+  const int m0 = blockIdx.z * BM;
+  C += ((size_t)blockIdx.y * M + m0) * ldc;
+  A += (size_t)m0 * lda;
+  M = min(BM, M - m0);
+  if (MODE == 2) {
+    rope.positions += m0;
+    rope.token_seq += m0;
+  }
   bf16* ring = reinterpret_cast<bf16*>(gr_smem) + (size_t)wave * R * SLOT;
 
   // staging: lane l of a load instruction brings piece (l % P) ^ swizzle of row l / P of its RPL rows
@@ -287,7 +297,7 @@ static int gr_launch(const void* A, const void* W, void* C, int M, int N, int K,
   static_assert(smem >= (size_t)4 * BM * (BN + 4) * sizeof(float), "the partial tiles fit where the ring was");
   const int n_tiles = (N + (MODE == 1 ? BN / 2 : BN) - 1) / (MODE == 1 ? BN / 2 : BN);
   const int k_per_group = ((K + k_groups - 1) / k_groups + BK - 1) / BK * BK;
-  dim3 grid((unsigned)n_tiles, (unsigned)k_groups), block(256);
+  dim3 grid((unsigned)n_tiles, (unsigned)k_groups, (unsigned)((M + BM - 1) / BM)), block(256);
   hipLaunchKernelGGL((gemm_rows_kernel<BM, BN, BK, R, MODE, TC>), grid, block, smem, stream, (const bf16*)A, (const bf16*)W, (TC*)C, M,
                      N, K, lda, ldw, ldc, k_per_group, rope);
   BLM_LAUNCH_CHECK("gemm_rows");
@@ -312,8 +322,8 @@ extern "C" int blm_gemm_rows_init() {
 // compute unit a block, else 64) at all of them.
 extern "C" int blm_gemm_rows(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc,
                              int mode, int k_groups, int columns, hipStream_t stream) {
-  BLM_REQUIRE(M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0, "gemm_rows: sizes M=%d N=%d K=%d not supported (M <= 64, K a multiple of 8)",
-              M, N, K);
+  BLM_REQUIRE(M >= 1 && M <= GR_MAX_ROWS && N >= 1 && K >= 8 && K % 8 == 0,
+              "gemm_rows: sizes M=%d N=%d K=%d not supported (M <= %d, K a multiple of 8)", M, N, K, GR_MAX_ROWS);
   BLM_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= N, "gemm_rows: bad strides lda=%d ldw=%d ldc=%d", lda, ldw, ldc);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_rows: operands must be 16-byte aligned");
   BLM_REQUIRE(columns == 64 || (columns == 32 && mode == 0), "gemm_rows: %d columns per block: 64, or 32 without gating", columns);
@@ -349,8 +359,9 @@ extern "C" int blm_gemm_rows_qkv_rope(const void* A, const void* W, void* qkv_ou
                                       const int* block_table, int table_width, const float* cos_sin, void* kcache, void* vcache,
                                       int page_size, int M, int K, int lda, int ldw, int ldq, int nh, int nkv, int hd, int store,
                                       hipStream_t stream) {
-  BLM_REQUIRE(M >= 1 && M <= 64 && K >= 8 && K % 8 == 0 && hd >= 2 && hd % 2 == 0,
-              "gemm_rows_qkv_rope: M=%d K=%d head_dim=%d not supported (M <= 64, K a multiple of 8, an even head size)", M, K, hd);
+  BLM_REQUIRE(M >= 1 && M <= GR_MAX_ROWS && K >= 8 && K % 8 == 0 && hd >= 2 && hd % 2 == 0,
+              "gemm_rows_qkv_rope: M=%d K=%d head_dim=%d not supported (M <= %d, K a multiple of 8, an even head size)", M, K, hd,
+              GR_MAX_ROWS);
   BLM_REQUIRE(nh > 0 && nkv > 0 && page_size > 0 && table_width > 0, "gemm_rows_qkv_rope: bad geometry");
   BLM_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldq >= nh * hd && ldq % 2 == 0,
               "gemm_rows_qkv_rope: bad strides lda=%d ldw=%d ldq=%d", lda, ldw, ldq);

@@ -10,6 +10,8 @@ Matrix products ``x[M,K] @ w[N,K]^T``:
   on, the gated product run on the kernel whose wavefronts each stream their own stages of K through
   shared memory (ops.gemm_rows): with that many rows the activations cost as much traffic as the
   weights, and its loads never stop for a barrier (see rows_plan and gated_linear).
+* bfloat16 weights, 65 to 256 rows, K up to 2048 and few columns (the output projection at the 1B
+  width): ops.gemm_rows again, a block for every 64 rows (see mid_rows_ring).
 * bfloat16 weights, 65 rows and more, narrow output and long K (the down projection of short
   prompts): partial planes from the hand-written matrix-core kernel (see mid_k_groups).
 * bfloat16 weights, many rows (prefill): the library product (hipBLASLt through torch), as the
@@ -135,6 +137,25 @@ class Runtime:
         """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial planes."""
         return rows_plan(N, K, self.compute_units)
 
+    def mid_rows_ring(self, M, N, K, planes):
+        """65 to 256 rows, K up to 2048, few columns (the output projection of short prompts and of decode
+        steps of many sequences at the 1B width): the product of 17 to 64 rows with a block for every 64
+        rows, while all its blocks of 32 columns run at once.  Returns the groups of K (two where that
+        still gives every block a compute unit and the caller takes partial planes), 0 for another kernel.
+        Measured per call at the 1B shape against the library's product: 6.8-7.2 against 9.8 us at 65-128
+        rows, 8.0 against 10.8 at 192, 8.9 against 11.1 at 256; at K = 3072 and 4096 (3B, 8B) equal or
+        behind, hence the bound on K."""
+        if not (self.rows_ring and MFMA_SKINNY_MAX_ROWS < M <= 256 and K <= 2048):
+            return 0
+        blocks = self.rows_ring_blocks(M, N)
+        if blocks > self.compute_units:
+            return 0
+        return 2 if planes and K >= 1024 and blocks * 2 <= self.compute_units else 1
+
+    def rows_ring_blocks(self, M, N):
+        """Blocks of 64 rows and 32 columns that ops.gemm_rows and ops.gemm_rows_qkv_rope launch."""
+        return -(-N // 32) * -(-M // 64)
+
     def mid_k_groups(self, M, N, K):
         """Short prompts, narrow output, long K (the down projection): the product as partial planes
         of 128x64 tiles over groups of K (the block's next norm sums the planes), when eight, four
@@ -168,6 +189,14 @@ class Runtime:
                 return ops.gemv_skinny(x, w, out)
             return ops.gemm_tiled(x, w, out)
         aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+        if (M > MFMA_SKINNY_MAX_ROWS and aligned and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1
+                and w.is_contiguous() and out_dtype == torch.bfloat16):
+            groups = self.mid_rows_ring(M, N, K, planes=partials and out is None)
+            if groups > 1:
+                return ops.gemm_rows(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), columns=32)
+            if groups == 1:
+                return ops.gemm_rows(x, w, out if out is not None else torch.empty(M, N, dtype=out_dtype, device=x.device),
+                                     columns=32)
         if (partials and out is None and self.mid_partials and M > self.skinny_planes_rows and aligned
                 and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()):
             groups = self.mid_k_groups(M, N, K)

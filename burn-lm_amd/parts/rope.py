@@ -96,7 +96,14 @@ class RotaryEncoding(PositionEncoding):
         packed = getattr(w_qkv, "packed", None)
         M, K = x.shape
         raw = getattr(w_qkv, "w", None)
-        if (16 < M <= 64 and (M > 32 or K > 2048) and self.pairing == PAIRING["interleaved"] and getattr(rt, "rows_ring", False)
+        few = 16 < M <= 64 and (M > 32 or K > 2048)
+        # 65 to 256 rows: the same kernel with a block for every 64 rows, while its blocks of 32 columns (nearly) all
+        # run at once (per layer at the 1B shape against the library's product and the rotation kernel: 10 against
+        # 14-16 us at 65-128 rows, 16.5 against 21 at 192, behind at 256; at the 3B and 8B shapes, which have more
+        # columns, equal or behind)
+        mid = (64 < M <= 256 and getattr(rt, "rows_ring", False)
+               and rt.rows_ring_blocks(M, (heads + 2 * kv_heads) * head_dim) * 20 <= rt.compute_units * 23)
+        if ((few or mid) and self.pairing == PAIRING["interleaved"] and getattr(rt, "rows_ring", False)
                 and raw is not None
                 and x.dtype == raw.dtype == view.k.dtype == torch.bfloat16 and head_dim % 2 == 0 and K % 8 == 0
                 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and raw.is_contiguous()):

@@ -55,18 +55,25 @@ def rel_err(got, want):
 
 
 class Trace:
-    """Collects steps for bin/trace_run and remembers which (request, position) each wanted row is."""
+    """Collects steps for bin/trace_run and remembers which (request, position) each wanted row is, and
+    for each step and request how the request's tokens so far were fed (history)."""
 
     def __init__(self):
         self.lines, self.index, self.n = [], {}, 0
         self.live, self.peak = {}, 0
+        self.fed_by, self.history = {}, {}
 
     def step(self, entries, end=()):
         """entries: (request id, start position, tokens, want list)."""
         rows = []
+        total = sum(len(toks) for _, _, toks, _ in entries)
         for rid, start, toks, want in entries:
             rows += [(rid, start + w) for w in want]
             self.live[rid] = start + len(toks)
+            # for every token the request holds, the rows of the step that fed it and whether it came alone
+            self.fed_by[rid] = (self.fed_by[rid] if start else []) + [(total, len(toks) == 1 and start > 0)] * len(toks)
+            if want:
+                self.history[self.n, rid] = list(self.fed_by[rid])
         self.peak = max(self.peak, sum((n + 63) // 64 * 64 for n in self.live.values()))
         for rid in end:
             self.live.pop(rid)

@@ -356,6 +356,10 @@ def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
     planes = []
     monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: ((tiles if k.get("gated") else planes).append(k.get("tile")),
                                                            real(*a, **k))[1])
+    rings, real_rows = [], ops.gemm_rows
+    monkeypatch.setattr(ops, "gemm_rows", lambda a, w, out, **k: (rings.append(tuple(out.shape)), real_rows(a, w, out, **k))[1])
+    fused_qkv, real_qkv = [], ops.gemm_rows_qkv_rope
+    monkeypatch.setattr(ops, "gemm_rows_qkv_rope", lambda x, *a, **k: (fused_qkv.append(x.shape[0]), real_qkv(x, *a, **k))[1])
     eng = load(folder, "bfloat16", max_tokens=4096, graphs=False)
     # 70 rows: 128 blocks of the 128x64 tile; 100 + 150 rows: 256 of them; 300 + 90: 512, so the 128x128
     # tile with 256; 700 rows: 192 tiles of 256x128, one round on three quarters of the units; 600 rows fill
@@ -365,12 +369,19 @@ def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
         reqs = [random_tokens(300 + i + sum(lengths), 300, n) for i, n in enumerate(lengths)]
         want = [P.transformer_forward([r], plain)[0] for r in reqs]
         slots = [eng.open() for _ in reqs]
-        del tiles[:], planes[:]
+        del tiles[:], planes[:], rings[:], fused_qkv[:]
         got = eng.step([(s, r, [0, len(r) // 2, len(r) - 1]) for s, r in zip(slots, reqs)]).double().cpu().numpy()
         assert tiles == ([tile] if tile else []), (lengths, tiles)
-        # the output and down projections come as partial planes where a few groups of K fill the chip
-        n_planes = sum(1 for N, K in ((2048, 2048), (2048, 4096)) if eng.rt.mid_k_groups(sum(lengths), N, K))
-        assert len(planes) == n_planes and (n_planes >= 1) == (sum(lengths) <= 512), (lengths, planes)
+        # up to 256 rows the output projection (K = 2048) runs on the product of 17 to 64 rows with a block for
+        # every 64 rows: two partial planes while that leaves every block a compute unit, else one result; the
+        # q/k/v projection with the rotation too while its 96 blocks of columns times the row blocks about fit
+        M = sum(lengths)
+        assert rings == ([(2, M, 2048)] if M <= 128 else [(M, 2048)] if M <= 256 else []), (lengths, rings)
+        assert fused_qkv == ([M] if M <= 192 else []), (lengths, fused_qkv)
+        # the other narrow products come as partial planes where a few groups of K fill the chip
+        n_planes = sum(1 for N, K in ((2048, 2048), (2048, 4096))
+                       if not eng.rt.mid_rows_ring(M, N, K, True) and eng.rt.mid_k_groups(M, N, K))
+        assert len(planes) == n_planes and (n_planes >= 1) == (M <= 512), (lengths, planes)
         for i, r in enumerate(reqs):
             for j, pos in enumerate([0, len(r) // 2, len(r) - 1]):
                 assert rel_err(got[3 * i + j], want[i][pos]) <= TOL["bfloat16"], (lengths, i, pos)

@@ -577,11 +577,12 @@ def test_gemv_mfma_gated(ops, M, I, K):
 
 @pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
 @pytest.mark.parametrize("M,N,K,columns", [(64, 128, 64, 64), (33, 200, 136, 32), (17, 72, 1000, 64), (32, 100, 264, 64), (20, 264, 520, 32),
-                                           (50, 96, 4104, 64), (1, 40, 72, 32), (48, 3072, 2048, 32), (64, 1000, 3080, 64)])
+                                           (50, 96, 4104, 64), (1, 40, 72, 32), (48, 3072, 2048, 32), (64, 1000, 3080, 64),
+                                           (65, 72, 136, 32), (130, 200, 264, 64), (256, 96, 1000, 32), (200, 64, 2048, 64)])
 def test_gemm_rows(ops, out_dtype, M, N, K, columns):
     """The product for 17 to 64 rows whose wavefronts each stream their own stages of K: both stagings of
     the rows (32 and 64), both widths of a block, tails in N, K and M, more and fewer stages than the
-    rings hold."""
+    rings hold; up to 256 rows as blocks of 64, the last one with 1, 2, 8 or all 64 rows."""
     g = torch.Generator().manual_seed(26)
     A = torch.randn(M, K, generator=g).bfloat16()
     W = (torch.randn(N, K, generator=g) * 0.1).bfloat16()
@@ -601,7 +602,7 @@ def test_gemm_rows(ops, out_dtype, M, N, K, columns):
 
 
 @pytest.mark.parametrize("M,N,K,groups,columns", [(64, 2048, 8192, 4, 32), (24, 100, 8200, 8, 64), (40, 48, 3000, 2, 32), (33, 64, 14336, 4, 64),
-                                                  (17, 200, 1096, 3, 32)])
+                                                  (17, 200, 1096, 3, 32), (100, 100, 2048, 2, 32), (192, 64, 3000, 3, 64)])
 def test_gemm_rows_partial_products_sum_to_the_product(ops, M, N, K, groups, columns):
     g = torch.Generator().manual_seed(27)
     A = torch.randn(M, K, generator=g).bfloat16()
@@ -614,7 +615,8 @@ def test_gemm_rows_partial_products_sum_to_the_product(ops, M, N, K, groups, col
     close(planes[groups - 1], A[:, (groups - 1) * per:].double() @ W[:, (groups - 1) * per:].double().T, 1e-5)
 
 
-@pytest.mark.parametrize("M,I,K", [(64, 1000, 2048), (20, 176, 1544), (37, 384, 144), (50, 8, 520), (32, 176, 4096), (33, 100, 3080)])
+@pytest.mark.parametrize("M,I,K", [(64, 1000, 2048), (20, 176, 1544), (37, 384, 144), (50, 8, 520), (32, 176, 4096), (33, 100, 3080),
+                                   (70, 176, 520), (256, 100, 264)])
 def test_gemm_rows_gated(ops, M, I, K):
     """The SwiGLU gating where the partial tiles of a block meet: w is [gate rows; up rows] as the checkpoint
     has them, a block takes 32 gate columns and the matching up columns."""
@@ -631,9 +633,9 @@ def test_gemm_rows_gated(ops, M, I, K):
 
 def test_gemm_rows_refuses_what_it_cannot_do(ops):
     from burn_lm_amd.csrc.ops import KernelError
-    a, w = dev(torch.zeros(65, 64).bfloat16()), dev(torch.zeros(8, 64).bfloat16())
-    with pytest.raises(KernelError, match="M <= 64"):
-        ops.gemm_rows(a, w, torch.zeros(65, 8, dtype=torch.bfloat16, device="cuda"))
+    a, w = dev(torch.zeros(257, 64).bfloat16()), dev(torch.zeros(8, 64).bfloat16())
+    with pytest.raises(KernelError, match="M <= 256"):
+        ops.gemm_rows(a, w, torch.zeros(257, 8, dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(KernelError, match="32 without gating"):
         ops.gemm_rows(a[:8], w, torch.zeros(8, 4, dtype=torch.bfloat16, device="cuda"), gated=True, columns=32)
     with pytest.raises(KernelError, match="32 without gating"):
@@ -839,10 +841,12 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
 
 
 @pytest.mark.parametrize("M,K,nh,nkv,hd", [(33, 2048, 4, 2, 64), (64, 520, 3, 1, 48), (20, 4096, 2, 1, 64), (17, 264, 30, 2, 128),
-                                           (48, 2056, 2, 1, 32), (64, 3072, 3, 1, 128), (40, 4104, 2, 2, 80), (32, 72, 1, 1, 6)])
+                                           (48, 2056, 2, 1, 32), (64, 3072, 3, 1, 128), (40, 4104, 2, 2, 80), (32, 72, 1, 1, 6),
+                                           (65, 264, 3, 1, 48), (128, 2048, 4, 2, 64), (200, 520, 2, 1, 128), (256, 72, 1, 1, 6)])
 def test_gemm_rows_qkv_rope(ops, M, K, nh, nkv, hd):
-    """The same for 17 to 64 rows on the product whose wavefronts stream their own stages of K: any K,
-    head sizes that put two heads into a block's 32 columns or a head across several blocks."""
+    """The same for 17 to 256 rows on the product whose wavefronts stream their own stages of K: any K,
+    head sizes that put two heads into a block's 32 columns or a head across several blocks, one to
+    four blocks of rows (each with its own rows' positions and sequences)."""
 
     def run(x, W, out, positions, token_seq, perm, cs, kd, vd, page, write_kv):
         ops.gemm_rows_qkv_rope(x, W, out, positions, token_seq, perm, cs, kd, vd, page, nh, nkv, hd, write_kv=write_kv)
@@ -853,7 +857,7 @@ def test_gemm_rows_qkv_rope(ops, M, K, nh, nkv, hd):
 def _check_qkv_rope(run, pairing, M, K, nh, nkv, hd):
     from burn_lm_amd.parts.rope import rope_frequencies
     g = torch.Generator().manual_seed(19)
-    page, n_pages = 64, (16 if M <= 16 else 64)       # four pages for every sequence
+    page, n_pages = 64, (16 if M <= 16 else max(64, M))       # four pages for every sequence
     N = (nh + 2 * nkv) * hd
     x = torch.randn(M, K, generator=g).bfloat16()
     W = (torch.randn(N, K, generator=g) / K ** 0.5).bfloat16()

@@ -2,10 +2,12 @@
 each request whole; with its last 32 tokens one by one; and in batches of unequal lengths whose
 shorter requests end earlier, one batch after another on a cache so small that pages and slots
 are used again.  In 32-bit and in bfloat16, on two tiny configurations and a middle-sized one."""
+import numpy as np
 import pytest
 
 import plain_llama as P
 from helpers import TINIES, TOL, Trace, make_folder, random_tokens, rel_err, run_trace
+from test_bf16_roundings import rounding_for
 
 pytestmark = pytest.mark.gpu
 
@@ -19,7 +21,7 @@ def case(request, tmp_path_factory):
     plain = P.load_model_folder(folder)
     reqs = {f"r{i}": random_tokens(100 * seed + i, cfg["vocab_size"], n) for i, n in enumerate(LENGTHS)}
     want = {rid: P.transformer_forward([t], plain)[0] for rid, t in reqs.items()}
-    return request.param, folder, reqs, want
+    return request.param, folder, reqs, want, plain
 
 
 def build_trace(reqs):
@@ -64,21 +66,37 @@ def build_trace(reqs):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_replay_matches_plain_whole_tail_and_batched(case, dtype, tmp_path):
-    name, folder, reqs, want = case
+    name, folder, reqs, want, plain = case
     tr, mode_of = build_trace(reqs)
     out = run_trace(folder, dtype, tr, tmp_path / "out")
     worst = {"whole": 0.0, "tail": 0.0, "batched": 0.0}
     seen = {m: set() for m in worst}
+    rounded, excused = {}, 0
     for step, rows in tr.index.items():
         got = out[step]
         for k, (rid, pos) in enumerate(rows):
             e = rel_err(got[k], want[rid][pos])
             m = mode_of[step]
             seen[m].add((rid, pos))
+            if e > TOL[dtype] and dtype == "bfloat16":
+                # About one row in a thousand of configuration B sits on a near-tie of its attention: exact
+                # arithmetic between the engine's roundings (the plain implementation with roundings, on the
+                # CPU) is then 0.03-0.04 of the largest logit from the exact result by itself (request r5, row
+                # 89: 0.042).  Such a row has to agree with that computation instead, and twice as closely.
+                fed = tr.history[step, rid]
+                if (step, rid) not in rounded:
+                    style = rounding_for(name, np.array([r for r, _ in fed]), np.array([d for _, d in fed]))
+                    rounded[step, rid] = P.transformer_forward([reqs[rid][:len(fed)]], plain, rounding=style)[0]
+                by_rounding = rel_err(rounded[step, rid][pos], want[rid][pos])
+                assert by_rounding > 0.8 * TOL[dtype] and rel_err(got[k], rounded[step, rid][pos]) <= TOL[dtype] / 2, \
+                    (f"config {name} {m}: request {rid} position {pos} differs by {e:.3g}; roundings alone give {by_rounding:.3g}")
+                excused += 1
+                continue
             if e > worst[m]:
                 worst[m] = e
             assert e <= TOL[dtype], (f"config {name} {dtype} {m}: request {rid} position {pos} of "
                                      f"{len(reqs[rid])} (step {step}) differs by {e:.3g} of the largest logit")
+    assert excused <= 3, excused
     everything = {(rid, p) for rid, t in reqs.items() for p in range(len(t))}
     assert seen["whole"] == everything and seen["tail"] == everything
     assert len(seen["batched"]) > 400
@@ -88,7 +106,7 @@ def test_replay_matches_plain_whole_tail_and_batched(case, dtype, tmp_path):
 def test_cache_is_sized_by_max_tokens(case, tmp_path):
     """--max-tokens counts each live request rounded up to 64: one token too few pages must be
     refused by the cache, not answered wrongly."""
-    name, folder, reqs, _ = case
+    name, folder, reqs, _, _ = case
     tr = Trace()
     tr.step([("a", 0, reqs["r5"][:65], [64]), ("b", 0, reqs["r2"], [0])])   # 128 + 64 tokens of room
     assert tr.peak == 192
