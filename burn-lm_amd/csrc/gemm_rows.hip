@@ -312,7 +312,7 @@ extern "C" int blm_gemm_rows_init() {
   GR_PREP(64, 64, 2, 0) GR_PREP(64, 32, 3, 0) GR_PREP(32, 64, 3, 0) GR_PREP(32, 32, 5, 0)
   GR_PREP(64, 64, 2, 1) GR_PREP(32, 64, 3, 1)
 #undef GR_PREP
-  if (gr_prepare<64, 32, 64, 3, 2, bf16>() || gr_prepare<32, 32, 64, 5, 2, bf16>()) return 1;
+  if (gr_prepare<64, 32, 64, 3, 2, bf16>() || gr_prepare<32, 32, 64, 5, 2, bf16>() || gr_prepare<64, 64, 64, 2, 2, bf16>()) return 1;
   return 0;
 }
 
@@ -350,15 +350,17 @@ extern "C" int blm_gemm_rows(const void* A, const void* W, void* C, int c_dtype,
 #undef GR_GO
 }
 
-// The q/k/v projection of 17 to 64 rows with the rotation and the cache write where the partial tiles meet
-// (32 columns per block).  W: W_qkv [(nh + 2 nkv) * hd, K] with rotary partners in adjacent rows; qkv_out:
+// The q/k/v projection of 17 to 256 rows with the rotation and the cache write where the partial tiles meet
+// (columns: 32 per block, or 64 with 64 rows staged and a ring of two, for shapes whose blocks of 32 columns
+// would not all run at once).  W: W_qkv [(nh + 2 nkv) * hd, K] with rotary partners in adjacent rows; qkv_out:
 // [M, ldq] bf16, of which only the first nh * hd columns (the rotated queries) are written; key plane
 // [pages, nkv, page, hd], value plane [pages, nkv, hd, page].  store = 0: keys and values are neither
 // computed nor written.
 extern "C" int blm_gemm_rows_qkv_rope(const void* A, const void* W, void* qkv_out, const int* positions, const int* token_seq,
                                       const int* block_table, int table_width, const float* cos_sin, void* kcache, void* vcache,
                                       int page_size, int M, int K, int lda, int ldw, int ldq, int nh, int nkv, int hd, int store,
-                                      hipStream_t stream) {
+                                      int columns, hipStream_t stream) {
+  BLM_REQUIRE(columns == 32 || columns == 64, "gemm_rows_qkv_rope: %d columns per block: 32 or 64", columns);
   BLM_REQUIRE(M >= 1 && M <= GR_MAX_ROWS && K >= 8 && K % 8 == 0 && hd >= 2 && hd % 2 == 0,
               "gemm_rows_qkv_rope: M=%d K=%d head_dim=%d not supported (M <= %d, K a multiple of 8, an even head size)", M, K, hd,
               GR_MAX_ROWS);
@@ -372,6 +374,7 @@ extern "C" int blm_gemm_rows_qkv_rope(const void* A, const void* W, void* qkv_ou
               "gemm_rows_qkv_rope: matrices of 4 GiB and more are not supported");
   const GrRope rope{positions, token_seq, block_table, (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache,
                     table_width, page_size, nh, nkv, hd, store};
+  if (columns == 64) return gr_launch<64, 64, 64, 2, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
   if (M > 32) return gr_launch<64, 32, 64, 3, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
   return gr_launch<32, 32, 64, 5, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
 }

@@ -152,9 +152,9 @@ class Runtime:
             return 0
         return 2 if planes and K >= 1024 and blocks * 2 <= self.compute_units else 1
 
-    def rows_ring_blocks(self, M, N):
-        """Blocks of 64 rows and 32 columns that ops.gemm_rows and ops.gemm_rows_qkv_rope launch."""
-        return -(-N // 32) * -(-M // 64)
+    def rows_ring_blocks(self, M, N, columns=32):
+        """Blocks of 64 rows and 32 or 64 columns that ops.gemm_rows and ops.gemm_rows_qkv_rope launch."""
+        return -(-N // columns) * -(-M // 64)
 
     def mid_k_groups(self, M, N, K):
         """Short prompts, narrow output, long K (the down projection): the product as partial planes

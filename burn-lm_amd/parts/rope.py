@@ -97,12 +97,18 @@ class RotaryEncoding(PositionEncoding):
         M, K = x.shape
         raw = getattr(w_qkv, "w", None)
         few = 16 < M <= 64 and (M > 32 or K > 2048)
-        # 65 to 256 rows: the same kernel with a block for every 64 rows, while its blocks of 32 columns (nearly) all
-        # run at once (per layer at the 1B shape against the library's product and the rotation kernel: 10 against
-        # 14-16 us at 65-128 rows, 16.5 against 21 at 192, behind at 256; at the 3B and 8B shapes, which have more
-        # columns, equal or behind)
-        mid = (64 < M <= 256 and getattr(rt, "rows_ring", False)
-               and rt.rows_ring_blocks(M, (heads + 2 * kv_heads) * head_dim) * 20 <= rt.compute_units * 23)
+        # 65 to 256 rows: the same kernel with a block for every 64 rows: 32 columns per block while those blocks all
+        # run at once, else 64 while there are at most one and a half per compute unit (per layer against the
+        # library's product and the rotation kernel: 1B shape 10 against 14-16 us at 65-128 rows, 13.3 against 21
+        # at 192, 13.6 against 16 at 256; 3B 16-17 against 18-27 at 65-192, 28.5 against 33 at 256; 8B 21-24.5
+        # against 28-31 at 65-128, 36 against 39 at 192, 38.5 against 46 at 256)
+        columns, mid = 32, False
+        if 64 < M <= 256 and getattr(rt, "rows_ring", False):
+            n_qkv = (heads + 2 * kv_heads) * head_dim
+            if rt.rows_ring_blocks(M, n_qkv) <= rt.compute_units:
+                mid = True
+            elif rt.rows_ring_blocks(M, n_qkv, 64) * 2 <= rt.compute_units * 3:
+                columns, mid = 64, True
         if ((few or mid) and self.pairing == PAIRING["interleaved"] and getattr(rt, "rows_ring", False)
                 and raw is not None
                 and x.dtype == raw.dtype == view.k.dtype == torch.bfloat16 and head_dim % 2 == 0 and K % 8 == 0
@@ -116,7 +122,8 @@ class RotaryEncoding(PositionEncoding):
                 raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
             qkv = torch.empty(M, (heads + 2 * kv_heads) * head_dim, dtype=torch.bfloat16, device=x.device)
             return rt.ops.gemm_rows_qkv_rope(x, raw, qkv, step.positions, step.token_seq, view.block_table(step), self.table,
-                                             view.k, view.v, view.page_size, heads, kv_heads, head_dim, write_kv=view.store)
+                                             view.k, view.v, view.page_size, heads, kv_heads, head_dim, write_kv=view.store,
+                                             columns=columns)
         if (packed is not None and not getattr(w_qkv, "gated", False) and x.dtype == torch.bfloat16
                 and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing) and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0 and view.k.dtype == torch.bfloat16):
