@@ -86,8 +86,8 @@ __global__ void __launch_bounds__(256)
 }
 
 // ---------------------------------------------------------------------------------------
-// the same product on the matrix cores' float instruction: 128x128 tile per 256 threads, each
-// wavefront a 64x64 quarter as 2x2 instructions of 32x32, K in steps of 16 through shared memory
+// the same product on the matrix cores' float instruction: 128x128 tile per 512 threads, each
+// wavefront 64 rows x 32 columns as two instructions of 32x32, K in steps of 16 through shared memory
 // (operands of either type become float there).  Lane l of a 32x32x2 instruction supplies
 // A[l % 32][l / 32] and B[l / 32][l % 32] and holds C[8 (v / 4) + 4 (l / 32) + v % 4][l % 32], v < 16.
 // ---------------------------------------------------------------------------------------
@@ -98,85 +98,74 @@ __global__ void __launch_bounds__(256)
 typedef __attribute__((ext_vector_type(16))) float gf_f32x16;
 
 template <typename TA, typename TW, typename TC>
-__global__ void __launch_bounds__(256, 2)   // two wavefronts per SIMD: left to itself the compiler takes 300 registers and runs one
+__global__ void __launch_bounds__(512, 4)   // 128 registers: two blocks per compute unit
     gemm_f32_mfma_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
                          int lda, int ldc) {
   __shared__ float As[GF_BK][GF_BM + 4];
   __shared__ float Ws[GF_BK][GF_BN + 4];
   const int tid = threadIdx.x, wave = tid / BLM_WAVE, lane = tid & (BLM_WAVE - 1);
   const int m0 = blockIdx.y * GF_BM, n0 = blockIdx.x * GF_BN;
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int wm = (wave >> 2) * 64, wn = (wave & 3) * 32;   // eight wavefronts, each 64 rows x 32 columns
   const int li = lane & 31, lk = lane >> 5;
   // Sums in two levels: `acc` takes the products of GF_CHUNK elements of K and is then added to
   // `total`.  One accumulator over all of K would make K/2 additions in a row to a sum that keeps
   // growing, and its rounding error grows with them (measured at K = 8,192 against a 64-bit
-  // product: 5e-6 of the largest result, four times a product that is split over K).
-  gf_f32x16 total[2][2];
+  // product: 5e-6 of the largest result, four times a product that is split over K).  The second
+  // set of sums is why a wavefront's tile is no larger: with 64 x 64 the two sets take the
+  // registers of half the wavefronts.
+  gf_f32x16 total[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) total[i][j][v] = 0.f;
+    for (int v = 0; v < 16; ++v) total[i][v] = 0.f;
   for (int c0 = 0; c0 < K; c0 += GF_CHUNK) {
-  gf_f32x16 acc[2][2];
+    gf_f32x16 acc[2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+    const int c1 = c0 + GF_CHUNK < K ? c0 + GF_CHUNK : K;
+    for (int k0 = c0; k0 < c1; k0 += GF_BK) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-  const int c1 = c0 + GF_CHUNK < K ? c0 + GF_CHUNK : K;
-  for (int k0 = c0; k0 < c1; k0 += GF_BK) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {   // 128 rows x 16 k per operand, 8 elements per thread, k fastest
-      const int idx = tid + e * 256;
-      const int r = idx / GF_BK, kk = idx % GF_BK;
-      const int gk = k0 + kk;
-      float a = 0.f, w = 0.f;
-      if (gk < K) {
-        if (m0 + r < M) a = to_float(A[(size_t)(m0 + r) * lda + gk]);
-        if (n0 + r < N) w = to_float(W[(size_t)(n0 + r) * K + gk]);
+      for (int e = 0; e < 4; ++e) {   // 128 rows x 16 k per operand, 4 elements per thread, k fastest
+        const int idx = tid + e * 512;
+        const int r = idx / GF_BK, kk = idx % GF_BK;
+        const int gk = k0 + kk;
+        float a = 0.f, w = 0.f;
+        if (gk < K) {
+          if (m0 + r < M) a = to_float(A[(size_t)(m0 + r) * lda + gk]);
+          if (n0 + r < N) w = to_float(W[(size_t)(n0 + r) * K + gk]);
+        }
+        As[kk][r] = a;
+        Ws[kk][r] = w;
       }
-      As[kk][r] = a;
-      Ws[kk][r] = w;
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < GF_BK; kk += 2) {
+        const float b = Ws[kk + lk][wn + li];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(As[kk + lk][wm + i * 32 + li], b, acc[i], 0, 0, 0);
+      }
+      __syncthreads();
     }
-    __syncthreads();
 #pragma unroll
-    for (int kk = 0; kk < GF_BK; kk += 2) {
-      float a[2], b[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = As[kk + lk][wm + i * 32 + li];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = Ws[kk + lk][wn + j * 32 + li];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
-    }
-    __syncthreads();
+    for (int i = 0; i < 2; ++i) total[i] += acc[i];
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) total[i][j] += acc[i][j];
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3), n = n0 + wn + j * 32 + li;
-        if (m < M && n < N) C[(size_t)m * ldc + n] = from_float<TC>(total[i][j][v]);
-      }
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + wm + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3), n = n0 + wn + li;
+      if (m < M && n < N) C[(size_t)m * ldc + n] = from_float<TC>(total[i][v]);
+    }
 }
 
 template <typename TA, typename TW, typename TC>
 static int launch_tiled(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldc,
                         hipStream_t stream) {
   if (M >= 32 && N >= 32) {
-    dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM), block(256);
+    dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM), block(512);
     if (grid.y > 65535) return blm_fail("gemm_tiled: M=%d too large", M);
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)A, (const TW*)W,
                        (TC*)C, M, N, K, lda, ldc);
