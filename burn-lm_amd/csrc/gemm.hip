@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(512, 4)   // 128 registers: two blocks per com
     const int c1 = c0 + GF_CHUNK < K ? c0 + GF_CHUNK : K;
     for (int k0 = c0; k0 < c1; k0 += GF_BK) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {   // 128 rows x 16 k per operand, 4 elements per thread, k fastest
+      for (int e = 0; e < GF_BK / 4; ++e) {   // 128 rows x GF_BK k per operand, k fastest
         const int idx = tid + e * 512;
         const int r = idx / GF_BK, kk = idx % GF_BK;
         const int gk = k0 + kk;
