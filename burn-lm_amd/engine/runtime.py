@@ -222,10 +222,18 @@ class Runtime:
                 return ops.gemv_mfma(x, packed, out, K)
         if out is None:
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+        if (out_dtype == torch.float32 and M > 32 and aligned and x.dtype == w.dtype == torch.bfloat16
+                and x.stride(1) == 1 and w.is_contiguous() and out.stride(1) == 1 and N * K * 2 < 1 << 32):
+            # float32 results (logits) for more rows than one skinny product takes at this width (more than 64,
+            # or more than 32 where K is above 2048): the matrix-core kernel with a float output, which reads
+            # the weights once.  Measured per call with a vocabulary of 128,256 against the skinny product in
+            # chunks of rows (us): width 2048, 65 / 128 / 256 rows: 141 / 156 / 189 against 202 / 230 / 453;
+            # width 3072, 33-64 rows: 154-169 against 268-298; width 4096: 233-238 against 329-350, 65-128 rows
+            # 240-252 against 509-687; the library's product with a float output: equal to 5 % behind.
+            return ops.gemm_mfma(x, w, out, tile=(128, 128, 4) if M <= 128 else (256, 128))
         if packed is not None and aligned and out_dtype == torch.float32:
-            # float32 results (logits) for more rows than one skinny product takes at this width: the
-            # most rows it does take at a time (64, 32 or 16); the weights stream once per chunk, which
-            # still beats the plain tiled kernel by far
+            # 17 to 32 rows at a K above 4096: the most rows the skinny product does take at a time (16); the
+            # weights stream once per chunk, which still beats the plain tiled kernel by far
             chunk = next((c for c in (64, 32, 16) if ops.gemv_mfma_supported(c, N, K)), 0)
             if chunk:
                 for r in range(0, M, chunk):
