@@ -340,6 +340,26 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
             assert rel_err(got[i], want[i][cut[i] + k]) <= TOL["bfloat16"], f"request {i}, decode step {k}"
 
 
+@pytest.mark.parametrize("M,K,tile", [(33, 3072, (128, 128, 4)), (64, 2048, None), (65, 2048, (128, 128, 4)), (128, 520, (128, 128, 4)),
+                                      (129, 2048, (256, 128)), (300, 4096, (256, 128)), (32, 3072, None)])
+def test_float32_logits_of_many_rows_read_the_weights_once(monkeypatch, M, K, tile):
+    """More rows than one skinny product takes at the width (more than 64, or more than 32 above K = 2048): the
+    matrix-core kernel with a float32 output instead of the skinny product over chunks of rows."""
+    from burn_lm_amd.csrc import ops
+    from burn_lm_amd.engine.runtime import Runtime
+    rt = Runtime(torch.bfloat16, "cuda:0")
+    g = torch.Generator().manual_seed(M + K)
+    N = 1000
+    x = torch.randn(M, K, generator=g).bfloat16().cuda()
+    raw = (torch.randn(N, K, generator=g) * 0.05).bfloat16().cuda()
+    tiles, real = [], ops.gemm_mfma
+    monkeypatch.setattr(ops, "gemm_mfma", lambda *a, **k: (tiles.append(k.get("tile")), real(*a, **k))[1])
+    out = rt.linear(x, rt.weight(raw), out_dtype=torch.float32)
+    assert tiles == ([tile] if tile else []) and out.dtype == torch.float32
+    want = x.double() @ raw.double().T
+    assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-6
+
+
 def test_short_prompts_take_the_fused_gate_up_product(tmp_path, monkeypatch):
     """Prompts of 65 rows and more whose gate/up tiles all run at once go through the matrix-core
     kernel with the gating in its epilogue (both of its deep-ring tiles), longer ones through the
