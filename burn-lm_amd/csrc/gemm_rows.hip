@@ -352,15 +352,17 @@ extern "C" int blm_gemm_rows(const void* A, const void* W, void* C, int c_dtype,
 
 // The q/k/v projection of 17 to 256 rows with the rotation and the cache write where the partial tiles meet
 // (columns: 32 per block, or 64 with 64 rows staged and a ring of two, for shapes whose blocks of 32 columns
-// would not all run at once).  W: W_qkv [(nh + 2 nkv) * hd, K] with rotary partners in adjacent rows; qkv_out:
+// would not all run at once; rows: 64 staged per block, or 32 with a deeper ring, which up to 32 rows is what
+// runs anyway and above makes twice the blocks).  W: W_qkv [(nh + 2 nkv) * hd, K] with rotary partners in adjacent rows; qkv_out:
 // [M, ldq] bf16, of which only the first nh * hd columns (the rotated queries) are written; key plane
 // [pages, nkv, page, hd], value plane [pages, nkv, hd, page].  store = 0: keys and values are neither
 // computed nor written.
 extern "C" int blm_gemm_rows_qkv_rope(const void* A, const void* W, void* qkv_out, const int* positions, const int* token_seq,
                                       const int* block_table, int table_width, const float* cos_sin, void* kcache, void* vcache,
                                       int page_size, int M, int K, int lda, int ldw, int ldq, int nh, int nkv, int hd, int store,
-                                      int columns, hipStream_t stream) {
+                                      int columns, int rows, hipStream_t stream) {
   BLM_REQUIRE(columns == 32 || columns == 64, "gemm_rows_qkv_rope: %d columns per block: 32 or 64", columns);
+  BLM_REQUIRE(rows == 64 || (rows == 32 && columns == 32), "gemm_rows_qkv_rope: %d rows per block: 64, or 32 with 32 columns", rows);
   BLM_REQUIRE(M >= 1 && M <= GR_MAX_ROWS && K >= 8 && K % 8 == 0 && hd >= 2 && hd % 2 == 0,
               "gemm_rows_qkv_rope: M=%d K=%d head_dim=%d not supported (M <= %d, K a multiple of 8, an even head size)", M, K, hd,
               GR_MAX_ROWS);
@@ -375,6 +377,6 @@ extern "C" int blm_gemm_rows_qkv_rope(const void* A, const void* W, void* qkv_ou
   const GrRope rope{positions, token_seq, block_table, (const float2*)cos_sin, (bf16*)kcache, (bf16*)vcache,
                     table_width, page_size, nh, nkv, hd, store};
   if (columns == 64) return gr_launch<64, 64, 64, 2, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
-  if (M > 32) return gr_launch<64, 32, 64, 3, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
+  if (M > 32 && rows != 32) return gr_launch<64, 32, 64, 3, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
   return gr_launch<32, 32, 64, 5, 2, bf16>(A, W, qkv_out, M, N, K, lda, ldw, ldq, 1, stream, rope);
 }

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 _lib = None
 _lock = threading.Lock()
 
@@ -62,7 +62,7 @@ _SIGNATURES = {
                           _c_int, _c_void_p],
     "blm_gemm_rows_qkv_rope": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                                _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                               _c_int, _c_int, _c_void_p],
+                               _c_int, _c_int, _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_decode_ffn_supported": [_c_int, _c_int, _c_int, _c_int],
     "blm_decode_ffn": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_float, _c_void_p,
@@ -687,10 +687,11 @@ def gemv_qkv_rope(x, packed, qkv_out, positions, token_seq, block_table, cos_sin
 
 
 def gemm_rows_qkv_rope(x, w, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache, page_size,
-                       nh, nkv, hd, write_kv=True, columns=32):
+                       nh, nkv, hd, write_kv=True, columns=32, rows=64):
     """17 to 256 rows: x [M, K] @ W_qkv^T (w [(nh + 2 nkv) * hd, K] as bound, rotary partners in adjacent
     rows), rotary encoding of q and k on the float results, q into qkv_out[:, :nh*hd], k and v into
-    their cache pages, in one kernel (the product of gemm_rows).  columns: 32 or 64 per block."""
+    their cache pages, in one kernel (the product of gemm_rows).  columns: 32 or 64 per block; rows: 64
+    staged per block, or 32 (with 32 columns), which is what runs up to 32 rows in any case."""
     _gpu(x, w, qkv_out, positions, token_seq, block_table, cos_sin, kcache, vcache)
     gemm_rows_init(x.device)
     M, K = x.shape
@@ -711,7 +712,7 @@ def gemm_rows_qkv_rope(x, w, qkv_out, positions, token_seq, block_table, cos_sin
     _call("blm_gemm_rows_qkv_rope", x.data_ptr(), w.data_ptr(), qkv_out.data_ptr(), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], cos_sin.data_ptr(), kcache.data_ptr(),
           vcache.data_ptr(), page_size, M, K, x.stride(0), w.stride(0), qkv_out.stride(0), nh, nkv, hd,
-          1 if write_kv else 0, columns, _stream())
+          1 if write_kv else 0, columns, rows, _stream())
     return qkv_out
 
 

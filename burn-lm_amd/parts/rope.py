@@ -102,9 +102,11 @@ class RotaryEncoding(PositionEncoding):
         # library's product and the rotation kernel: 1B shape 10 against 14-16 us at 65-128 rows, 13.3 against 21
         # at 192, 13.6 against 16 at 256; 3B 16-17 against 18-27 at 65-192, 28.5 against 33 at 256; 8B 21-24.5
         # against 28-31 at 65-128, 36 against 39 at 192, 38.5 against 46 at 256)
-        columns, mid = 32, False
+        columns, mid, rows = 32, False, 64
+        n_qkv = (heads + 2 * kv_heads) * head_dim
+        if few and M > 32 and getattr(rt, "rows_ring", False) and rt.rows_ring_blocks(64, n_qkv) * 2 <= rt.compute_units:
+            rows = 32    # 33 to 64 rows as two blocks of 32 while both sets run at once (1B shape: 7.8-8.2 against 9.3-9.8 us)
         if 64 < M <= 256 and getattr(rt, "rows_ring", False):
-            n_qkv = (heads + 2 * kv_heads) * head_dim
             if rt.rows_ring_blocks(M, n_qkv) <= rt.compute_units:
                 mid = True
             elif rt.rows_ring_blocks(M, n_qkv, 64) * 2 <= rt.compute_units * 3:
@@ -123,7 +125,7 @@ class RotaryEncoding(PositionEncoding):
             qkv = torch.empty(M, (heads + 2 * kv_heads) * head_dim, dtype=torch.bfloat16, device=x.device)
             return rt.ops.gemm_rows_qkv_rope(x, raw, qkv, step.positions, step.token_seq, view.block_table(step), self.table,
                                              view.k, view.v, view.page_size, heads, kv_heads, head_dim, write_kv=view.store,
-                                             columns=columns)
+                                             columns=columns, rows=rows)
         if (packed is not None and not getattr(w_qkv, "gated", False) and x.dtype == torch.bfloat16
                 and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing) and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0 and view.k.dtype == torch.bfloat16):

@@ -843,15 +843,15 @@ def test_gemv_qkv_rope(ops, pairing, M, K, nh, nkv, hd):
 @pytest.mark.parametrize("M,K,nh,nkv,hd", [(33, 2048, 4, 2, 64), (64, 520, 3, 1, 48), (20, 4096, 2, 1, 64), (17, 264, 30, 2, 128),
                                            (48, 2056, 2, 1, 32), (64, 3072, 3, 1, 128), (40, 4104, 2, 2, 80), (32, 72, 1, 1, 6),
                                            (65, 264, 3, 1, 48), (128, 2048, 4, 2, 64), (200, 520, 2, 1, 128), (256, 72, 1, 1, 6)])
-@pytest.mark.parametrize("columns", [32, 64])
-def test_gemm_rows_qkv_rope(ops, M, K, nh, nkv, hd, columns):
+@pytest.mark.parametrize("columns,rows", [(32, 64), (64, 64), (32, 32)])
+def test_gemm_rows_qkv_rope(ops, M, K, nh, nkv, hd, columns, rows):
     """The same for 17 to 256 rows on the product whose wavefronts stream their own stages of K: any K,
     head sizes that put two heads into a block's 32 or 64 columns or a head across several blocks, one to
-    four blocks of rows (each with its own rows' positions and sequences)."""
+    eight blocks of 64 or 32 rows (each with its own rows' positions and sequences)."""
 
     def run(x, W, out, positions, token_seq, perm, cs, kd, vd, page, write_kv):
         ops.gemm_rows_qkv_rope(x, W, out, positions, token_seq, perm, cs, kd, vd, page, nh, nkv, hd, write_kv=write_kv,
-                               columns=columns)
+                               columns=columns, rows=rows)
 
     _check_qkv_rope(run, "interleaved", M, K, nh, nkv, hd)
 
