@@ -1,8 +1,9 @@
-// Matrix product for up to 64 rows, made for 17 to 64 (decode steps of many sequences), on the matrix
-// cores: C[M <= 64, N] = A[M, K] * W[N, K]^T, bf16 operands, W as the checkpoint stores it, float accumulation,
-// bf16 or float output.
+// Matrix product for few rows, made for 17 to 64 (decode steps of many sequences), on the matrix
+// cores: C[M, N] = A[M, K] * W[N, K]^T, bf16 operands, W as the checkpoint stores it, float accumulation,
+// bf16 or float output.  Up to 256 rows it runs as one block for every 32 or 64 rows (blockIdx.z), each a
+// product of its own: for narrow products of short prompts and of decode steps of more than 64 sequences.
 //
-// A block of four wavefronts owns all rows (staged as 32 or 64) and BN columns of C (and one group of
+// A block of four wavefronts owns its rows (staged as 32 or 64) and BN columns of C (and one group of
 // K).  Its wavefronts take the block's stages of 64 along K in turn (wavefront w: stages w, w + 4, ...), a stage being the
 // rows' and the columns' slices of 64, loaded 16 bytes per lane straight from global memory into a ring
 // of R slots of shared memory that belongs to the wavefront alone.  A wavefront waits only for its own
