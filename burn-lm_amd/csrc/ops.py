@@ -626,8 +626,8 @@ def gemm_rows_init(device=None):
 
 
 def gemm_rows(a, w, out, gated=False, columns=64):
-    """bfloat16 product for up to 64 rows whose loads never stop for a barrier: out = a[M, K] @ w[N, K]^T,
-    w as the checkpoint stores it.  out: bfloat16 or float32 [M, N], or float32 [groups, M, N] partial
+    """bfloat16 product for few rows (made for 17 to 64; up to 256 as one block for every 64 rows) whose loads
+    never stop for a barrier: out = a[M, K] @ w[N, K]^T, w as the checkpoint stores it.  out: bfloat16 or float32 [M, N], or float32 [groups, M, N] partial
     products over that many groups of K (the reader sums them).  gated=True: w is [gate rows; up rows]
     ([2I, K]) and out is [M, I] = silu(a gate^T) * (a up^T).  columns: 64 or (without gating) 32 columns
     of out (of gate and up together when gated) per block."""
