@@ -20,7 +20,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libburnlm_hip.so"
 ARCH = "gfx950"
 # packed-fp32 instructions are kept off for every device pass
-HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
+# (-Wno-inline-asm: the direct-load statements of common.h name m0 as clobbered, which the compiler
+# answers with a warning per use because it keeps that register for itself)
+HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wno-inline-asm",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # The matrix-core attention takes maxima of matrix-core results; told that they are no NaNs (masked
 # scores are replaced by -infinity before any maximum, stale values are zeroed as integers) the
@@ -231,15 +233,20 @@ def build(verbose=True, jobs=None, with_ref=False):
             s = pending.pop(0)
             o = os.path.join(bdir, s[:-4] + ".o")
             objs.append(o)
+            # the compiler writes into a file, not a pipe: nobody reads while it runs, and a pipe that
+            # fills up (a warning per template instance is enough) would stop it for good
+            said = open(os.path.join(bdir, s[:-4] + ".log"), "w+")
             p = subprocess.Popen([hipcc, *HIPCC_FLAGS, *PER_FILE_FLAGS.get(s, []), "-I", HERE, "-c", os.path.join(HERE, s), "-o", o],
-                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-            running[s] = p
-        for s, p in list(running.items()):
+                                 stdout=said, stderr=subprocess.STDOUT, stdin=subprocess.DEVNULL)
+            running[s] = (p, said)
+        for s, (p, said) in list(running.items()):
             if p.poll() is not None:
-                out = p.stdout.read()
+                said.seek(0)
+                out = said.read()
+                said.close()
                 del running[s]
                 if p.returncode != 0:
-                    for q in running.values():
+                    for q, _ in running.values():
                         q.kill()
                     raise RuntimeError(f"hipcc failed on {s}:\n{out}")
                 log(f"  {s} done ({time.time() - t0:.0f} s)")

@@ -90,16 +90,16 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 // full address per lane.  Written as assembly: when the compiler knows of such a load it waits for
 // every outstanding one (vmcnt(0)) in front of the next read of shared memory, whatever address that
 // read has, so a ring of several stages would never have more than one in flight; with these, the
-// waits are the kernel's own (loads complete in order).  m0 holds the address in shared memory; the
-// kernels that use this have no other instruction that reads m0.
+// waits are the kernel's own (loads complete in order).  m0 holds the address in shared memory and is
+// declared as clobbered, so the compiler keeps nothing of its own there across the statement.
 typedef __attribute__((address_space(3))) void* blm_lds_ptr;
 __device__ __forceinline__ void blm_dma16(const char* base, uint32_t lane_offset, const void* lds) {
   const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(blm_lds_ptr)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void blm_dma16_lanes(const char* address, const void* lds) {
   const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(blm_lds_ptr)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(address) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(address) : "memory", "m0");
 }
 
 // Error reporting shared by the host entry points (defined in api.hip).

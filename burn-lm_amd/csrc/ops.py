@@ -64,10 +64,6 @@ _SIGNATURES = {
                                _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                _c_int, _c_int, _c_int, _c_void_p],
     "blm_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
-    "blm_decode_ffn_supported": [_c_int, _c_int, _c_int, _c_int],
-    "blm_decode_ffn": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_float, _c_void_p,
-                       _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
-                       _c_int, _c_void_p],
     "blm_probe_read": [_c_void_p, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p],
     "blm_probe_mfma": [_c_int, _c_int, _c_int, _c_void_p, _c_void_p],
     "blm_static_scratch_init": [],
@@ -174,81 +170,6 @@ def arrival_counters(device):
             raise KernelError("arrival_counters: the first call for a device must come before any graph capture")
         buf = _arrivals[key] = torch.zeros(ARRIVAL_COUNTERS, dtype=torch.int32, device=torch.device("cuda", key))
     return buf
-
-
-_grid_sync = {}
-SPIN_LIMIT = 2_000_000     # polls of a grid-wide wait before a block gives up (about a second)
-
-
-def grid_sync(device):
-    """Per device: the two zeroed counters at which the blocks of a resident grid meet (they return
-    to zero by themselves) and the word in pinned host memory that a kernel sets if a wait gave up.
-    First call outside any graph capture (Runtime() makes it)."""
-    device = torch.device(device)
-    key = device.index if device.index is not None else torch.cuda.current_device()
-    pair = _grid_sync.get(key)
-    if pair is None:
-        if torch.cuda.is_current_stream_capturing():
-            raise KernelError("grid_sync: the first call for a device must come before any graph capture")
-        pair = _grid_sync[key] = (torch.zeros(2, dtype=torch.int32, device=torch.device("cuda", key)),
-                                  torch.zeros(1, dtype=torch.int32).pin_memory())
-    return pair
-
-
-def check_fault(device):
-    """Raises if a kernel of this device ever gave up a bounded wait (its results were wrong from
-    then on).  Cheap: reads a word of host memory."""
-    pair = _grid_sync.get(torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device())
-    if pair is not None and int(pair[1][0]) != 0:
-        raise KernelError("a resident-grid kernel gave up waiting for the other blocks of its grid (were all of them "
-                          "on the chip?); results since then are not valid")
-
-
-def decode_ffn_supported(M, D, inner, blocks):
-    return bool(library().blm_decode_ffn_supported(int(M), int(D), int(inner), int(blocks)))
-
-
-def decode_ffn(h, delta, gamma, eps, w_gate_up_packed, w_down_packed, inner, blocks, spin_limit=None):
-    """The feed-forward half of a decode layer in one kernel: h += delta (bfloat16 [M, D], float32
-    [planes, M, D], or None); x = rmsnorm(h) * gamma; silu(x gate^T) * (x up^T) times down^T, returned
-    as float32 partial planes [groups, M, D] for the next norm to sum.  The packed weights are
-    pack_weight(gate/up, gated=True) and pack_weight(down); blocks: the grid, at most the device's
-    compute units (every block waits for all the others)."""
-    _gpu(h, delta, gamma, w_gate_up_packed, w_down_packed)
-    M, D = h.shape
-    if h.dtype != torch.float32 or not h.is_contiguous():
-        raise KernelError("decode_ffn: the residual stream must be contiguous float32")
-    if not decode_ffn_supported(M, D, inner, blocks):
-        raise KernelError(f"decode_ffn: {M} rows of width {D} with inner size {inner} on {blocks} blocks are not supported")
-    if w_gate_up_packed.dtype != torch.bfloat16 or w_down_packed.dtype != torch.bfloat16:
-        raise KernelError("decode_ffn: the packed weights must be bfloat16")
-    if w_gate_up_packed.numel() != (2 * inner // 16) * ((D + 31) // 32) * 512 or \
-            w_down_packed.numel() != ((D + 15) // 16) * ((inner + 31) // 32) * 512:
-        raise KernelError("decode_ffn: the packed weights do not have the sizes of [2 inner, D] and [D, inner] matrices")
-    _contig("gamma", gamma)
-    if gamma.numel() != D:
-        raise KernelError("decode_ffn: gamma must have one weight per column")
-    planes, stride, dcode = 1, 0, 0
-    if delta is not None:
-        _contig("delta", delta)
-        if delta.dim() == 3:
-            if delta.shape[1:] != h.shape or delta.dtype != torch.float32:
-                raise KernelError("decode_ffn: partial deltas must be float32 [planes, M, D]")
-            planes, stride = delta.shape[0], M * D
-        elif delta.shape != h.shape or delta.dtype != torch.bfloat16:
-            raise KernelError("decode_ffn: a whole delta must be bfloat16 [M, D]")
-        dcode = _code(delta)
-    tiles = (D + 15) // 16
-    groups = 1
-    while tiles * groups * 2 <= blocks and ((inner + 31) // 32) // (groups * 2) >= 8:
-        groups *= 2
-    counters, fault = grid_sync(h.device)
-    act = torch.empty(M, inner, dtype=torch.bfloat16, device=h.device)
-    out = torch.empty(groups, M, D, dtype=torch.float32, device=h.device)
-    _call("blm_decode_ffn", h.data_ptr(), _ptr(delta), dcode, planes, stride, gamma.data_ptr(), _code(gamma), float(eps),
-          w_gate_up_packed.data_ptr(), w_down_packed.data_ptr(), act.data_ptr(), out.data_ptr(), M, D, int(inner),
-          groups, int(blocks), counters.data_ptr(), fault.data_ptr(), int(spin_limit or SPIN_LIMIT), _stream())
-    return out
 
 
 def _check_planes(who, kcache, vcache, nkv, page_size, hd):

@@ -73,7 +73,6 @@ class Engine:
         return packed
 
     def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> Optional[torch.Tensor]:
-        self.rt.check_fault()
         packed = self._pack(entries)
         self.cache.reserve_step(packed)  # raises before any change
         key = self.graphs.key_for(packed) if self.graphs is not None else None

@@ -92,7 +92,7 @@ def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_s
     dtype = parse_dtype(dtype)
     arch = registry.architecture_of(config)
     cfg = arch.read_config(config)
-    rt = Runtime(dtype=dtype, device=device, page_size=page_size)
+    rt = Runtime(dtype=dtype, device=device)
     made = dict(random_tensors(arch, cfg, seed, std=std, norm_jitter=norm_jitter, dtype=stored_dtype, device=rt.device))
     plan = arch.plan(cfg, set(made))
     model = Model(plan)

@@ -64,7 +64,7 @@ class LinearWeight:
 
 
 class Runtime:
-    def __init__(self, dtype=torch.bfloat16, device="cuda:0", page_size=64):
+    def __init__(self, dtype=torch.bfloat16, device="cuda:0"):
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"activation dtype must be bfloat16 or float32, got {dtype}")
         self.dtype = dtype
@@ -73,13 +73,11 @@ class Runtime:
             raise RuntimeError("burn-lm_amd runs on the GPU only (device 'cuda:N'); there is no CPU path")
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible to this process; burn-lm_amd has no CPU path")
-        self.page_size = page_size
         self.ops = ops
         ops.library()  # fail now, loudly, if the kernel library cannot be had
         ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
         ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
         ops.static_scratch_init(self.device)   # likewise: the address of the library's own scratch array
-        ops.grid_sync(self.device)             # likewise: the counters and the fault word of resident-grid kernels
         ops.attn_paged_init(self.device)       # likewise: the shared memory of the generic attention's value tiles
         ops.gemm_rows_init(self.device)        # likewise: the rings of stages of the product for 17 to 64 rows
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
@@ -92,15 +90,8 @@ class Runtime:
         # from 33 rows on those are 1-2 % ahead at some shapes and as much behind at others)
         self.skinny_gated_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_GATED_ROWS", MFMA_SKINNY_MAX_ROWS))
         self.skinny_planes_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_PLANES_ROWS", MFMA_SKINNY_MAX_ROWS))
-        # "1": the feed-forward half of a decode layer as one resident-grid kernel (ops.decode_ffn) instead of
-        # three kernels.  Off unless asked for: measured 36-53 us against 24-29 us for the three kernels (a
-        # hand-over between blocks through device-wide counters costs more than a kernel boundary here).
-        self.resident_decode = os.environ.get("BURN_LM_AMD_RESIDENT_DECODE") == "1"
         # "0": 17 to 64 rows stay on the packed skinny kernels (for measurements)
         self.rows_ring = os.environ.get("BURN_LM_AMD_ROWS_RING") != "0"
-
-    def check_fault(self):
-        ops.check_fault(self.device)
 
     def empty(self, *shape, dtype=None):
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)

@@ -38,20 +38,3 @@ class SwiGLU(FeedForward):
     def forward(self, x, step):
         rt = self.rt
         return rt.linear(rt.gated_linear(x, self.w_gate_up), self.w_down, partials=True)
-
-    def forward_after_norm(self, h, delta, norm, step):
-        """A decode step of up to 16 rows in bfloat16 behind a plain RMS norm: norm, gate/up product
-        with the gating, and down product as phases of one kernel whose blocks stay resident."""
-        rt = self.rt
-        rms = norm.rms_constants()
-        M, D = h.shape
-        if (rms is not None and rt.resident_decode and rt.dtype == torch.bfloat16 and M <= 16
-                and self.w_gate_up.packed is not None and self.w_gate_up.gated and self.w_down.packed is not None
-                and (delta is None or delta.is_contiguous())
-                and (delta is None or (delta.dim() == 3 and delta.dtype == torch.float32) or
-                     (delta.dim() == 2 and delta.dtype == torch.bfloat16))
-                and rt.ops.decode_ffn_supported(M, D, self.inner, rt.compute_units)):
-            gamma, eps = rms
-            return rt.ops.decode_ffn(h, delta, gamma, eps, self.w_gate_up.packed, self.w_down.packed, self.inner,
-                                     rt.compute_units)
-        return super().forward_after_norm(h, delta, norm, step)

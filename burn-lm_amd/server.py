@@ -17,7 +17,7 @@ from dataclasses import asdict, dataclass, fields
 from typing import Callable, List, Optional, Sequence
 
 from .engine.generate import ContextLengthExceeded, generate
-from .cli.tokenizer import StreamingDecoder
+from .text.tokenizer import StreamingDecoder
 from .engine.stats import Stats
 from .sampling.sampler import Sampler
 
@@ -147,7 +147,7 @@ class InferenceServer:
 
     def _tokenizer(self):
         if self.tokenizer is None:
-            from .cli.tokenizer import for_folder
+            from .text.tokenizer import for_folder
             self.tokenizer = for_folder(self.folder, self.engine.vocab_size,
                                         self.engine.model.architecture.special_tokens)
         return self.tokenizer

@@ -1,4 +1,4 @@
-"""Text <-> token ids for the command line.
+"""Text <-> token ids for the server layer and the command line.
 
 ``ByteTokenizer``: a token is a byte value, as the reference's test tokenizer
 (crates/burn-lm-llama/src/tokenizer/byte.rs:3-49: bos 0, eos 1, stop ids [2]); it needs a

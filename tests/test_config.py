@@ -117,12 +117,21 @@ def test_presets_are_valid_configurations():
     assert (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads,
             c.intermediate_size, c.vocab_size) == (2048, 16, 32, 8, 8192, 128256)
     assert c.rope_scaling.factor == 32.0 and c.rope_theta == 500000.0
+    # the two tiny shapes of the tests can be named from the command line as well: same sizes and options
+    from helpers import TINY_A, TINY_B
+    for name, tiny in (("tiny-a", TINY_A), ("tiny-b", TINY_B)):
+        p = preset(name)
+        for key, value in tiny.items():
+            if key != "max_position_embeddings":      # the tests give themselves a longer context
+                assert p[key] == value, (name, key)
+    assert preset("tiny-a")["max_position_embeddings"] == 128 and preset("tiny-b")["max_position_embeddings"] == 96
+    assert LlamaConfig.from_dict(preset("tiny-b")).head_dim == 24
 
 
 def test_tokenizers_for_the_command_line(tmp_path):
     """Bytes by default; a tokenizer.json in the model folder is used when there is one, with the
     stop ids of the special tokens it defines (tiktoken.rs:12-15, 126-132)."""
-    from burn_lm_amd.cli.tokenizer import ByteTokenizer, FileTokenizer, for_folder
+    from burn_lm_amd.text.tokenizer import ByteTokenizer, FileTokenizer, for_folder
     t = for_folder(str(tmp_path), 256)
     assert isinstance(t, ByteTokenizer) and t.decode(t.encode("héllo")) == "héllo" and t.stop_ids() == [2]
     assert t.encode("a", bos=True, eos=True) == [0, 97, 1]
@@ -196,7 +205,7 @@ def test_text_comes_out_piece_by_piece_as_the_whole_would():
     """The streaming decoder against two tokenizers whose tokens cannot be decoded one by one: bytes
     (a character of several bytes spans tokens) and a word tokenizer that puts a space between the
     words of one call and none in front of the first (crates/burn-lm-llama/src/generation/streaming.rs:10-57)."""
-    from burn_lm_amd.cli.tokenizer import ByteTokenizer, StreamingDecoder
+    from burn_lm_amd.text.tokenizer import ByteTokenizer, StreamingDecoder
 
     text = "héllo wörld — ça va? 日本語"
     ids = ByteTokenizer().encode(text)

@@ -946,36 +946,3 @@ def test_random_weights_are_the_same_bytes_on_the_gpu_and_in_a_folder(tmp_path):
         b = random_engine(cfg, seed=21, dtype=dtype, max_tokens=1024, std=0.08, norm_jitter=0.1)
         sa, sb = a.open(), b.open()
         assert torch.equal(a.step([(sa, toks, list(range(40)))]), b.step([(sb, toks, list(range(40)))]))
-
-
-def test_the_resident_feed_forward_kernel_in_the_engine(folders, monkeypatch):
-    """With BURN_LM_AMD_RESIDENT_DECODE=1 the feed-forward half of a decode layer (norm, gate/up with the
-    gating, down) runs as one kernel whose blocks wait for each other (ops.decode_ffn), eagerly and from
-    recorded graphs: the logits stay the plain implementation's, the kernel is really the one that ran,
-    and no wait ever gave up."""
-    from burn_lm_amd.csrc import ops
-    monkeypatch.setenv("BURN_LM_AMD_RESIDENT_DECODE", "1")
-    calls = [0]
-    real = ops.decode_ffn
-
-    def counted(*a, **kw):
-        calls[0] += 1
-        return real(*a, **kw)
-
-    monkeypatch.setattr(ops, "decode_ffn", counted)
-    cfg, seed = TINIES["C"]
-    plain = P.load_model_folder(folders["C"])
-    eng = load(folders["C"], "bfloat16", max_tokens=4096, max_seqs=8)
-    assert eng.rt.resident_decode
-    reqs = [random_tokens(1200 + i, cfg["vocab_size"], n) for i, n in enumerate([90, 41, 70, 33, 120])]
-    want = [P.transformer_forward([r], plain)[0] for r in reqs]
-    slots = [eng.open() for _ in reqs]
-    cut = [len(r) - 30 for r in reqs]
-    eng.step([(s, r[:c], []) for s, r, c in zip(slots, reqs, cut)])
-    for k in range(30):
-        got = eng.step([(s, [r[c + k]], [0]) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
-        for i in range(5):
-            assert rel_err(got[i], want[i][cut[i] + k]) <= TOL["bfloat16"], f"request {i}, decode step {k}"
-    torch.cuda.synchronize()
-    eng.rt.check_fault()
-    assert calls[0] >= 2 * cfg["num_hidden_layers"] and eng.graphs.replays >= 25

@@ -901,57 +901,3 @@ def _check_qkv_rope(run, pairing, M, K, nh, nkv, hd):
     out2 = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
     run(dev(x), dev(W), out2, dev(positions), dev(token_seq), dev(perm), dev(cs), kd2, dev(v), page, False)
     assert torch.equal(out2.cpu(), out.cpu()) and bool((kd2.cpu() == 99).all())
-
-
-@pytest.mark.parametrize("M,D,I,delta,blocks", [(1, 2048, 8192, "planes4", 256), (8, 2048, 8192, "bf16", 256), (16, 264, 176, "none", 256),
-                                                (5, 3072, 1024, "planes2", 256), (3, 4096, 2064, "planes3", 256), (7, 64, 176, "bf16", 5),
-                                                (9, 520, 48, "planes1", 31), (16, 2048, 8192, "planes4", 200)])
-def test_decode_ffn(ops, M, D, I, delta, blocks):
-    """The feed-forward half of a decode layer as one resident-grid kernel against its formula:
-    h + delta, the RMS norm rounded to bfloat16, the gated product rounded to bfloat16, the down
-    product as planes whose sum is compared; widths with and without whole k-steps, every form of the
-    pending delta, grids that give a block several tiles and items or none; twice in a row, so that
-    the counters must have come back to zero."""
-    g = torch.Generator().manual_seed(23)
-    assert ops.decode_ffn_supported(M, D, I, blocks)
-    h = torch.randn(M, D, generator=g)
-    gamma = (1 + 0.2 * torch.randn(D, generator=g)).bfloat16()
-    wgu = (torch.randn(2 * I, D, generator=g) * (1.5 / D ** 0.5)).bfloat16()
-    wd = (torch.randn(D, I, generator=g) * (1.0 / I ** 0.5)).bfloat16()
-    if delta == "none":
-        dl = None
-    elif delta == "bf16":
-        dl = (torch.randn(M, D, generator=g) * 0.3).bfloat16()
-    else:
-        dl = torch.randn(int(delta[6:]), M, D, generator=g) * 0.2
-    v = h.double() + (0 if dl is None else dl.double() if dl.dim() == 2 else dl.double().sum(0))
-    x = (v / torch.sqrt((v * v).mean(-1, keepdim=True) + 1e-5) * gamma.double()).bfloat16().double()
-    gate, up = x @ wgu[:I].double().T, x @ wgu[I:].double().T
-    act = (torch.nn.functional.silu(gate) * up).bfloat16().double()
-    want = act @ wd.double().T
-    pgu, pd = ops.pack_weight(dev(wgu), gated=True), ops.pack_weight(dev(wd))
-    for turn in range(2):
-        hd_ = dev(h.clone())
-        out = ops.decode_ffn(hd_, None if dl is None else dev(dl), dev(gamma), 1e-5, pgu, pd, I, blocks, spin_limit=200000)
-        torch.cuda.synchronize()
-        ops.check_fault("cuda")
-        assert out.dim() == 3 and out.shape[1:] == (M, D) and out.dtype == torch.float32
-        close(hd_, v, 1e-6)
-        close(out.double().sum(0), want, 8e-3)
-    counters, fault = ops.grid_sync("cuda")
-    assert counters.tolist() == [0, 0] and int(fault[0]) == 0
-
-
-def test_decode_ffn_refuses_what_it_cannot_do(ops):
-    from burn_lm_amd.csrc.ops import KernelError
-    assert not ops.decode_ffn_supported(17, 2048, 8192, 256)       # more rows than one matrix-core tile
-    assert not ops.decode_ffn_supported(8, 4104, 8192, 256)        # wider than the rows that fit shared memory
-    assert not ops.decode_ffn_supported(8, 2048, 8200, 256)        # inner size no multiple of 16
-    h = torch.zeros(8, 64, device="cuda")
-    gamma = torch.ones(64, dtype=torch.bfloat16, device="cuda")
-    pgu = ops.pack_weight(torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda"), gated=True)
-    pd = ops.pack_weight(torch.zeros(64, 16, dtype=torch.bfloat16, device="cuda"))
-    with pytest.raises(KernelError, match="compute units"):        # a grid that could not be resident at once
-        ops.decode_ffn(h, None, gamma, 1e-5, pgu, pd, 16, 100000)
-    with pytest.raises(KernelError, match="sizes"):
-        ops.decode_ffn(h, None, gamma, 1e-5, pgu[:-512], pd, 16, 64)

@@ -17,7 +17,7 @@ TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
 def rt(request):
     from burn_lm_amd.engine.runtime import Runtime
     import burn_lm_amd  # noqa: F401
-    return Runtime(dtype=request.param, device="cuda:0", page_size=16)
+    return Runtime(dtype=request.param, device="cuda:0")
 
 
 def rel(got, want):
