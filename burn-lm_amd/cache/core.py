@@ -8,7 +8,7 @@ from typing import List, Sequence
 
 from ..csrc import build as _build
 
-HOST_ABI = 3
+HOST_ABI = 4
 OK, E_FULL, E_OVERFLOW, E_USAGE = 0, 1, 2, 3
 
 _lib = None
@@ -35,6 +35,7 @@ _SIGNATURES = {
     "blm_step_check": ([_ptr, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _int], _int),
     "blm_step_key": ([_int, _ptr, _ints, _ptr, _ptr, _int, _ints, _int, _ints, _int, _int, _int, _ints], None),
     "blm_plan_batches": ([_int, _ints, _int, _int, _int, _int, _int, _int, _ints], _int),
+    "blm_plan_prompt_steps": ([_int, _ints, _int, _int, _ints, _ints, _ints, _ints], _int),
     "blm_gen_new": ([_int, _ints, _int, _int, _int, _ints], _ptr), "blm_gen_free": ([_ptr], None),
     "blm_gen_start": ([_ptr, _int, _ints], _int), "blm_gen_ahead_rows": ([_ptr, _ints], _int),
     "blm_gen_launched": ([_ptr, _int, _ints], _int), "blm_gen_take": ([_ptr, _ints, _ints], _int),

@@ -10,7 +10,7 @@
 extern "C" {
 #endif
 
-#define BLM_HOST_ABI 3
+#define BLM_HOST_ABI 4
 
 #define BLM_OK 0
 #define BLM_E_FULL 1      // no free slot, or not enough free pages

@@ -12,6 +12,10 @@ extern "C" int blm_plan_batches(int n, const int* prompt_lens, int sample_len, i
   for (int i = 0; i < n; ++i) {
     const long long reach = std::min<long long>((long long)prompt_lens[i] + sample_len, max_context);
     const long long need = (reach + page_size - 1) / page_size;
+    if (need > n_pages) {       // it would not fit if it had the cache to itself: the caller answers it with an error
+      batch_of[i] = -1;
+      continue;
+    }
     if (in_batch > 0 && (in_batch >= most || used + need > n_pages)) {
       ++batch;
       in_batch = 0;
@@ -21,7 +25,34 @@ extern "C" int blm_plan_batches(int n, const int* prompt_lens, int sample_len, i
     ++in_batch;
     used += need;
   }
-  return n > 0 ? batch + 1 : 0;
+  return in_batch > 0 ? batch + 1 : batch;
+}
+
+extern "C" int blm_plan_prompt_steps(int n, const int* prompt_lens, int budget, int max_pieces, int* piece_step,
+                                     int* piece_seq, int* piece_from, int* piece_count) {
+  if (n < 0 || budget <= 0) return -1;
+  int pieces = 0, step = 0;
+  long long room = budget;
+  for (int i = 0; i < n; ++i) {
+    if (prompt_lens[i] <= 0) return -1;
+    int from = 0;
+    while (from < prompt_lens[i]) {
+      if (room == 0) {
+        ++step;
+        room = budget;
+      }
+      const int take = (int)std::min<long long>(room, prompt_lens[i] - from);
+      if (pieces >= max_pieces) return -1;
+      piece_step[pieces] = step;
+      piece_seq[pieces] = i;
+      piece_from[pieces] = from;
+      piece_count[pieces] = take;
+      ++pieces;
+      from += take;
+      room -= take;
+    }
+  }
+  return pieces;
 }
 
 struct BlmGen {

@@ -13,9 +13,19 @@ extern "C" {
 // ---- batches ------------------------------------------------------------------------------------
 // Cuts n requests, in order, into batches that fit: at most batch_size sequences and n_slots slots,
 // and pages enough for every sequence of a batch to reach min(prompt + sample_len, max_context).
-// batch_of[i] receives the batch number of request i; returns the number of batches.
+// batch_of[i] receives the batch number of request i, or -1 for a request that would not fit if it
+// had all n_pages to itself; returns the number of batches.
 int blm_plan_batches(int n, const int* prompt_lens, int sample_len, int batch_size, int max_context, int page_size,
                      int n_pages, int n_slots, int* batch_of);
+
+// Cuts the prompts of one batch (n sequences, prompt_lens[i] > 0 tokens each) into steps of at most
+// `budget` tokens: the sequences in order, a step filled before the next one starts, a prompt cut
+// wherever a step is full.  Piece p says that step piece_step[p] brings sequence piece_seq[p] its
+// tokens piece_from[p] .. + piece_count[p]; pieces come in the order of the steps and, within a step,
+// of the sequences.  Returns the number of pieces, or -1 for bad sizes or more than max_pieces
+// (n + total / budget + 1 always suffice).
+int blm_plan_prompt_steps(int n, const int* prompt_lens, int budget, int max_pieces, int* piece_step, int* piece_seq,
+                          int* piece_from, int* piece_count);
 
 // ---- one generation ------------------------------------------------------------------------------
 #define BLM_GEN_GOES_ON 0

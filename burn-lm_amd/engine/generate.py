@@ -13,6 +13,14 @@ The reference's loop is ``Llama::generate`` (crates/burn-lm-llama/src/generation
 is counted and returned but is not text.  Where the reference slides its window when the
 context is full (nn/transformer.rs:156-163), a sequence here ends with the reason ``length``.
 
+A batch's prompts run in one step while they are at most ``prompt_budget`` tokens together; a
+larger batch is fed in several steps of that many tokens (the step function takes a prompt in
+pieces; a sequence's last piece asks for its logits), so that the activations of a step stay
+bounded whatever the requests bring.  A request that could not run even with the whole cache to
+itself ends with ``finish_reason="error"`` and the others run, as a request whose prompt is longer
+than the context does (crates/burn-lm-llama/src/nn/transformer.rs:148-154 and
+server/llama3.rs:476-478 answer one request with an error and stay usable).
+
 The loop needs of its engine only ``open / close / step / length / max_context / cache`` and of
 its sampler only ``pick``, so its decisions are testable without a GPU.  With those alone the
 stop is seen on the host in the same step and no extra step runs.  If the engine also has
@@ -50,11 +58,16 @@ class Generation:
     error: Optional[str] = None
 
 
+# Most prompt tokens that one step runs; a batch whose prompts are more is fed in several steps.
+PROMPT_BUDGET = 16384
+
+
 def plan_batches(prompt_lens: Sequence[int], sample_len: int, batch_size: int, max_context: int,
-                 page_size: int, n_pages: int, n_slots: int) -> List[List[int]]:
+                 page_size: int, n_pages: int, n_slots: int, unfit: Optional[List[int]] = None) -> List[List[int]]:
     """Cuts the requests, in order, into batches that fit: at most batch_size sequences and slots,
     and pages enough for every sequence of the batch to reach its longest possible length (decided
-    by the native core, blm_plan_batches)."""
+    by the native core, blm_plan_batches).  A request that needs more pages than the cache has is in
+    no batch; its index is appended to ``unfit`` if that list is given."""
     n = len(prompt_lens)
     if n == 0:
         return []
@@ -63,8 +76,36 @@ def plan_batches(prompt_lens: Sequence[int], sample_len: int, batch_size: int, m
                                                  int(max_context), int(page_size), int(n_pages), int(n_slots), batch_of)
     batches = [[] for _ in range(n_batches)]
     for i in range(n):
-        batches[batch_of[i]].append(i)
+        if batch_of[i] >= 0:
+            batches[batch_of[i]].append(i)
+        elif unfit is not None:
+            unfit.append(i)
     return batches
+
+
+def plan_prompt_steps(prompt_lens: Sequence[int], budget: int) -> List[List[tuple]]:
+    """The prompts of one batch as steps of at most `budget` tokens: per step a list of (sequence,
+    first token, number of tokens), sequences in order, a prompt cut wherever a step is full (decided
+    by the native core, blm_plan_prompt_steps)."""
+    n = len(prompt_lens)
+    if budget <= 0:
+        raise ValueError("the prompt budget must be positive")
+    most = n + sum(prompt_lens) // budget + 1
+    arrays = [(_core.ctypes.c_int * most)() for _ in range(4)]
+    pieces = _core.library().blm_plan_prompt_steps(n, _core.ints(list(prompt_lens)), int(budget), most, *arrays)
+    if pieces < 0:
+        raise ValueError("prompts must hold at least one token each")
+    steps: List[List[tuple]] = []
+    for p in range(pieces):
+        if arrays[0][p] == len(steps):
+            steps.append([])
+        steps[-1].append((arrays[1][p], arrays[2][p], arrays[3][p]))
+    return steps
+
+
+def _cache_refusals():
+    from ..cache.cache import CacheFull, ContextOverflow
+    return (CacheFull, ContextOverflow)
 
 
 class _Book:
@@ -110,13 +151,37 @@ class _Book:
         return self._buf[:n], self._buf2[:n]
 
 
+def run_prompts(engine, slots: Sequence[int], prompts: Sequence[Sequence[int]], budget: int):
+    """Feeds the prompts of a batch, in steps of at most `budget` tokens.  -> (the logits after every
+    prompt's last token, in the order of the prompts; the number of steps it took)."""
+    if sum(len(p) for p in prompts) <= budget:
+        return engine.step([(s, list(p), [len(p) - 1]) for s, p in zip(slots, prompts)]), 1
+    steps = plan_prompt_steps([len(p) for p in prompts], budget)
+    rows = [None] * len(prompts)
+    for pieces in steps:
+        ends = [k for k, first, count in pieces if first + count == len(prompts[k])]
+        logits = engine.step([(slots[k], list(prompts[k][first:first + count]),
+                               [count - 1] if first + count == len(prompts[k]) else []) for k, first, count in pieces])
+        for r, k in enumerate(ends):
+            rows[k] = logits[r].clone()     # a later step may write into the buffer these logits live in
+    return _stack(rows), len(steps)
+
+
+def _stack(rows):
+    import torch
+    return torch.stack(rows)
+
+
 def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int, stop_ids: Sequence[int] = (),
              batch_size: int = 8, on_token: Optional[Callable[[int, int], None]] = None,
-             clock: Callable[[], float] = time.perf_counter):
+             clock: Callable[[], float] = time.perf_counter, prompt_budget: int = PROMPT_BUDGET):
     """-> (list of Generation in request order, Stats).  ``on_token(request, token)`` is called
-    for every generated token as soon as it is known (stop tokens included)."""
+    for every generated token as soon as it is known (stop tokens included).  ``prompt_budget``: the
+    most prompt tokens one step runs."""
     if sample_len < 0:
         raise ValueError("sample_len must be >= 0")
+    if prompt_budget <= 0:
+        raise ValueError("prompt_budget must be positive")
     stop = set(int(s) for s in stop_ids)
     results = [Generation(i, len(p)) for i, p in enumerate(prompts)]
     stats = Stats()
@@ -133,13 +198,21 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
         else:
             runnable.append(i)
     cache = engine.cache
+    unfit: List[int] = []
     batches = plan_batches([len(prompts[i]) for i in runnable], sample_len, batch_size, engine.max_context,
-                           cache.page_size, cache.n_pages, cache.max_seqs)
+                           cache.page_size, cache.n_pages, cache.max_seqs, unfit)
+    for j in unfit:
+        i = runnable[j]
+        reach = min(len(prompts[i]) + sample_len, engine.max_context)
+        results[i].finish_reason = "error"
+        results[i].error = (f"the request may grow to {reach} tokens, which takes {-(-reach // cache.page_size)} pages of the "
+                            f"cache; it has {cache.n_pages}")
     ahead = hasattr(engine, "step_ahead") and hasattr(sampler, "pick_device")
     book = _Book([len(p) for p in prompts], sample_len, engine.max_context, stop)
     reason_names = {_Book.STOP: "stop", _Book.LENGTH: "length"}
-    for batch in batches:
-        ids = [runnable[j] for j in batch]
+    queue = [[runnable[j] for j in batch] for batch in batches]
+    while queue:
+        ids = queue.pop(0)
         slot_of, open_slots = {}, set()
 
         def close(slot):
@@ -152,11 +225,23 @@ def generate(engine, prompts: Sequence[Sequence[int]], sampler, sample_len: int,
                 open_slots.add(slot)
                 slot_of[i] = slot
             t0 = clock()
-            logits = engine.step([(slot_of[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in ids])
+            try:
+                logits, n_steps = run_prompts(engine, [slot_of[i] for i in ids], [prompts[i] for i in ids], prompt_budget)
+            except _cache_refusals() as e:
+                # The cache could not take the prompts after all (the planner counts the pages of one group of
+                # layers; a cache may have several).  Nothing of the refused step has changed anything: the slots
+                # go back, a batch of several is tried one request at a time, a single request ends with the error.
+                for slot in list(open_slots):
+                    close(slot)
+                if len(ids) > 1:
+                    queue[0:0] = [[i] for i in ids]
+                else:
+                    results[ids[0]].finish_reason, results[ids[0]].error = "error", str(e)
+                continue
             picked = sampler.pick(logits, ids, [0] * len(ids))
             stats.prompt_tokens += sum(len(prompts[i]) for i in ids)
             stats.prompt_seconds += clock() - t0
-            stats.steps += 1
+            stats.steps += n_steps
             t0 = clock()
             from_prompt = True
             book.start(ids)

@@ -35,6 +35,13 @@ from ..csrc import ops
 
 SKINNY_MAX_ROWS = 8
 MFMA_SKINNY_MAX_ROWS = 64
+# The longest K one group of the row-ring product walks before the sum is better cut into partial planes,
+# and up to which that product beats the library's at 65 to 256 rows (a block streams its stages of K one
+# after another, so its time grows with K while the library's tiles get longer runs): measured at
+# widths of 2048, 3072 and 4096.
+RING_GROUP_K = 2048
+# The shortest K a group keeps when a short K is cut for more blocks.
+RING_MIN_GROUP_K = 512
 # Rows for which the fused gate/up product is used when it is switched on (below, the library is
 # ahead by far; above, its better rate on long runs of tiles has made up for the extra pass).
 FUSED_GATE_UP_ROWS = (192, 4096)
@@ -42,17 +49,34 @@ FUSED_GATE_UP_ROWS = (192, 4096)
 
 def rows_plan(N, K, compute_units):
     """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial
-    planes (ops.gemm_rows).  A group spans about 2048 of K (measured at the 1B, 3B and 8B layer
+    planes (ops.gemm_rows).  A group spans about RING_GROUP_K of K (measured at the 1B, 3B and 8B layer
     shapes: shorter groups write more planes than they gain, longer ones leave compute units
     idle); 32 columns per block where that gives at most one block per compute unit, else 64;
-    and a short K is cut further, down to 512, until three quarters of the units have a block."""
+    and a short K is cut further, down to RING_MIN_GROUP_K, until three quarters of the units have a block."""
     groups = 1
-    while groups < 8 and K // (groups * 2) >= 2048:
+    while groups < 8 and K // (groups * 2) >= RING_GROUP_K:
         groups *= 2
     columns = 32 if -(-N // 32) * groups <= compute_units else 64
-    while groups < 8 and K // (groups * 2) >= 512 and -(-N // columns) * groups * 4 < compute_units * 3:
+    while groups < 8 and K // (groups * 2) >= RING_MIN_GROUP_K and -(-N // columns) * groups * 4 < compute_units * 3:
         groups *= 2
     return groups, columns
+
+
+class FusedProjectionPlan:
+    """Launch geometry of a projection that a part fuses with work of its own (Runtime.qkv_plan).
+    kernel: "rows" (ops.gemm_rows_qkv_rope's geometry: `rows` rows staged per block, `columns` columns
+    per block, weights as the checkpoint stores them) or "packed" (ops.gemv_qkv_rope's: the packed
+    copy of the weights, all rows in registers)."""
+    __slots__ = ("kernel", "columns", "rows")
+
+    def __init__(self, kernel, columns=0, rows=0):
+        self.kernel, self.columns, self.rows = kernel, columns, rows
+
+    def __repr__(self):
+        return f"FusedProjectionPlan({self.kernel!r}, columns={self.columns}, rows={self.rows})"
+
+    def __eq__(self, other):
+        return isinstance(other, FusedProjectionPlan) and (self.kernel, self.columns, self.rows) == (other.kernel, other.columns, other.rows)
 
 
 class LinearWeight:
@@ -107,16 +131,15 @@ class Runtime:
             return LinearWeight(w, ops.pack_weight(w, gated=gated), gated)
         return LinearWeight(w)
 
-    @staticmethod
-    def k_groups(N, K, M=1):
+    def k_groups(self, N, K, M=1):
         """Into how many groups a skinny product's K is cut so that a narrow output still gives
-        every compute unit two blocks: groups * (N / 16) tiles should reach 512 and a group should
-        span at most 2048 of K, but keeps at least 512 (measured at the 1B shape: the output
-        projection in 4 groups of 512 is 0.8 % of a step faster than in 2); and a group must fit what
-        the kernel takes for M rows."""
+        every compute unit two blocks: groups * (N / 16) tiles should reach twice the compute units and a
+        group should span at most RING_GROUP_K of K, but keeps at least RING_MIN_GROUP_K (measured at the
+        1B shape: the output projection in 4 groups of 512 is 0.8 % of a step faster than in 2); and a
+        group must fit what the kernel takes for M rows."""
         tiles = (N + 15) // 16
         g = 1
-        while g < 8 and K // (g * 2) >= 512 and (tiles * g < 512 or K // g > 2048):
+        while g < 8 and K // (g * 2) >= RING_MIN_GROUP_K and (tiles * g < 2 * self.compute_units or K // g > RING_GROUP_K):
             g *= 2
         limit = ops.gemv_mfma_group_limit(M)
         steps = (K + 31) // 32
@@ -136,7 +159,7 @@ class Runtime:
         Measured per call at the 1B shape against the library's product: 6.8-7.2 against 9.8 us at 65-128
         rows, 8.0 against 10.8 at 192, 8.9 against 11.1 at 256; at K = 3072 and 4096 (3B, 8B) equal or
         behind, hence the bound on K."""
-        if not (self.rows_ring and MFMA_SKINNY_MAX_ROWS < M <= 256 and K <= 2048):
+        if not (self.rows_ring and MFMA_SKINNY_MAX_ROWS < M <= 256 and K <= RING_GROUP_K):
             return 0
         blocks = self.rows_ring_blocks(M, N)
         if blocks > self.compute_units:
@@ -146,6 +169,34 @@ class Runtime:
     def rows_ring_blocks(self, M, N, columns=32):
         """Blocks of 64 rows and 32 or 64 columns that ops.gemm_rows and ops.gemm_rows_qkv_rope launch."""
         return -(-N // columns) * -(-M // 64)
+
+    def qkv_plan(self, M, N, K):
+        """Which fused projection geometry a position encoding should build on for M rows of width K and
+        N = all query, key and value columns, or None (project with linear(), then encode).  The encoding
+        only has to check that its own kernel exists for the answer; the thresholds live here.
+        17 to 64 rows: the row-ring geometry from 33 rows on, and from 17 where K is beyond RING_GROUP_K
+        (measured over whole decode steps against the packed kernel with two to four row tiles: 1.4 %
+        faster at batch 64 of the 1B shape and 1.3 % slower at batch 17-32, hence the rule; 2-6 % faster at
+        every batch from 17 to 64 of the 3B and 8B shapes); 33 to 64 rows as two blocks of 32 while both
+        sets run at once (1B shape: 7.8-8.2 against 9.3-9.8 us).  65 to 256 rows: a block for every 64
+        rows, 32 columns per block while those blocks all run at once, else 64 while there are at most one
+        and a half per compute unit (per layer against the library's product and the rotation kernel: 1B
+        shape 10 against 14-16 us at 65-128 rows, 13.3 against 21 at 192, 13.6 against 16 at 256; 3B 16-17
+        against 18-27 at 65-192, 28.5 against 33 at 256; 8B 21-24.5 against 28-31 at 65-128, 36 against 39
+        at 192, 38.5 against 46 at 256).  Up to 16 rows, and whenever the row-ring kernel is not to be
+        had: the packed geometry."""
+        if self.rows_ring:
+            if 16 < M <= MFMA_SKINNY_MAX_ROWS and (M > 32 or K > RING_GROUP_K):
+                halves = M > 32 and self.rows_ring_blocks(64, N) * 2 <= self.compute_units
+                return FusedProjectionPlan("rows", 32, 32 if halves else 64)
+            if MFMA_SKINNY_MAX_ROWS < M <= 256:
+                if self.rows_ring_blocks(M, N) <= self.compute_units:
+                    return FusedProjectionPlan("rows", 32, 64)
+                if self.rows_ring_blocks(M, N, 64) * 2 <= self.compute_units * 3:
+                    return FusedProjectionPlan("rows", 64, 64)
+        if M <= MFMA_SKINNY_MAX_ROWS:
+            return FusedProjectionPlan("packed")
+        return None
 
     def mid_k_groups(self, M, N, K):
         """Short prompts, narrow output, long K (the down projection): the product as partial planes
@@ -247,7 +298,7 @@ class Runtime:
         fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
         if fusable and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and (
-                M > 32 or (K > 2048 and -(-inner // 32) <= self.compute_units)):
+                M > 32 or (K > RING_GROUP_K and -(-inner // 32) <= self.compute_units)):
             # 33 to 64 rows (measured against the packed skinny kernel: 4-15 % faster at the 1B and 3B shapes, and
             # at wider ones in place of the library's product, which the packed kernel's registers leave them to);
             # from 17 rows on where K is above 2048 and the blocks come in one round (3B: 10-15 %)
@@ -286,14 +337,14 @@ class Runtime:
             # 2-6 % with a partial last round, and at width 3072 behind from 1,536 rows on).  Beyond
             # 4,096 rows the library's large tiles are ahead (whole prefill of 8,192 tokens 19.4 ms
             # against 20.7, of 16,384 tokens 47.9 against 49.0).
-            if K <= 2048 and 256 <= M <= 4096 and (-(-M // 256) * -(-inner // 128)) % self.compute_units == 0:
+            if K <= RING_GROUP_K and 256 <= M <= 4096 and (-(-M // 256) * -(-inner // 128)) % self.compute_units == 0:
                 return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
                                      gated=True, tile=(256, 256))
         if fusable and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]:
             # the largest tile that still gives every compute unit a block (a tile of n columns holds n / 2 gated pairs)
             m256 = -(-M // 256)
-            tile = ((256, 256) if m256 * -(-inner // 128) >= 256 else
-                    (256, 128) if m256 * -(-inner // 64) >= 256 else (128, 128))
+            tile = ((256, 256) if m256 * -(-inner // 128) >= self.compute_units else
+                    (256, 128) if m256 * -(-inner // 64) >= self.compute_units else (128, 128))
             return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True, tile=tile)
         gu = self.linear(x, plain)
         act = torch.empty(M, inner, dtype=gu.dtype, device=x.device)

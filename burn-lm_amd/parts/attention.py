@@ -14,18 +14,18 @@ import torch
 
 from .base import KVNeed, Mixer, TensorSpec
 
-# blocks the decode attention aims for when it cuts the key ranges into splits
-DECODE_TARGET_BLOCKS = 512
-DECODE_MIN_BLOCKS = 128
+# Blocks the decode attention aims for when it cuts the key ranges into pieces, per compute unit: two
+# (one where heads are wider than 64), at least half a block, and no cutting from one block per unit on.
+DECODE_TARGET_PER_UNIT = 2
+DECODE_MIN_PER_UNIT = 0.5
 DECODE_MAX_PIECES = 32
-DECODE_WHOLE_BLOCKS = 256
 
 
-def decode_splits(pages: int, blocks: int, head_dim: int) -> int:
+def decode_splits(pages: int, blocks: int, head_dim: int, compute_units: int = 256) -> int:
     """Into how many pieces the decode attention cuts a sequence's pages.  Every piece is a block of
     four wavefronts that take pages in turn, and the pieces' results are merged by the last block to
     finish, so a piece should hold two pages per wavefront (eight), or one (four) while that leaves
-    fewer than DECODE_MIN_BLOCKS blocks; and there is no point in more blocks than the chip takes at
+    fewer than half a block per compute unit; and there is no point in more blocks than the chip takes at
     once (pages of wide heads hold more bytes: half as many blocks reach the same memory rate).
     Measured at context 4096, head_dim 64, ms per step: batch 1: 16 pieces 0.870, 8: 0.880, 64: 1.002;
     batch 2: 8 pieces 0.909, 16: 0.928; batch 4: 8 pieces 0.961, 16: 0.988; batch 8: 8 pieces best.
@@ -34,12 +34,13 @@ def decode_splits(pages: int, blocks: int, head_dim: int) -> int:
     its arrival; the merge reads them all).  And no cutting at all once every compute unit has a block:
     an uncut sequence needs no partial result, no arrival and no merge (batch 32, context 4096: 48.5 us
     uncut, 57.8 in two pieces; context 16,384: 171 against 186)."""
-    if blocks >= DECODE_WHOLE_BLOCKS:
+    if blocks >= compute_units:
         return 1
-    target = DECODE_TARGET_BLOCKS if head_dim <= 64 else max(1, DECODE_TARGET_BLOCKS // 2)
+    target = compute_units * DECODE_TARGET_PER_UNIT if head_dim <= 64 else max(1, compute_units * DECODE_TARGET_PER_UNIT // 2)
+    least = max(1, int(compute_units * DECODE_MIN_PER_UNIT))
     n = min(max(1, pages // 8), (target + blocks - 1) // blocks, DECODE_MAX_PIECES)
-    if blocks * n < DECODE_MIN_BLOCKS:
-        n = max(n, min(max(1, pages // 4), (DECODE_MIN_BLOCKS + blocks - 1) // blocks))
+    if blocks * n < least:
+        n = max(n, min(max(1, pages // 4), (least + blocks - 1) // blocks))
     return max(1, n)
 
 
@@ -110,7 +111,7 @@ class Attention(Mixer):
             span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
             pages = (span + view.page_size - 1) // view.page_size
             blocks = qkv.shape[0] * nkv * ((nh // nkv + 15) // 16)
-            n_splits = decode_splits(pages, blocks, hd)
+            n_splits = decode_splits(pages, blocks, hd, rt.compute_units)
             rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                                view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
         elif aligned and rt.ops.attn_prefill_mfma_supported(rt.dtype, hd, view.page_size):
@@ -122,7 +123,7 @@ class Attention(Mixer):
             n_splits = 1
             if step.max_new == 1:
                 span = step.max_len_after if not self.window else min(step.max_len_after, self.window)
-                n_splits = max(1, min((span + 255) // 256, (4 * DECODE_TARGET_BLOCKS) // max(1, qkv.shape[0] * nh)))
+                n_splits = max(1, min((span + 255) // 256, (4 * DECODE_TARGET_PER_UNIT * rt.compute_units) // max(1, qkv.shape[0] * nh)))
             rt.ops.attn_paged(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                               view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
         return out

@@ -90,49 +90,33 @@ class RotaryEncoding(PositionEncoding):
                                   write_kv=store)
 
     def project_encode_store(self, x, w_qkv, step, view, heads, kv_heads, head_dim):
-        """Decode (few rows, bfloat16, packed weights): projection, rotation and cache write in one
-        kernel, the rotation applied to the float accumulators.  Otherwise the three steps apart."""
+        """Projection, rotation and cache write in one kernel (the rotation applied to the float
+        accumulators) where the runtime has a fused geometry for these sizes and this encoding's kernel
+        exists for it; otherwise the three steps apart.  Which geometry suits which sizes is the
+        runtime's answer (Runtime.qkv_plan); what is checked here is only what the rotation itself needs."""
         rt = self.rt
-        packed = getattr(w_qkv, "packed", None)
         M, K = x.shape
-        raw = getattr(w_qkv, "w", None)
-        few = 16 < M <= 64 and (M > 32 or K > 2048)
-        # 65 to 256 rows: the same kernel with a block for every 64 rows: 32 columns per block while those blocks all
-        # run at once, else 64 while there are at most one and a half per compute unit (per layer against the
-        # library's product and the rotation kernel: 1B shape 10 against 14-16 us at 65-128 rows, 13.3 against 21
-        # at 192, 13.6 against 16 at 256; 3B 16-17 against 18-27 at 65-192, 28.5 against 33 at 256; 8B 21-24.5
-        # against 28-31 at 65-128, 36 against 39 at 192, 38.5 against 46 at 256)
-        columns, mid, rows = 32, False, 64
         n_qkv = (heads + 2 * kv_heads) * head_dim
-        if few and M > 32 and getattr(rt, "rows_ring", False) and rt.rows_ring_blocks(64, n_qkv) * 2 <= rt.compute_units:
-            rows = 32    # 33 to 64 rows as two blocks of 32 while both sets run at once (1B shape: 7.8-8.2 against 9.3-9.8 us)
-        if 64 < M <= 256 and getattr(rt, "rows_ring", False):
-            if rt.rows_ring_blocks(M, n_qkv) <= rt.compute_units:
-                mid = True
-            elif rt.rows_ring_blocks(M, n_qkv, 64) * 2 <= rt.compute_units * 3:
-                columns, mid = 64, True
-        if ((few or mid) and self.pairing == PAIRING["interleaved"] and getattr(rt, "rows_ring", False)
-                and raw is not None
-                and x.dtype == raw.dtype == view.k.dtype == torch.bfloat16 and head_dim % 2 == 0 and K % 8 == 0
-                and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and raw.is_contiguous()):
-            # 33 to 64 rows, and 17 to 32 where K is above 2048: the product whose wavefronts stream their own stages
-            # of K, rotation and cache write where its partial tiles meet (measured over whole decode steps against
-            # the packed kernel with two to four row tiles, and against the library's product and the rotation kernel
-            # where that kernel's registers do not take the width: 1.4 % faster at batch 64 of the 1B shape and 1.3 %
-            # slower at batch 17-32, hence the rule; 2-6 % faster at every batch from 17 to 64 of the 3B and 8B shapes)
-            if step.max_position >= self.n_positions:
-                raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
-            qkv = torch.empty(M, (heads + 2 * kv_heads) * head_dim, dtype=torch.bfloat16, device=x.device)
+        plan = rt.qkv_plan(M, n_qkv, K) if hasattr(rt, "qkv_plan") else None
+        bf16 = x.dtype == view.k.dtype == torch.bfloat16 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+        raw, packed = getattr(w_qkv, "w", None), getattr(w_qkv, "packed", None)
+        fused = None
+        if (plan is not None and plan.kernel == "rows" and bf16 and self.pairing == PAIRING["interleaved"]
+                and raw is not None and raw.dtype == torch.bfloat16 and raw.is_contiguous()
+                and head_dim % 2 == 0 and K % 8 == 0 and x.stride(1) == 1):
+            fused = "rows"
+        elif (plan is not None and M <= 64 and bf16 and packed is not None and not getattr(w_qkv, "gated", False)
+                and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing)):
+            fused = "packed"     # also where the row-ring kernel was the plan and this encoding has none for it
+        if fused is None:
+            return super().project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)
+        if step.max_position >= self.n_positions:
+            raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
+        qkv = torch.empty(M, n_qkv, dtype=torch.bfloat16, device=x.device)
+        if fused == "rows":
             return rt.ops.gemm_rows_qkv_rope(x, raw, qkv, step.positions, step.token_seq, view.block_table(step), self.table,
                                              view.k, view.v, view.page_size, heads, kv_heads, head_dim, write_kv=view.store,
-                                             columns=columns, rows=rows)
-        if (packed is not None and not getattr(w_qkv, "gated", False) and x.dtype == torch.bfloat16
-                and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing) and x.stride(0) % 8 == 0
-                and x.data_ptr() % 16 == 0 and view.k.dtype == torch.bfloat16):
-            if step.max_position >= self.n_positions:
-                raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
-            qkv = torch.empty(M, (heads + 2 * kv_heads) * head_dim, dtype=torch.bfloat16, device=x.device)
-            return rt.ops.gemv_qkv_rope(x, packed, qkv, step.positions, step.token_seq, view.block_table(step),
-                                        self.table, view.k, view.v, view.page_size, heads, kv_heads, head_dim,
-                                        self.pairing, write_kv=view.store)
-        return super().project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)
+                                             columns=plan.columns, rows=plan.rows)
+        return rt.ops.gemv_qkv_rope(x, packed, qkv, step.positions, step.token_seq, view.block_table(step),
+                                    self.table, view.k, view.v, view.page_size, heads, kv_heads, head_dim,
+                                    self.pairing, write_kv=view.store)

@@ -158,8 +158,9 @@ def test_decode_attention_split_rule():
     """How many pieces a sequence's pages are cut into for the decode attention: never more pieces
     than pages, pieces of at least eight pages (four while the chip would be mostly idle), no more
     blocks than the target."""
-    from burn_lm_amd.parts.attention import DECODE_MIN_BLOCKS, DECODE_TARGET_BLOCKS, decode_splits
-    assert DECODE_TARGET_BLOCKS == 512 and DECODE_MIN_BLOCKS == 128
+    from burn_lm_amd.parts.attention import decode_splits
+    # the targets follow the chip: on half as many compute units, half as many pieces
+    assert decode_splits(64, 8, 64, compute_units=128) == 8 and decode_splits(64, 64, 64, compute_units=64) == 1
     # context 4096 (64 pages), 8 key-value heads: batch 1, 2, 4, 8, 16, 64
     assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 32, 64)] == [16, 8, 8, 8, 4, 1, 1]
     assert decode_splits(256, 32 * 8, 64) == 1                                      # every compute unit has a block: no cutting

@@ -322,8 +322,10 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
     cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=4096, num_hidden_layers=1,
                num_attention_heads=16, num_key_value_heads=4, head_dim=128, vocab_size=300, max_position_embeddings=256,
                rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False)
-    assert Runtime.k_groups(2048, 2048) == 4 and Runtime.k_groups(2048, 4096) == 4 and Runtime.k_groups(6144, 2048) == 2
-    assert Runtime.k_groups(2048, 8192) == 4 and Runtime.k_groups(16384, 2048) == 1 and Runtime.k_groups(4096, 4096) == 2
+    rt = Runtime(torch.bfloat16, "cuda:0")
+    assert rt.compute_units == 256
+    assert rt.k_groups(2048, 2048) == 4 and rt.k_groups(2048, 4096) == 4 and rt.k_groups(6144, 2048) == 2
+    assert rt.k_groups(2048, 8192) == 4 and rt.k_groups(16384, 2048) == 1 and rt.k_groups(4096, 4096) == 2
     folder = make_folder(tmp_path / "wide", cfg, seed=5, std=0.03)
     plain = P.load_model_folder(folder)
     reqs = [random_tokens(200 + i, 300, n) for i, n in enumerate([20, 9, 41])]

@@ -36,13 +36,14 @@ class ToyEngine:
         self.steps.append([(s, len(t)) for s, t, _ in entries])
         rows = []
         for s, toks, want in entries:
-            assert want == [len(toks) - 1]
+            assert want in ([len(toks) - 1], [])    # a prompt's earlier pieces ask for nothing
             self.sums[s] += sum(toks)
             self.cache.advance(s, len(toks))
-            row = torch.zeros(self.vocab_size)
-            row[self.sums[s] % self.vocab_size] = 1.0
-            rows.append(row)
-        return torch.stack(rows)
+            if want:
+                row = torch.zeros(self.vocab_size)
+                row[self.sums[s] % self.vocab_size] = 1.0
+                rows.append(row)
+        return torch.stack(rows) if rows else None
 
 
 class HostArgmax:
@@ -123,6 +124,70 @@ def test_context_end_and_refused_prompts():
     assert res[2].finish_reason == "error" and not res[2].tokens
     assert res[3].finish_reason == "length" and len(res[3].tokens) == 12
     assert eng.cache.pages_in_use() == 0
+
+
+def test_a_batch_of_long_prompts_is_fed_in_steps_of_the_budget():
+    """Prompts of 5, 3, 9 and 1 tokens with a budget of 6: three steps, the sequences in order, a prompt
+    cut where a step is full, logits asked for with each prompt's last piece only; tokens and statistics
+    as with one step."""
+    from burn_lm_amd.engine.generate import plan_prompt_steps
+    assert plan_prompt_steps([5, 3, 9, 1], 6) == [[(0, 0, 5), (1, 0, 1)], [(1, 1, 2), (2, 0, 4)], [(2, 4, 5), (3, 0, 1)]]
+    assert plan_prompt_steps([5, 3], 8) == [[(0, 0, 5), (1, 0, 3)]]
+    assert plan_prompt_steps([13], 4) == [[(0, 0, 4)], [(0, 4, 4)], [(0, 8, 4)], [(0, 12, 1)]]
+    assert plan_prompt_steps([], 4) == []
+    with pytest.raises(ValueError):
+        plan_prompt_steps([3, 0], 4)
+    prompts = [[1, 2, 3, 4, 5], [4] * 3, [7, 1, 2, 3, 4, 5, 6, 7, 8], [9]]
+    whole_eng = ToyEngine(max_tokens=512)
+    whole, whole_stats = generate(whole_eng, prompts, HostArgmax(), sample_len=5, batch_size=4)
+    eng = ToyEngine(max_tokens=512)
+    res, stats = generate(eng, prompts, HostArgmax(), sample_len=5, batch_size=4, prompt_budget=6)
+    assert [r.tokens for r in res] == [r.tokens for r in whole] == [expected(p, 5) for p in prompts]
+    s = eng.opened
+    assert eng.steps[:3] == [[(s[0], 5), (s[1], 1)], [(s[1], 2), (s[2], 4)], [(s[2], 5), (s[3], 1)]]
+    assert all(n == 1 for st in eng.steps[3:] for _, n in st) and len(eng.steps[3]) == 4
+    assert stats.prompt_tokens == whole_stats.prompt_tokens == 18
+    assert stats.steps == whole_stats.steps + 2 and stats.generated_tokens == whole_stats.generated_tokens
+    assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 4
+    # a budget that the prompts do not exceed changes nothing
+    eng2 = ToyEngine(max_tokens=512)
+    generate(eng2, prompts, HostArgmax(), sample_len=5, batch_size=4, prompt_budget=18)
+    assert eng2.steps == whole_eng.steps
+    with pytest.raises(ValueError):
+        generate(eng, prompts, HostArgmax(), sample_len=5, prompt_budget=0)
+
+
+def test_a_request_that_cannot_fit_the_cache_ends_with_an_error_and_the_others_run():
+    # pages of 16 and 4 of them; a context of 128: the second request may grow to 100 tokens = 7 pages
+    unfit = []
+    assert plan_batches([10, 90, 10], 10, 8, 128, 16, 4, 8, unfit) == [[0, 2]] and unfit == [1]
+    eng = ToyEngine(max_tokens=64, max_context=64)
+    eng.max_context = 128       # an engine whose context is longer than its cache (several groups of layers can make it so)
+    res, _ = generate(eng, [[1] * 10, [2] * 90, [3] * 10], HostArgmax(), sample_len=10, batch_size=8)
+    assert res[1].finish_reason == "error" and "pages" in res[1].error and not res[1].tokens
+    assert [r.tokens for r in (res[0], res[2])] == [expected([1] * 10, 10), expected([3] * 10, 10)]
+    assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 4
+
+
+def test_a_prompt_step_that_the_cache_refuses_fails_its_request_only():
+    """The planner counts pages; a cache may still refuse (here: a stand-in that takes no more than 30 new tokens
+    per step).  The batch is tried again one request at a time, the one that is refused alone ends with
+    the cache's message, nothing stays open."""
+    from burn_lm_amd.cache.cache import CacheFull
+
+    class Narrow(ToyEngine):
+        def step(self, entries):
+            if sum(len(t) for _, t, _ in entries) > 30:
+                raise CacheFull("no room for %d tokens" % sum(len(t) for _, t, _ in entries))
+            return super().step(entries)
+
+    eng = Narrow(max_tokens=256)
+    prompts = [[1] * 10, [2] * 40, [3] * 12]
+    res, _ = generate(eng, prompts, HostArgmax(), sample_len=4, batch_size=4)
+    assert res[1].finish_reason == "error" and "no room for 40" in res[1].error
+    assert [r.tokens for r in (res[0], res[2])] == [expected(prompts[0], 4), expected(prompts[2], 4)]
+    assert [r.finish_reason for r in (res[0], res[2])] == ["length", "length"]
+    assert eng.cache.pages_in_use() == 0 and eng.cache.free_slots == 4
 
 
 def test_sample_len_zero_and_callback_order():

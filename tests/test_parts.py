@@ -8,6 +8,8 @@ import torch
 
 import plain_llama as P
 
+PAGE = 64
+
 pytestmark = pytest.mark.gpu
 
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
@@ -104,7 +106,7 @@ def test_attention_part(rt, pairing, heads, kv_heads, hd):
     want = [P.attention_layer(x.double().numpy()[None], wq, wk, tn["v"], tn["o"], heads, kv_heads, hd, freqs)[0]
             for x in xs]
     for cuts in ([37, 1, 20], [30, 1, 7]):
-        cache = Cache([attn.cache_need()], [None], 1024, 8, 256, rt.page_size, rt.dtype, rt.device)
+        cache = Cache([attn.cache_need()], [None], 1024, 8, 256, PAGE, rt.dtype, rt.device)
         slots = [cache.open() for _ in lens]
         done = [0, 0, 0]
         outs = [[], [], []]
@@ -185,7 +187,7 @@ def test_pre_norm_block(rt):
     for p in parts:
         p.bind(on_gpu(t), rt)
     block = registry.part("block", "pre_norm")(dict(mixer=parts[0], feed_forward=parts[1], mixer_norm=parts[2], ffn_norm=parts[3]))
-    cache = Cache([parts[0].cache_need()], [None], 256, 2, 64, rt.page_size, rt.dtype, rt.device)
+    cache = Cache([parts[0].cache_need()], [None], 256, 2, 64, PAGE, rt.dtype, rt.device)
     s = cache.open()
     cache.reserve([(s, 19)])
     step = build_step([(s, [0] * 19, [])], cache, rt.device)

@@ -207,3 +207,93 @@ def test_a_routed_feed_forward_and_another_position_encoding(tmp_path, dtype, to
     for s in slots:
         eng.close(s)
     assert eng.cache.pages_in_use() == 0
+
+
+def test_a_toy_encoding_with_a_fused_projection_asks_the_runtime_for_its_geometry(tmp_path):
+    """A position encoding defined here that fuses the q/k/v projection with its own work (it turns
+    nothing: a table of cosine one and sine zero, handed to the library's fused kernels as its own)
+    holds no threshold: which launch geometry suits which number of rows is the runtime's answer
+    (Runtime.qkv_plan), and the encoding only checks what its own kernels take.  Steps of 1 to 300 rows
+    meet every answer (packed, row ring with 32 and 64 rows staged, none); the logits are the plain
+    attention's without rotation."""
+    from burn_lm_amd import registry
+    from burn_lm_amd.engine.loading import load_engine
+    from burn_lm_amd.models.plan import LayerPlan, ModelPlan, Place
+    from burn_lm_amd.parts.base import PartSpec, PositionEncoding
+    from burn_lm_amd.weights import safetensors_io as st
+    asked = []
+
+    class Still(PositionEncoding):
+        graph_safe = True
+
+        def prepare(self, n_positions, rt):
+            hd = self.params["head_dim"]
+            self.table = torch.stack([torch.ones(n_positions, hd // 2), torch.zeros(n_positions, hd // 2)], -1).to(rt.device)
+
+        def encode_and_store(self, qkv, step, view, heads, kv_heads, head_dim, store=True):
+            self.rt.ops.rope_kv_write(qkv, step.positions, step.token_seq, view.block_table(step), self.table, view.k, view.v,
+                                      view.page_size, heads, kv_heads, head_dim, 0, write_kv=store)
+
+        def project_encode_store(self, x, w_qkv, step, view, heads, kv_heads, head_dim):
+            rt, (M, K) = self.rt, x.shape
+            N = (heads + 2 * kv_heads) * head_dim
+            plan = rt.qkv_plan(M, N, K)
+            asked.append((M, plan))
+            if x.dtype != torch.bfloat16 or plan is None:
+                return super().project_encode_store(x, w_qkv, step, view, heads, kv_heads, head_dim)
+            qkv = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+            common = (step.positions, step.token_seq, view.block_table(step), self.table, view.k, view.v, view.page_size,
+                      heads, kv_heads, head_dim)
+            if plan.kernel == "rows":
+                return rt.ops.gemm_rows_qkv_rope(x, w_qkv.w, qkv, *common, write_kv=view.store, columns=plan.columns, rows=plan.rows)
+            return rt.ops.gemv_qkv_rope(x, w_qkv.packed, qkv, *common, 0, write_kv=view.store)
+
+    cfg = dict(architectures=["ToyStillLM"], width=256, inner=512, heads=4, kv_heads=2, head_dim=64, vocab=97, eps=1e-5)
+
+    def plan(c, names=None):
+        D = c["width"]
+        norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=c["eps"]), dict(weight=n))
+        layer = LayerPlan("pre_norm", position="still", mixer_norm=norm("n1"), ffn_norm=norm("n2"),
+                          mixer=PartSpec("attention", dict(width=D, heads=c["heads"], kv_heads=c["kv_heads"], head_dim=c["head_dim"],
+                                                           scale=c["head_dim"] ** -0.5), dict(q="q", k="k", v="v", o="o")),
+                          feed_forward=PartSpec("swiglu", dict(width=D, inner=c["inner"]), dict(gate="gate", up="up", down="down")))
+        return ModelPlan(vocab_size=c["vocab"], width=D, max_positions=1024, layers=[layer], order=[Place(0)],
+                         embedding=PartSpec("table", dict(vocab=c["vocab"], width=D), dict(weight="emb")),
+                         final_norm=norm("norm"), head=PartSpec("linear", dict(vocab=c["vocab"], width=D), dict(weight="emb")),
+                         positions={"still": PartSpec("toy_still", dict(head_dim=c["head_dim"]))})
+
+    registry.register_part("position", "toy_still", Still)
+    registry.register_architecture(registry.Architecture("ToyStillLM", read_config=lambda d: d, plan=plan))
+    g = torch.Generator().manual_seed(9)
+    D, hd = cfg["width"], cfg["head_dim"]
+    m = lambda *s: (torch.randn(*s, generator=g) * 0.06).bfloat16()
+    t = {"emb": m(cfg["vocab"], D), "norm": torch.ones(D).bfloat16(), "n1": torch.ones(D).bfloat16(), "n2": torch.ones(D).bfloat16(),
+         "q": m(cfg["heads"] * hd, D), "k": m(cfg["kv_heads"] * hd, D), "v": m(cfg["kv_heads"] * hd, D), "o": m(D, cfg["heads"] * hd),
+         "gate": m(cfg["inner"], D), "up": m(cfg["inner"], D), "down": m(D, cfg["inner"])}
+    json.dump(cfg, open(tmp_path / "config.json", "w"))
+    st.write_file(str(tmp_path / "model.safetensors"), t.items())
+    w = {k: v.double().numpy() for k, v in t.items()}
+
+    def plain(tokens):
+        h = w["emb"][np.asarray(tokens)][None]
+        still = np.zeros(hd // 2)       # no turning at any position
+        h = h + P.attention_layer(P.rms_norm(h, w["n1"], cfg["eps"]), w["q"], w["k"], w["v"], w["o"], cfg["heads"], cfg["kv_heads"], hd, still)
+        h = h + P.swiglu_feed_forward(P.rms_norm(h, w["n2"], cfg["eps"]), w["gate"], w["up"], w["down"])
+        return (P.rms_norm(h, w["norm"], cfg["eps"]) @ w["emb"].T)[0]
+
+    eng = load_engine(str(tmp_path), dtype="bfloat16", max_tokens=4096, max_seqs=300, graphs=False)
+    rng = np.random.default_rng(4)
+    for rows in (1, 9, 40, 100, 300):
+        del asked[:]
+        reqs = [[int(x) for x in rng.integers(0, cfg["vocab"], 3 + (5 * i) % 7)] for i in range(rows)]
+        slots = [eng.open() for _ in reqs]
+        eng.step([(s, r[:-1], []) for s, r in zip(slots, reqs)])
+        got = eng.step([(s, [r[-1]], [0]) for s, r in zip(slots, reqs)]).double().cpu().numpy()    # one row per sequence
+        assert asked[-1][0] == rows and asked[-1][1] == eng.rt.qkv_plan(rows, (cfg["heads"] + 2 * cfg["kv_heads"]) * hd, D)
+        kind = asked[-1][1].kernel if asked[-1][1] is not None else None
+        assert kind == {1: "packed", 9: "packed", 40: "rows", 100: "rows", 300: None}[rows], (rows, asked[-1])
+        for i in range(0, rows, max(1, rows // 12)):
+            want = plain(reqs[i])[-1]
+            assert float(np.abs(got[i] - want).max() / np.abs(want).max()) <= 3e-2, (rows, i)
+        for s in slots:
+            eng.close(s)
