@@ -948,3 +948,85 @@ def test_random_weights_are_the_same_bytes_on_the_gpu_and_in_a_folder(tmp_path):
         b = random_engine(cfg, seed=21, dtype=dtype, max_tokens=1024, std=0.08, norm_jitter=0.1)
         sa, sb = a.open(), b.open()
         assert torch.equal(a.step([(sa, toks, list(range(40)))]), b.step([(sb, toks, list(range(40)))]))
+
+
+def test_prompts_fed_within_a_budget_give_the_tokens_of_one_step(folders):
+    """generate() with a prompt budget smaller than a batch's prompts feeds them in several steps (prompts cut
+    where a step is full); in 32-bit the tokens equal those of the run that feeds each batch in one step,
+    and the plain implementation's."""
+    from burn_lm_amd.engine.generate import generate
+    from burn_lm_amd.sampling.sampler import Sampler
+    cfg, _ = TINIES["B"]
+    plain = P.load_model_folder(folders["B"])
+    lens = [41, 3, 77, 20, 1, 58, 9]
+    prompts = [random_tokens(900 + i, cfg["vocab_size"], n) for i, n in enumerate(lens)]
+    want = [P.greedy_generate(plain, p, 6) for p in prompts]
+    eng = load(folders["B"], "float32", max_tokens=2048, max_seqs=4)
+    steps = []
+    real = eng.step
+    eng.step = lambda entries: (steps.append([len(t) for _, t, _ in entries]), real(entries))[1]
+    whole, whole_stats = generate(eng, prompts, Sampler(temperature=0.0), 6, batch_size=4)
+    n_whole = len(steps)
+    cut, stats = generate(eng, prompts, Sampler(temperature=0.0), 6, batch_size=4, prompt_budget=32)
+    assert [r.tokens for r in cut] == [r.tokens for r in whole] == want
+    prompt_steps = [s for s in steps[n_whole:] if max(s) > 1 or sum(s) > len(s)]
+    assert all(sum(s) <= 32 for s in prompt_steps) and len(prompt_steps) == -(-sum(lens[:4]) // 32) + -(-sum(lens[4:]) // 32)
+    assert stats.prompt_tokens == whole_stats.prompt_tokens == sum(lens)
+    assert eng.cache.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("name,vocab", [("llama3.2-1b", 20008), ("llama3.2-3b", 20008), ("llama3.1-8b", 20008)])
+def test_decode_steps_of_100_and_200_sequences_at_the_benchmark_widths(tmp_path, monkeypatch, name, vocab):
+    """One layer of each benchmark shape, a batch of 100 and one of 200 short prompts, then six tokens one by one with
+    every row's logits wanted, against the plain implementation in both dtypes.  These are the decode steps of 65
+    to 256 rows: the fused q/k/v projection with a block for every 64 rows, the output projection on the row-ring
+    product at the 1B width, the head of many rows on the matrix-core kernel with a float32 output, and the decode
+    attention uncut; the counters say that these kernels were the ones that ran."""
+    from burn_lm_amd.config.presets import preset
+    from burn_lm_amd.csrc import ops
+    cfg = dict(preset(name))
+    cfg["num_hidden_layers"] = 1
+    cfg["vocab_size"] = vocab
+    cfg.pop("eos_token_id", None), cfg.pop("bos_token_id", None)
+    folder = make_folder(tmp_path / "shape", cfg, seed=4, std=0.02)
+    plain = P.load_model_folder(folder)
+    n_dec = 6
+    reqs = [random_tokens(70 + i, vocab, 1 + (7 * i) % 23 + n_dec) for i in range(200)]
+
+    def plain_rows(toks, rows):
+        h = plain["tok_embeddings"][np.asarray([toks])]
+        for lw in plain["layers"]:
+            h = P.block(h, lw, plain["cfg"], plain["freqs"], 0)
+        return P.rms_norm(h, plain["norm"], plain["cfg"]["eps"])[0][rows] @ plain["output"].T
+
+    want = [plain_rows(r, list(range(len(r) - n_dec, len(r)))) for r in reqs]
+    calls = {"qkv": [], "rows": [], "head": [], "attn": []}
+    real_qkv, real_rows, real_mfma, real_attn = ops.gemm_rows_qkv_rope, ops.gemm_rows, ops.gemm_mfma, ops.attn_decode
+    monkeypatch.setattr(ops, "gemm_rows_qkv_rope", lambda x, *a, **k: (calls["qkv"].append(x.shape[0]), real_qkv(x, *a, **k))[1])
+    monkeypatch.setattr(ops, "gemm_rows", lambda a, w, out, **k: (calls["rows"].append(tuple(out.shape)), real_rows(a, w, out, **k))[1])
+    monkeypatch.setattr(ops, "gemm_mfma", lambda a, w, out, **k: (calls["head"].append(tuple(out.shape)) if out.dtype == torch.float32
+                                                                  and out.dim() == 2 else None, real_mfma(a, w, out, **k))[1])
+    monkeypatch.setattr(ops, "attn_decode", lambda q, *a, **k: (calls["attn"].append(q.shape[0]), real_attn(q, *a, **k))[1])
+    width = cfg["hidden_size"]
+    for dtype, tol in (("float32", 1e-5), ("bfloat16", TOL["bfloat16"])):
+        eng = load(folder, dtype, max_tokens=200 * 64, max_seqs=200, graphs=False)
+        for n in (100, 200):
+            group = list(range(n))
+            slots = [eng.open() for _ in group]
+            eng.step([(slots[i], reqs[i][:-n_dec], []) for i in group])
+            for k in calls:
+                del calls[k][:]
+            for s in range(n_dec):
+                got = eng.step([(slots[i], [reqs[i][len(reqs[i]) - n_dec + s]], [0]) for i in group]).double().cpu().numpy()
+                for i in group:
+                    assert rel_err(got[i], want[i][s]) <= tol, f"{dtype} batch of {n}: request {i}, decode step {s}"
+            if dtype == "bfloat16":
+                assert calls["qkv"] == [n] * n_dec, (n, calls["qkv"])
+                assert calls["attn"] == [n] * n_dec
+                assert calls["head"] == [(n, vocab)] * n_dec, calls["head"]
+                ring_o = [s for s in calls["rows"] if s[-1] == width and s[-2] == n]
+                assert (len(ring_o) == n_dec) == (width <= 2048), (n, calls["rows"])
+            for s in slots:
+                eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
