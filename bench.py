@@ -110,6 +110,67 @@ def time_workload(engine, batch, prompt_len=512, generated=256):
     return stats.decode_tokens / stats.decode_seconds, stats.prompt_tokens / stats.prompt_seconds
 
 
+def workload_hbm_frac(engine, batch, steps_per_second, prompt_len=512, generated=256):
+    """The 512 + 256 workload's decode steps against the memory roofline: the bytes a step at the
+    workload's mean context has to read (every weight once, the live cache) x steps a second / 8 TB/s."""
+    mean_ctx = prompt_len + generated // 2
+    c = engine.model.step_costs([mean_ctx - 1] * batch, [1] * batch, batch, engine.cache)
+    return round((c["weight_bytes"] + c["cache_bytes"]) * steps_per_second / 1e9 / HBM_PEAK_GBS, 4)
+
+
+def other_shape(name, dtype, batch, context, steps, prefill_tokens):
+    """Decode at `batch` and a prefill of `prefill_tokens` for another preset with all its layers: flat
+    figures for the record's `shapes` block."""
+    import torch
+    from burn_lm_amd.config.presets import preset
+    from burn_lm_amd.engine.loading import random_engine
+    from burn_lm_amd.sampling.sampler import Sampler
+    engine = random_engine(preset(name), seed=0, dtype=dtype, max_tokens=batch * context, max_seqs=batch, max_context=context)
+    sec, _ = time_decode(engine, Sampler(temperature=0.0), batch, context, steps, 4)
+    roof = decode_roofline(engine, batch, context, steps, sec)
+    psec = time_prefill(engine, prefill_tokens, reps=3)
+    pflops = engine.model.step_costs([0], [prefill_tokens], 1)["flops"]
+    short = "bf16" if dtype == "bfloat16" else "fp32"
+    out = {f"{name}_layers": engine.config.num_hidden_layers,
+           f"{name}_decode_b{batch}": round(batch / sec, 1), f"{name}_decode_b{batch}_ms": round(sec * 1e3, 4),
+           f"{name}_decode_b{batch}_hbm_frac": roof["frac"],
+           f"{name}_prefill_{prefill_tokens}": round(prefill_tokens / psec, 1), f"{name}_prefill_{prefill_tokens}_ms": round(psec * 1e3, 3),
+           f"{name}_prefill_{prefill_tokens}_frac": round(pflops / psec / MFMA_PEAK[short], 4)}
+    del engine
+    torch.cuda.empty_cache()
+    return out
+
+
+def reference_bench_shapes(dtype):
+    """The reference's own benchmark (benchmarks/benches/transformer.rs:72-102): one layer of the Llama-3.2-1B, 3B and
+    8B shapes with the whole vocabulary, a forward of (batch 32, 1 token) and of (batch 1, 512 tokens) on an empty
+    cache with the logits of every position: milliseconds per forward (median)."""
+    import torch
+    from burn_lm_amd.config.presets import preset
+    from burn_lm_amd.engine.loading import random_engine
+    out = {}
+    for name in ("llama3.2-1b", "llama3.2-3b", "llama3.1-8b"):
+        cfg = preset(name)
+        cfg["num_hidden_layers"] = 1
+        engine = random_engine(cfg, seed=0, dtype=dtype, max_tokens=32 * 64 + 1024, max_seqs=32, max_context=1024)
+        for batch, length in ((32, 1), (1, 512)):
+            prompts = random_prompts(engine, batch, length, seed=2)
+            times = []
+            for r in range(8):
+                slots = [engine.open() for _ in range(batch)]
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                engine.step([(s, p, list(range(length))) for s, p in zip(slots, prompts)])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                for s in slots:
+                    engine.close(s)
+            out[f"{name}_1layer_b{batch}_s{length}_ms"] = round(statistics.median(times[3:]) * 1e3, 4)
+        del engine
+        torch.cuda.empty_cache()
+    return out
+
+
 def event_time(fn, reps=10, warm=2):
     """Median seconds of fn() between two events."""
     import torch
@@ -281,15 +342,19 @@ def main():
     ap.add_argument("--preset", default="llama3.2-1b")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points, the 512+256 workload and the single kernels")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points, the 512+256 workload, the single kernels "
+                                                             "and the other shapes")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the other presets' figures and the reference's own benchmark shapes")
     ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of picking greedily (0: greedy)")
     ap.add_argument("--top-p", type=float, default=1.0, help="nucleus mass when sampling")
     ap.add_argument("--unequal", type=int, default=0, metavar="N",
                     help="instead of the decode measurement: N prompts of 64..2048 tokens through the generation loop")
     ap.add_argument("--generate", type=int, default=256, help="tokens generated per prompt with --unequal")
-    ap.add_argument("--profile", choices=["decode", "prefill"], default=None,
-                    help="run only this part, for a profiler: the decode steps of the batch, or the prompt step ten times; "
-                         "prints its time and no JSON line")
+    ap.add_argument("--profile", choices=["decode", "prefill", "decode-loop"], default=None,
+                    help="run only this part, for a profiler: the decode steps of the batch through generate(), the prompt "
+                         "step ten times, or (decode-loop, for counter runs, where every launch is slow) --steps decode steps "
+                         "launched kernel by kernel on a cache that is filled without a prompt step; prints its time and "
+                         "no JSON line, and says on stderr where it is")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this library has no multi-GPU path (run with --gpus 1)")
@@ -302,20 +367,49 @@ def main():
     from burn_lm_amd.engine.loading import random_engine
     from burn_lm_amd.sampling.sampler import Sampler
 
+    def say(what):      # a profiled run that stalls should show how far it came
+        if args.profile:
+            print(f"[bench] {what}", file=sys.stderr, flush=True)
+
     config = preset(args.preset)
     full_layers = config["num_hidden_layers"]
     layers = args.layers or full_layers
     config["num_hidden_layers"] = layers
     biggest = max(args.batch, 1 if args.no_points else 64)
+    if args.profile:
+        from burn_lm_amd.csrc import build as _build
+        if _build.under_profiler() and not (_build.is_current() and _build.host_is_current()):
+            print("bench.py: the kernel libraries do not match their sources; build them before profiling "
+                  "(python -c 'import __graft_entry__ as g; g.build()')")
+            sys.exit(2)
+    say("building the engine (random weights)")
     engine = random_engine(config, seed=0, dtype=args.dtype, max_tokens=biggest * args.context,
-                           max_seqs=biggest, max_context=args.context)
+                           max_seqs=biggest, max_context=args.context, graphs=args.profile != "decode-loop")
+    say("engine built")
     cfg = engine.config
+    page_size = engine.cache.page_size
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     sampler = Sampler(temperature=args.temperature, top_p=args.top_p, seed=1)
 
     if args.profile == "prefill":
         print(f"prefill of {args.prefill_tokens} tokens: {time_prefill(engine, args.prefill_tokens, reps=10) * 1e3:.3f} ms")
         return
+    if args.profile == "decode-loop":
+        import torch
+        slots = [engine.open() for _ in range(args.batch)]
+        for s in slots:     # the cache filled by the books alone: what the pages hold does not matter to the kernels' work
+            engine.cache.reserve([(s, args.context - args.steps - 1)])
+            engine.cache.advance(s, args.context - args.steps - 1)
+        say("cache filled; decode steps, kernel by kernel")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            engine.step([(s, [1 + k], [0]) for s in slots])
+        torch.cuda.synchronize()
+        print(f"{args.steps} eager decode steps of batch {args.batch} at context {args.context}: "
+              f"{(time.perf_counter() - t0) / args.steps * 1e3:.3f} ms each")
+        return
+    say("decode through generate()")
     sec, median = time_decode(engine, sampler, args.batch, args.context, args.steps, args.warmup)
     if args.profile == "decode":
         print(f"decode step of batch {args.batch} at context {args.context}: {sec * 1e3:.4f} ms")
@@ -336,9 +430,22 @@ def main():
         for b in (1, 8, 64):
             d, p = time_workload(engine, b)
             workload[f"decode_b{b}"] = round(d, 1)
+            workload[f"decode_b{b}_hbm_frac"] = workload_hbm_frac(engine, b, d / b)
             workload[f"prefill_b{b}"] = round(p, 1)
         measured = machine_rates(engine.rt.device)
         kernels = kernel_rates(engine, args.batch, args.context, T)
+
+    shapes = {}
+    if not (args.no_points or args.no_shapes) and args.preset == "llama3.2-1b" and layers == full_layers:
+        import torch
+        roof = decode_roofline(engine, args.batch, args.context, args.steps, sec)
+        del engine      # its storage goes back before the wider shapes are built
+        torch.cuda.empty_cache()
+        for name in ("llama3.2-3b", "llama3.1-8b"):
+            shapes.update(other_shape(name, args.dtype, args.batch, args.context, 24, T))
+        shapes.update(reference_bench_shapes(args.dtype))
+    else:
+        roof = decode_roofline(engine, args.batch, args.context, args.steps, sec)
 
     out = {
         "metric": "decode_tokens_per_second", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
@@ -349,14 +456,14 @@ def main():
                    "layers_of_shape": full_layers, "hidden_size": cfg.hidden_size,
                    "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size,
-                   "tied_head": cfg.tie_word_embeddings, "page_size": engine.cache.page_size,
+                   "tied_head": cfg.tie_word_embeddings, "page_size": page_size,
                    "sampling": "greedy" if args.temperature == 0 else f"temperature {args.temperature:g} top-p {args.top_p:g}",
                    "parallelism": "single GPU"},
         "step_ms_median": round(median * 1e3, 4),
         "prefill": {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
                     "frac": round(pflops / psec / MFMA_PEAK[short], 4)},
-        "roofline": decode_roofline(engine, args.batch, args.context, args.steps, sec),
-        "points": points, "workload_512_256": workload, "measured": measured, "kernels": kernels,
+        "roofline": roof,
+        "points": points, "workload_512_256": workload, "shapes": shapes, "measured": measured, "kernels": kernels,
     }
     print(json.dumps(out))
 

@@ -198,6 +198,7 @@ def ensure_ref_built(verbose=True):
 def ensure_host_built(verbose=True):
     if host_is_current():
         return host_lib_path()
+    _refuse_under_profiler(HOST_LIB_NAME)
     return build_host(verbose=verbose)
 
 
@@ -266,10 +267,26 @@ def build(verbose=True, jobs=None, with_ref=False):
     return os.path.join(od, LIB_NAME)
 
 
+def under_profiler():
+    """Whether this process runs under a profiler that preloads a tool library into every child (rocprofv3
+    does): a compiler started from here would load it too and start collecting on its own."""
+    env = os.environ
+    return ("rocprof" in env.get("LD_PRELOAD", "").lower() or
+            any(k.startswith(("ROCPROF", "ROCP_TOOL", "ROCPROFILER")) for k in env))
+
+
+def _refuse_under_profiler(what):
+    if under_profiler():
+        raise RuntimeError(f"{what} does not match its sources and would have to be compiled, but this process runs "
+                           f"under a profiler whose preloaded library every compiler process would inherit: build first "
+                           f"(python -c 'import __graft_entry__ as g; g.build()'), then profile")
+
+
 def ensure_built(verbose=True):
     """Path of a library that matches the sources, building it first if there is none."""
     if is_current():
         return lib_path()
+    _refuse_under_profiler(LIB_NAME)
     return build(verbose=verbose)
 
 
