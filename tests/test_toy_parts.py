@@ -281,7 +281,7 @@ def test_a_toy_encoding_with_a_fused_projection_asks_the_runtime_for_its_geometr
         h = h + P.swiglu_feed_forward(P.rms_norm(h, w["n2"], cfg["eps"]), w["gate"], w["up"], w["down"])
         return (P.rms_norm(h, w["norm"], cfg["eps"]) @ w["emb"].T)[0]
 
-    eng = load_engine(str(tmp_path), dtype="bfloat16", max_tokens=4096, max_seqs=300, graphs=False)
+    eng = load_engine(str(tmp_path), dtype="bfloat16", max_tokens=300 * 64, max_seqs=300, graphs=False)
     rng = np.random.default_rng(4)
     for rows in (1, 9, 40, 100, 300):
         del asked[:]
