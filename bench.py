@@ -223,13 +223,13 @@ def kernel_rates(engine, batch, context, prefill_tokens):
         all_ = list(weights)
         while size < least:
             for w in weights:
-                all_.append(LinearWeight(w.w.clone(), None if w.packed is None else w.packed.clone(), w.gated))
+                all_.append(LinearWeight(w.w.clone(), w.packable, w.gated))
             size *= 2
         return all_
 
     def graph_time(calls):
         """Seconds per call of the calls recorded one after another."""
-        for c in calls[:2]:
+        for c in calls:     # once outside the recording: a weight's packed copy is made at its first product
             c()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()

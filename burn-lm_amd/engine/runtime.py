@@ -80,11 +80,32 @@ class FusedProjectionPlan:
 
 
 class LinearWeight:
-    """A bound weight matrix [N, K] and, for bfloat16, its copy packed for the skinny product."""
+    """A bound weight matrix [N, K] and, where the skinny product takes it, its copy packed for that
+    product.  The copy is made when a product first asks for it (``packed``): an engine that only ever
+    runs prompts and large batches never holds a matrix twice.  ``packable`` says whether there is one to
+    be had; ``drop_packed()`` gives its memory back (it is made again on demand)."""
 
-    def __init__(self, w, packed=None, gated=False):
-        self.w, self.packed, self.gated = w, packed, gated
+    def __init__(self, w, packable=False, gated=False, packed=None):
+        self.w, self.gated = w, gated
+        self.packable = bool(packable) or packed is not None
+        self._packed = packed
         self.shape, self.dtype = w.shape, w.dtype
+
+    @property
+    def packed(self):
+        if self._packed is None and self.packable:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("a weight's packed copy would have to be made while a graph is being recorded; a step "
+                                   "of this shape has to run once outside a recording first")
+            self._packed = ops.pack_weight(self.w, gated=self.gated)
+        return self._packed
+
+    @property
+    def is_packed(self):
+        return self._packed is not None
+
+    def drop_packed(self):
+        self._packed = None
 
 
 class Runtime:
@@ -121,15 +142,15 @@ class Runtime:
         return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
 
     def weight(self, w, gated=False):
-        """Prepares a bound matrix for linear(): bfloat16 matrices get the packed copy that the
-        skinny product streams (it doubles their memory; the plain copy serves prefill).
+        """Prepares a bound matrix for linear(): bfloat16 matrices may get a packed copy that the
+        skinny product streams (made at the first product of up to 16 rows, or of up to 64 where no other
+        kernel takes them; it doubles the matrix's memory; the plain copy serves everything else).
         gated=True: w is [gate rows; up rows] of a gated feed-forward and will be used through
         gated_linear(); its packed copy pairs each gate row with its up row."""
         w = w.contiguous()
         N, K = w.shape
-        if w.dtype == torch.bfloat16 and ops.gemv_mfma_supported(1, N, K) and (not gated or N % 16 == 0):
-            return LinearWeight(w, ops.pack_weight(w, gated=gated), gated)
-        return LinearWeight(w)
+        packable = w.dtype == torch.bfloat16 and ops.gemv_mfma_supported(1, N, K) and (not gated or N % 16 == 0)
+        return LinearWeight(w, packable, gated)
 
     def k_groups(self, N, K, M=1):
         """Into how many groups a skinny product's K is cut so that a narrow output still gives
@@ -217,13 +238,14 @@ class Runtime:
         LinearWeight from weight(), or a plain tensor.  partials=True allows the result to come as
         float32 [groups, M, N] partial products (the caller hands it to a norm's add, which sums
         them); it is used for narrow outputs in decode."""
-        packed = None
+        packable, holder = False, None
         if isinstance(w, LinearWeight):
-            w, packed = w.w, (None if w.gated else w.packed)   # a gated copy has its rows re-ordered
+            holder, w = w, w.w
+            packable = holder.packable and not holder.gated   # a gated copy has its rows re-ordered
         M, K = x.shape
         N = w.shape[0]
         out_dtype = out_dtype or self.dtype
-        if out is None and not (partials and packed is not None):
+        if out is None and not (partials and packable):
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         if w.dtype == torch.float32 or x.dtype == torch.float32:
             if M <= SKINNY_MAX_ROWS and x.dtype == w.dtype == out_dtype == torch.float32 and K % 8 == 0 \
@@ -253,15 +275,15 @@ class Runtime:
             groups, columns = self.rows_plan(N, K)
             if groups > 1:
                 return ops.gemm_rows(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), columns=columns)
-        if packed is not None and M <= MFMA_SKINNY_MAX_ROWS and aligned:
+        if packable and M <= MFMA_SKINNY_MAX_ROWS and aligned:
             if partials and out is None:
                 groups = self.k_groups(N, K, M)
                 if groups > 1:
-                    return ops.gemv_mfma(x, packed, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), K)
+                    return ops.gemv_mfma(x, holder.packed, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), K)
             if ops.gemv_mfma_supported(M, N, K):
                 if out is None:
                     out = torch.empty(M, N, dtype=out_dtype, device=x.device)
-                return ops.gemv_mfma(x, packed, out, K)
+                return ops.gemv_mfma(x, holder.packed, out, K)
         if out is None:
             out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         if (out_dtype == torch.float32 and M > 32 and aligned and x.dtype == w.dtype == torch.bfloat16
@@ -273,13 +295,13 @@ class Runtime:
             # width 3072, 33-64 rows: 154-169 against 268-298; width 4096: 233-238 against 329-350, 65-128 rows
             # 240-252 against 509-687; the library's product with a float output: equal to 5 % behind.
             return ops.gemm_mfma(x, w, out, tile=(128, 128, 4) if M <= 128 else (256, 128))
-        if packed is not None and aligned and out_dtype == torch.float32:
+        if packable and aligned and out_dtype == torch.float32:
             # 17 to 32 rows at a K above 4096: the most rows the skinny product does take at a time (16); the
             # weights stream once per chunk, which still beats the plain tiled kernel by far
             chunk = next((c for c in (64, 32, 16) if ops.gemv_mfma_supported(c, N, K)), 0)
             if chunk:
                 for r in range(0, M, chunk):
-                    ops.gemv_mfma(x[r:r + chunk], packed, out[r:r + chunk], K)
+                    ops.gemv_mfma(x[r:r + chunk], holder.packed, out[r:r + chunk], K)
                 return out
         if M <= SKINNY_MAX_ROWS and aligned:
             return ops.gemv_skinny(x, w, out)
@@ -303,7 +325,7 @@ class Runtime:
             # at wider ones in place of the library's product, which the packed kernel's registers leave them to);
             # from 17 rows on where K is above 2048 and the blocks come in one round (3B: 10-15 %)
             return ops.gemm_rows(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True)
-        if (isinstance(w, LinearWeight) and w.packed is not None and w.gated and x.dtype == torch.bfloat16
+        if (isinstance(w, LinearWeight) and w.packable and w.gated and x.dtype == torch.bfloat16
                 and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)

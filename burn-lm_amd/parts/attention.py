@@ -33,8 +33,12 @@ def decode_splits(pages: int, blocks: int, head_dim: int, compute_units: int = 2
     32 pieces, 22.3 with 64 and 31.4 with 128 (every piece costs its look-ups, its partial result and
     its arrival; the merge reads them all).  And no cutting at all once every compute unit has a block:
     an uncut sequence needs no partial result, no arrival and no merge (batch 32, context 4096: 48.5 us
-    uncut, 57.8 in two pieces; context 16,384: 171 against 186)."""
-    if blocks >= compute_units:
+    uncut, 57.8 in two pieces; context 16,384: 171 against 186).  Nor for short ranges, two pages per
+    wavefront and (for heads up to 64) three: a merge costs three trips through device-coherent memory in a
+    row, about 3 us, a further page per wavefront about 2 (us per call, cut in two / uncut, 32 heads of 64
+    in 8 groups: 8 pages at batch 1 7.1 / 6.6, at batch 8 8.1 / 7.0; 11 pages 7.9 / 8.0 and 9.0 / 8.4;
+    16 pages, cut in four, 7.3 / 10.2; heads of 128: 8 pages 11.1 / 11.1, 11 pages 12.8 / 13.7)."""
+    if blocks >= compute_units or pages <= (12 if head_dim <= 64 else 8):
         return 1
     target = compute_units * DECODE_TARGET_PER_UNIT if head_dim <= 64 else max(1, compute_units * DECODE_TARGET_PER_UNIT // 2)
     least = max(1, int(compute_units * DECODE_MIN_PER_UNIT))

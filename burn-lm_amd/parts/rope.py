@@ -99,13 +99,13 @@ class RotaryEncoding(PositionEncoding):
         n_qkv = (heads + 2 * kv_heads) * head_dim
         plan = rt.qkv_plan(M, n_qkv, K) if hasattr(rt, "qkv_plan") else None
         bf16 = x.dtype == view.k.dtype == torch.bfloat16 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-        raw, packed = getattr(w_qkv, "w", None), getattr(w_qkv, "packed", None)
+        raw, packable = getattr(w_qkv, "w", None), getattr(w_qkv, "packable", False)
         fused = None
         if (plan is not None and plan.kernel == "rows" and bf16 and self.pairing == PAIRING["interleaved"]
                 and raw is not None and raw.dtype == torch.bfloat16 and raw.is_contiguous()
                 and head_dim % 2 == 0 and K % 8 == 0 and x.stride(1) == 1):
             fused = "rows"
-        elif (plan is not None and M <= 64 and bf16 and packed is not None and not getattr(w_qkv, "gated", False)
+        elif (plan is not None and M <= 64 and bf16 and packable and not getattr(w_qkv, "gated", False)
                 and rt.ops.gemv_qkv_rope_supported(M, K, head_dim, self.pairing)):
             fused = "packed"     # also where the row-ring kernel was the plan and this encoding has none for it
         if fused is None:
@@ -117,6 +117,6 @@ class RotaryEncoding(PositionEncoding):
             return rt.ops.gemm_rows_qkv_rope(x, raw, qkv, step.positions, step.token_seq, view.block_table(step), self.table,
                                              view.k, view.v, view.page_size, heads, kv_heads, head_dim, write_kv=view.store,
                                              columns=plan.columns, rows=plan.rows)
-        return rt.ops.gemv_qkv_rope(x, packed, qkv, step.positions, step.token_seq, view.block_table(step),
+        return rt.ops.gemv_qkv_rope(x, w_qkv.packed, qkv, step.positions, step.token_seq, view.block_table(step),
                                     self.table, view.k, view.v, view.page_size, heads, kv_heads, head_dim,
                                     self.pairing, write_kv=view.store)

@@ -165,7 +165,9 @@ def test_decode_attention_split_rule():
     assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 32, 64)] == [16, 8, 8, 8, 4, 1, 1]
     assert decode_splits(256, 32 * 8, 64) == 1                                      # every compute unit has a block: no cutting
     assert decode_splits(64, 8, 128) == 16 and decode_splits(64, 64, 128) == 4      # wide heads: half the blocks
-    assert decode_splits(1, 8, 64) == 1 and decode_splits(3, 8, 64) == 1 and decode_splits(8, 8, 64) == 2
+    assert decode_splits(1, 8, 64) == 1 and decode_splits(3, 8, 64) == 1 and decode_splits(8, 8, 64) == 1
+    # short ranges stay whole: up to two pages per wavefront, three with heads up to 64
+    assert decode_splits(12, 8, 64) == 1 and decode_splits(13, 8, 64) == 3 and decode_splits(8, 8, 128) == 1 and decode_splits(12, 8, 128) == 3
     assert decode_splits(2048, 8, 64) == 32 and decode_splits(512, 8, 64) == 32     # a long context at batch 1: the cap
     for pages in (1, 2, 5, 8, 9, 31, 64, 100, 1000):
         for blocks in (1, 3, 8, 64, 500, 5000):

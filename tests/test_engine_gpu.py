@@ -804,12 +804,12 @@ def test_checkpoints_stored_in_32_bit_and_in_float16(tmp_path, capsys):
     eng, got = run(f32, "bfloat16")
     note = capsys.readouterr().err
     assert "stored in 32 bits" in note and "cast_32bit" in note
-    assert eng.model.blocks[0].mixer.w_qkv.dtype == torch.float32 and eng.model.blocks[0].mixer.w_qkv.packed is None
+    assert eng.model.blocks[0].mixer.w_qkv.dtype == torch.float32 and not eng.model.blocks[0].mixer.w_qkv.packable
     assert max(rel_err(got[p], want32[p]) for p in range(150)) <= TOL["bfloat16"]
     # the same folder with its matrices rounded when they are loaded: the packed products, and the
     # bfloat16 folder's logits to the bit (the weights are the same bytes then; norm weights stay wide)
     eng_c, got_c = run(f32, "bfloat16", cast_32bit=True)
-    assert eng_c.model.blocks[0].mixer.w_qkv.dtype == torch.bfloat16 and eng_c.model.blocks[0].mixer.w_qkv.packed is not None
+    assert eng_c.model.blocks[0].mixer.w_qkv.dtype == torch.bfloat16 and eng_c.model.blocks[0].mixer.w_qkv.packable
     assert eng_c.model.blocks[0].mixer_norm.gamma.dtype == torch.float32
     plain16 = P.load_model_folder(b16)
     want16 = P.transformer_forward([toks], plain16)[0]
@@ -1030,3 +1030,29 @@ def test_decode_steps_of_100_and_200_sequences_at_the_benchmark_widths(tmp_path,
                 eng.close(s)
         del eng
         torch.cuda.empty_cache()
+
+
+def test_packed_copies_of_the_weights_are_made_when_a_small_step_first_needs_them(folders):
+    """A bound bfloat16 matrix is held once until a product of few rows asks for its packed copy: after a prompt of
+    many rows none has one, after the first decode step those that such a step multiplies have, and the logits are
+    the same with the copies dropped and made again."""
+    cfg, _ = TINIES["C"]
+    eng = load(folders["C"], "bfloat16", max_tokens=2048, max_seqs=4, graphs=False)
+    held = lambda: [w.is_packed for b in eng.model.blocks for w in (b.mixer.w_qkv, b.mixer.w_o, b.feed_forward.w_gate_up,
+                                                                     b.feed_forward.w_down)]
+    assert all(w.packable for b in eng.model.blocks for w in (b.mixer.w_qkv, b.feed_forward.w_gate_up))
+    toks = random_tokens(5, cfg["vocab_size"], 300)
+    s = eng.open()
+    eng.step([(s, toks[:290], [])])
+    assert not any(held()), "a prompt of 290 rows needs no packed copy"
+    first = eng.step([(s, [toks[290]], [0])]).clone()
+    assert all(held()), "a decode step of one row multiplies every matrix through its packed copy"
+    for b in eng.model.blocks:
+        for w in (b.mixer.w_qkv, b.mixer.w_o, b.feed_forward.w_gate_up, b.feed_forward.w_down):
+            w.drop_packed()
+    assert not any(held())
+    eng.close(s)
+    s = eng.open()
+    eng.step([(s, toks[:290], [])])
+    again = eng.step([(s, [toks[290]], [0])])
+    assert torch.equal(first, again) and all(held())
