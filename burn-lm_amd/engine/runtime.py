@@ -42,6 +42,14 @@ MFMA_SKINNY_MAX_ROWS = 64
 RING_GROUP_K = 2048
 # The shortest K a group keeps when a short K is cut for more blocks.
 RING_MIN_GROUP_K = 512
+# 65 to 256 rows: the longest K at which the row-ring product with a block for every 64 rows still beats the
+# library's and the matrix-core kernel's planes (measured: ahead at 1536, 2048 and 2560, behind at 3072 and 4096).
+RING_MID_K = 2560
+# The longest K at which the fused q/k/v projection on the row ring beats the library's product followed by the
+# rotation kernel (ahead at 5120 and below, 20-29 % behind at 8192).
+RING_QKV_K = 6144
+# The shortest K a group of the matrix-core kernel's partial planes keeps.
+MFMA_MIN_GROUP_K = 768
 # Rows for which the fused gate/up product is used when it is switched on (below, the library is
 # ahead by far; above, its better rate on long runs of tiles has made up for the extra pass).
 FUSED_GATE_UP_ROWS = (192, 4096)
@@ -52,12 +60,14 @@ def rows_plan(N, K, compute_units):
     planes (ops.gemm_rows).  A group spans about RING_GROUP_K of K (measured at the 1B, 3B and 8B layer
     shapes: shorter groups write more planes than they gain, longer ones leave compute units
     idle); 32 columns per block where that gives at most one block per compute unit, else 64;
-    and a short K is cut further, down to RING_MIN_GROUP_K, until three quarters of the units have a block."""
+    and a short K is cut further, down to RING_MIN_GROUP_K, while the blocks still all run at once (a
+    second, partial round costs more than the shorter walk along K gains: width 2560, 64 rows, two
+    groups 6.8 us, four groups 8.8)."""
     groups = 1
     while groups < 8 and K // (groups * 2) >= RING_GROUP_K:
         groups *= 2
     columns = 32 if -(-N // 32) * groups <= compute_units else 64
-    while groups < 8 and K // (groups * 2) >= RING_MIN_GROUP_K and -(-N // columns) * groups * 4 < compute_units * 3:
+    while groups < 8 and K // (groups * 2) >= RING_MIN_GROUP_K and -(-N // columns) * groups * 2 <= compute_units:
         groups *= 2
     return groups, columns
 
@@ -149,7 +159,10 @@ class Runtime:
         gated_linear(); its packed copy pairs each gate row with its up row."""
         w = w.contiguous()
         N, K = w.shape
-        packable = w.dtype == torch.bfloat16 and ops.gemv_mfma_supported(1, N, K) and (not gated or N % 16 == 0)
+        # (a K too long for one group of the skinny product still runs in several, as partial planes; the gated
+        # product has no planes)
+        packable = w.dtype == torch.bfloat16 and K % 8 == 0 and K >= 8 and (
+            ops.gemv_mfma_supported(1, N, K) and N % 16 == 0 if gated else True)
         return LinearWeight(w, packable, gated)
 
     def k_groups(self, N, K, M=1):
@@ -180,7 +193,7 @@ class Runtime:
         Measured per call at the 1B shape against the library's product: 6.8-7.2 against 9.8 us at 65-128
         rows, 8.0 against 10.8 at 192, 8.9 against 11.1 at 256; at K = 3072 and 4096 (3B, 8B) equal or
         behind, hence the bound on K."""
-        if not (self.rows_ring and MFMA_SKINNY_MAX_ROWS < M <= 256 and K <= RING_GROUP_K):
+        if not (self.rows_ring and MFMA_SKINNY_MAX_ROWS < M <= 256 and K <= RING_MID_K):
             return 0
         blocks = self.rows_ring_blocks(M, N)
         if blocks > self.compute_units:
@@ -195,19 +208,19 @@ class Runtime:
         """Which fused projection geometry a position encoding should build on for M rows of width K and
         N = all query, key and value columns, or None (project with linear(), then encode).  The encoding
         only has to check that its own kernel exists for the answer; the thresholds live here.
-        17 to 64 rows: the row-ring geometry from 33 rows on, and from 17 where K is beyond RING_GROUP_K
-        (measured over whole decode steps against the packed kernel with two to four row tiles: 1.4 %
-        faster at batch 64 of the 1B shape and 1.3 % slower at batch 17-32, hence the rule; 2-6 % faster at
-        every batch from 17 to 64 of the 3B and 8B shapes); 33 to 64 rows as two blocks of 32 while both
-        sets run at once (1B shape: 7.8-8.2 against 9.3-9.8 us).  65 to 256 rows: a block for every 64
+        17 to 64 rows: the row-ring geometry (per call against the packed kernel with two to four row tiles,
+        us: width 1536 at 24 / 32 rows 6.4 / 6.7 against 7.4 / 8.0; width 2048 at 17 / 24 / 32 rows 7.0 / 7.0 / 7.4
+        against 7.2 / 7.8 / 8.6; width 3072 8.5-9.2 against 16.5-21.8; whole decode steps at batch 17 to 64 of
+        the 3B and 8B shapes 2-6 % faster); 33 to 64 rows as two blocks of 32 while both sets run at once (1B
+        shape: 7.8-8.2 against 9.3-9.8 us).  65 to 256 rows: a block for every 64
         rows, 32 columns per block while those blocks all run at once, else 64 while there are at most one
         and a half per compute unit (per layer against the library's product and the rotation kernel: 1B
         shape 10 against 14-16 us at 65-128 rows, 13.3 against 21 at 192, 13.6 against 16 at 256; 3B 16-17
         against 18-27 at 65-192, 28.5 against 33 at 256; 8B 21-24.5 against 28-31 at 65-128, 36 against 39
         at 192, 38.5 against 46 at 256).  Up to 16 rows, and whenever the row-ring kernel is not to be
         had: the packed geometry."""
-        if self.rows_ring:
-            if 16 < M <= MFMA_SKINNY_MAX_ROWS and (M > 32 or K > RING_GROUP_K):
+        if self.rows_ring and K <= RING_QKV_K:
+            if 16 < M <= MFMA_SKINNY_MAX_ROWS:
                 halves = M > 32 and self.rows_ring_blocks(64, N) * 2 <= self.compute_units
                 return FusedProjectionPlan("rows", 32, 32 if halves else 64)
             if MFMA_SKINNY_MAX_ROWS < M <= 256:
@@ -219,19 +232,29 @@ class Runtime:
             return FusedProjectionPlan("packed")
         return None
 
+    def mid_planes_plan(self, M, N, K):
+        """More than 32 rows, narrow output, long K (the down projection, the output projection of wide models): the
+        product as partial planes of the matrix-core kernel over groups of K (the block's next norm sums the
+        planes).  -> (groups, tile), or (0, None) for the library's product.  Of the 128x128 and 128x64 tiles
+        with eight, four or two groups of at least MFMA_MIN_GROUP_K, the one whose blocks come closest to one
+        per compute unit without exceeding that, the larger tile on a tie, and nothing if even that leaves half the
+        units idle.  Measured at 128 rows (us, chosen / library): widths 2560, 5120 and 8192 with an inner size of
+        11008: 22.4 / 57.6, 37.5 / 60.9, 45.4 / 67.2; width 1536: 14.5 / 21.9; a tie (width 2560, 160 blocks): 128x128
+        in eight groups 22.4, 128x64 in four 25.9.  Over whole prompts of 65 to 128 tokens: 6 % faster at the
+        Llama-3.2-1B shape, 19 % at 3B, 21 % at 8B (the library's product of few rows and a long K streams the
+        weights at a quarter of the memory rate); 2-5 % up to 512 tokens, where two groups still fit; equal beyond."""
+        best = (0, None, 0)
+        for tile, tn in (((128, 128, 4), 128), ((128, 64, 6), 64)):
+            tiles = -(-M // 128) * -(-N // tn)
+            for g in (8, 4, 2):
+                blocks = tiles * g
+                if K // g >= MFMA_MIN_GROUP_K and self.compute_units // 2 <= blocks <= self.compute_units and blocks > best[2]:
+                    best = (g, tile, blocks)
+        return best[0], best[1]
+
     def mid_k_groups(self, M, N, K):
-        """Short prompts, narrow output, long K (the down projection): the product as partial planes
-        of 128x64 tiles over groups of K (the block's next norm sums the planes), when eight, four
-        or two groups of at least 768 give every compute unit at most one block and half of them
-        one; 0 otherwise (the library's product).  Measured over whole prompts of 65 to 128 tokens:
-        6 % faster at the Llama-3.2-1B shape, 19 % at 3B, 21 % at 8B (the library's product of few
-        rows and a long K streams the weights at a quarter of the memory rate); 2-5 % up to 512
-        tokens, where two groups still fit; equal beyond."""
-        tiles = -(-M // 128) * -(-N // 64)
-        for g in (8, 4, 2):
-            if K // g >= 768 and self.compute_units // 2 <= tiles * g <= self.compute_units:
-                return g
-        return 0
+        """Groups of K of mid_planes_plan (0: the library's product)."""
+        return self.mid_planes_plan(M, N, K)[0]
 
     def linear(self, x, w, out_dtype=None, out=None, partials=False):
         """x [M,K] @ w[N,K]^T -> [M,N] in out_dtype (default: the activation dtype).  w: a
@@ -245,9 +268,10 @@ class Runtime:
         M, K = x.shape
         N = w.shape[0]
         out_dtype = out_dtype or self.dtype
-        if out is None and not (partials and packable):
-            out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+        planes = partials and out is None       # the result may come as float32 partial planes
         if w.dtype == torch.float32 or x.dtype == torch.float32:
+            if out is None:
+                out = torch.empty(M, N, dtype=out_dtype, device=x.device)
             if M <= SKINNY_MAX_ROWS and x.dtype == w.dtype == out_dtype == torch.float32 and K % 8 == 0 \
                     and x.stride(0) % 8 == 0:
                 return ops.gemv_skinny(x, w, out)
@@ -255,28 +279,36 @@ class Runtime:
         aligned = K % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
         if (M > MFMA_SKINNY_MAX_ROWS and aligned and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1
                 and w.is_contiguous() and out_dtype == torch.bfloat16):
-            groups = self.mid_rows_ring(M, N, K, planes=partials and out is None)
+            groups = self.mid_rows_ring(M, N, K, planes=planes)
             if groups > 1:
                 return ops.gemm_rows(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), columns=32)
             if groups == 1:
                 return ops.gemm_rows(x, w, out if out is not None else torch.empty(M, N, dtype=out_dtype, device=x.device),
                                      columns=32)
-        if (partials and out is None and self.mid_partials and M > self.skinny_planes_rows and aligned
-                and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()):
-            groups = self.mid_k_groups(M, N, K)
+        plain_bf16 = aligned and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()
+        if planes and self.mid_partials and M > self.skinny_planes_rows and plain_bf16:
+            groups, tile = self.mid_planes_plan(M, N, K)
             if groups:
-                return ops.gemm_mfma(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device),
-                                     tile=(128, 64, 6))
-        if (partials and out is None and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and aligned
-                and (M > 32 or K <= 4096) and x.dtype == w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.is_contiguous()):
+                return ops.gemm_mfma(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), tile=tile)
+        if (planes and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and plain_bf16
+                and (M > 32 or K <= 4096 or -(-N // 32) * 8 <= 3 * self.compute_units)):
             # 17 to 64 rows as partial planes (measured against the packed skinny kernel at the 1B, 3B and 8B
             # shapes: output projection 15-35 % faster at every row count, down projection 25-40 % at K = 8192 of
-            # the 1B width, equal to 10 % at the wider ones from 33 rows on and up to 10 % behind below: left there)
+            # the 1B width, equal to 10 % at the wider ones from 33 rows on).  Up to 32 rows: where K is short or the
+            # output narrow (up to 96 blocks of 32 columns on 256 units: widths 1536 and 2560 with inner sizes of
+            # 6144 and 11008 at 32 rows 6.2-9.3 us against 8.1-12.0); a wide output with a long K stays with the
+            # packed kernel there (equal to 8 % ahead)
             groups, columns = self.rows_plan(N, K)
+            if M > 32 and self.mid_partials and -(-N // columns) * groups > self.compute_units:
+                # more blocks than compute units even with 64 columns each (a long K under a wide output): the
+                # matrix-core kernel's planes where they fill the chip (width 8192, K = 11008, 64 rows: 42.6 against 46.3 us)
+                g2, tile = self.mid_planes_plan(M, N, K)
+                if g2:
+                    return ops.gemm_mfma(x, w, torch.empty(g2, M, N, dtype=torch.float32, device=x.device), tile=tile)
             if groups > 1:
                 return ops.gemm_rows(x, w, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), columns=columns)
         if packable and M <= MFMA_SKINNY_MAX_ROWS and aligned:
-            if partials and out is None:
+            if planes:
                 groups = self.k_groups(N, K, M)
                 if groups > 1:
                     return ops.gemv_mfma(x, holder.packed, torch.empty(groups, M, N, dtype=torch.float32, device=x.device), K)
@@ -310,6 +342,17 @@ class Runtime:
         # float32 logits from bfloat16 operands with many rows: own kernel (float accumulation)
         return ops.gemm_tiled(x, w, out)
 
+    def _gated_by_library(self, M, K, inner):
+        """17 to 64 rows of a gated product that are better left to the library's product and the gating kernel:
+        from 33 rows on where K is beyond 4096 (measured at widths 5120 and 8192 with inner sizes of 6144 to 28672:
+        6-23 % ahead of the row ring, whose blocks each walk all of K, and of the matrix-core tiles of short
+        prompts) or the row ring would take more than two rounds of blocks (width 2560 with an inner size of
+        28672: 66.9 against 74.6 us); up to 32 rows where K is beyond what the packed kernel takes and the row
+        ring's blocks do not all run at once (width 5120, inner size 11008: 51.6 against 57.7)."""
+        if M > 32:
+            return K > 4096 or -(-inner // 32) > 2 * self.compute_units
+        return K > 4096 and -(-inner // 32) > self.compute_units
+
     def gated_linear(self, x, w):
         """silu(x gate^T) * (x up^T) for w = [gate rows; up rows] ([2I, K]) -> [M, I].  With few rows
         in bfloat16 the gating is fused into the product (weight(w, gated=True) pairs the rows for
@@ -319,18 +362,21 @@ class Runtime:
         plain = w.w if isinstance(w, LinearWeight) else w
         fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
-        if fusable and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and (
-                M > 32 or (K > RING_GROUP_K and -(-inner // 32) <= self.compute_units)):
+        by_library = 16 < M <= MFMA_SKINNY_MAX_ROWS and self._gated_by_library(M, K, inner)
+        if fusable and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and not by_library and (
+                M > 32 or -(-inner // 32) <= self.compute_units * (2 if K <= RING_GROUP_K else 1)):
             # 33 to 64 rows (measured against the packed skinny kernel: 4-15 % faster at the 1B and 3B shapes, and
             # at wider ones in place of the library's product, which the packed kernel's registers leave them to);
-            # from 17 rows on where K is above 2048 and the blocks come in one round (3B: 10-15 %)
+            # from 17 rows on where the blocks come in one round, or in two where K is short (us at 17 / 24 / 32
+            # rows against the packed kernel: width 2048, inner 8192: 14.0 / 14.3 / 14.3 against 16.4 / 17.7 / 18.2;
+            # width 1536: 11.8 / 11.9 / 12.0 against 13.3 / 14.1 / 14.6; 3B: 10-15 %)
             return ops.gemm_rows(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True)
-        if (isinstance(w, LinearWeight) and w.packable and w.gated and x.dtype == torch.bfloat16
+        if (isinstance(w, LinearWeight) and w.packable and w.gated and x.dtype == torch.bfloat16 and not by_library
                 and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
             return ops.gemv_mfma(x, w.packed, out, K, gated=True)
-        if fusable and self.fused_gate_up_measured:
+        if fusable and self.fused_gate_up_measured and M > MFMA_SKINNY_MAX_ROWS:
             # Short prompts: when all tiles of the product run at once (one block per compute unit,
             # most of the units busy), the fused kernel with a deep ring of stages streams the
             # weights faster than the library product and the gating pass after it (measured at
