@@ -48,8 +48,11 @@ RING_MID_K = 2560
 # The longest K at which the fused q/k/v projection on the row ring beats the library's product followed by the
 # rotation kernel (ahead at 5120 and below, 20-29 % behind at 8192).
 RING_QKV_K = 6144
-# The shortest K a group of the matrix-core kernel's partial planes keeps.
+# The shortest K a group of the matrix-core kernel's partial planes keeps, and the most rows for which a product
+# comes as such planes (every group writes a float32 plane of rows x columns that the next norm reads back: measured
+# over whole prompts, 2-5 % faster up to 512 tokens and equal beyond).
 MFMA_MIN_GROUP_K = 768
+MID_PLANES_MAX_ROWS = 512
 # Rows for which the fused gate/up product is used when it is switched on (below, the library is
 # ahead by far; above, its better rate on long runs of tiles has made up for the extra pass).
 FUSED_GATE_UP_ROWS = (192, 4096)
@@ -244,6 +247,8 @@ class Runtime:
         Llama-3.2-1B shape, 19 % at 3B, 21 % at 8B (the library's product of few rows and a long K streams the
         weights at a quarter of the memory rate); 2-5 % up to 512 tokens, where two groups still fit; equal beyond."""
         best = (0, None, 0)
+        if M > MID_PLANES_MAX_ROWS:
+            return 0, None
         for tile, tn in (((128, 128, 4), 128), ((128, 64, 6), 64)):
             tiles = -(-M // 128) * -(-N // tn)
             for g in (8, 4, 2):

@@ -25,25 +25,25 @@ from helpers import TINIES, make_folder, random_tokens, rel_err
 pytestmark = pytest.mark.gpu
 
 # (q/k rounded before the rotation, gate/up rounded before the gating, output projection rounded, down
-#  projection rounded) for steps of up to 32 rows, of up to 64, of up to 128, of up to 256, and beyond; then
+#  projection rounded) for steps of up to 16 rows, of up to 32, of up to 64, of up to 128, of up to 256, and beyond; then
 #  whether the attention rounds its probabilities (the matrix-core kernels do, the generic one, which takes
 #  head sizes that are no multiple of 16, does not).
 #  A: width 64.  Few rows: projection, rotation and cache write are one kernel, the gating is the
 #     product's epilogue.  Up to 256 rows projection, rotation and cache write stay one kernel (these
 #     models have few columns); beyond, every product is the library's and is rounded.
-#  B: head size 24: up to 32 rows the rotation is a kernel of its own, so q and k are rounded before it; from
-#     33 to 256 rows projection, rotation and cache write are one kernel again (the one that takes any even
+#  B: head size 24: up to 16 rows the rotation is a kernel of its own, so q and k are rounded before it; from
+#     17 to 256 rows projection, rotation and cache write are one kernel again (the one that takes any even
 #     head size).
 #  C: width 512, inner 1408: with few rows the down projection comes as unrounded partial sums over
 #     two halves of its long inner dimension, and so it does from 65 to 256 rows; from 129 rows on the
 #     gate/up product is the fused matrix-core kernel again (its tiles then fill enough of the chip).
 STYLES = {
-    "A": (((False, False, True, True), (False, False, True, True), (False, True, True, True), (False, True, True, True),
-           (True, True, True, True)), True),
-    "B": (((True, False, True, True), (False, False, True, True), (False, True, True, True), (False, True, True, True),
-           (True, True, True, True)), False),
-    "C": (((False, False, True, False), (False, False, True, False), (False, True, True, False), (False, False, True, False),
-           (True, False, True, True)), True),
+    "A": (((False, False, True, True), (False, False, True, True), (False, False, True, True), (False, True, True, True),
+           (False, True, True, True), (True, True, True, True)), True),
+    "B": (((True, False, True, True), (False, False, True, True), (False, False, True, True), (False, True, True, True),
+           (False, True, True, True), (True, True, True, True)), False),
+    "C": (((False, False, True, False), (False, False, True, False), (False, False, True, False), (False, True, True, False),
+           (False, False, True, False), (True, False, True, True)), True),
 }
 LENGTHS = [1, 2, 7, 16, 33, 64, 65, 100, 150, 300]
 # least share of rows that agree to 1e-5, and largest row error allowed (of the row's largest logit)
@@ -52,7 +52,7 @@ LIMITS = {"A": (0.5, 1.2e-2), "B": (0.1, 1.5e-2), "C": (0.0, 1.5e-2)}
 
 def style_for(name, rows):
     styles, _ = STYLES[name]
-    return styles[0 if rows <= 32 else 1 if rows <= 64 else 2 if rows <= 128 else 3 if rows <= 256 else 4]
+    return styles[0 if rows <= 16 else 1 if rows <= 32 else 2 if rows <= 64 else 3 if rows <= 128 else 4 if rows <= 256 else 5]
 
 
 def rounding_for(name, step_rows_of_token, decoded):
