@@ -746,11 +746,18 @@ extern "C" int blm_attn_decode_supported(int act_dtype, int hd, int page_size) {
   return (act_dtype == BLM_BF16 && page_size == AM_PAGE && hd_ok(hd, 128)) ? 1 : 0;
 }
 
+// Blocks that the 32-query form would launch (0 if the head size has no such form).
+extern "C" long long blm_attn_prefill_blocks32(int n_seqs, int max_new, int nh, int nkv, int hd) {
+  if (hd % 32 != 0 || hd > 128 || nkv <= 0 || nh % nkv != 0) return 0;
+  const long long units32 = (long long)(nh / nkv) * ((max_new + 31) / 32);
+  return (units32 + AM_WAVES - 1) / AM_WAVES * nkv * n_seqs;
+}
+
 extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out, int act_dtype,
                                      const int* positions, const int* cu_seqlens, const int* block_table,
                                      int table_width, const void* kcache, const void* vcache, int page_size,
                                      int n_seqs, int max_new, int nh, int nkv, int hd, float scale, int window,
-                                     hipStream_t stream) {
+                                     int queries, hipStream_t stream) {
   BLM_REQUIRE(n_seqs > 0 && n_seqs <= 65535 && max_new > 0 && nh > 0 && nkv > 0 && nkv <= 65535 && nh % nkv == 0,
               "attn_prefill_mfma: bad sizes seqs=%d max_new=%d heads=%d kv_heads=%d", n_seqs, max_new, nh, nkv);
   BLM_REQUIRE(blm_attn_prefill_mfma_supported(act_dtype, hd, page_size),
@@ -761,22 +768,16 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
   BLM_REQUIRE(q_row_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0,
               "attn_prefill_mfma: q rows must be 16-byte aligned");
   const int G = nh / nkv;
-  // 32 queries per wavefront (half the shared-memory reads per matrix instruction) once its blocks are
-  // three times the compute units: with fewer, all blocks run at once and the step lasts as long as
-  // the block with the most pages, whose pages take longer one after another than those of the
-  // 16-query form (measured at 32 heads of 64: 2,048 tokens 49.5 against 43.6 us, 4,096 tokens 108
-  // against 137 us; 24 heads of 128: 68 against 58 us, 141 against 187 us).
-  // BURN_LM_AMD_PREFILL_TILE=16 or 32 forces one form (for measurements).
+  // queries: 16 or 32 query rows per wavefront.  32 (head sizes 32, 64, 96, 128) halves the shared-memory
+  // reads per matrix instruction and is ahead once its blocks are three times the compute units: with fewer,
+  // all blocks run at once and the step lasts as long as the block with the most pages, whose pages take
+  // longer one after another than those of the 16-query form (measured at 32 heads of 64: 2,048 tokens 49.5
+  // against 43.6 us, 4,096 tokens 108 against 137 us; 24 heads of 128: 68 against 58 us, 141 against 187 us).
+  // The caller chooses (blm_attn_prefill_blocks32 gives it the number of blocks to compare).
+  BLM_REQUIRE(queries == 16 || (queries == 32 && hd % 32 == 0 && hd <= 128),
+              "attn_prefill_mfma: %d queries per wavefront with head_dim %d (16, or 32 with head sizes 32, 64, 96, 128)", queries, hd);
   const long long units32 = (long long)G * ((max_new + 31) / 32);
-  const long long blocks32 = (units32 + AM_WAVES - 1) / AM_WAVES * nkv * n_seqs;
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
-    else cus = 256;
-  }
-  const char* forced = getenv("BURN_LM_AMD_PREFILL_TILE");
-  const bool wide = forced ? forced[0] == '3' : blocks32 >= 3LL * cus;
+  const bool wide = queries == 32;
   if (hd % 32 == 0 && hd <= 128 && wide) {
     dim3 grid32((unsigned)((units32 + AM_WAVES - 1) / AM_WAVES), nkv, n_seqs), block32(AM_WAVES * BLM_WAVE);
 #define BLM_AP32(HD)                                                                                             \

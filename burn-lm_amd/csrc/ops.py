@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 _lib = None
 _lock = threading.Lock()
 
@@ -40,7 +40,7 @@ _SIGNATURES = {
     "blm_attn_prefill_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_attn_prefill_mfma": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                               _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                              _c_int, _c_void_p],
+                              _c_int, _c_int, _c_void_p],
     "blm_gemm_tiled": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_void_p],
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
@@ -91,6 +91,8 @@ def library():
                     fn.restype = _c_int
                 lib.blm_sample_scratch_bytes.argtypes = [_c_int, _c_int]
                 lib.blm_sample_scratch_bytes.restype = ctypes.c_longlong
+                lib.blm_attn_prefill_blocks32.argtypes = [_c_int] * 5
+                lib.blm_attn_prefill_blocks32.restype = ctypes.c_longlong
                 _lib = lib
     return _lib
 
@@ -313,11 +315,18 @@ def attn_prefill_mfma_supported(dtype, hd, page_size=64):
         library().blm_attn_prefill_mfma_supported(DTYPE_CODE[dtype], int(hd), int(page_size)))
 
 
+def attn_prefill_queries(n_seqs, max_new, nh, nkv, hd, compute_units):
+    """Query rows per wavefront that attn_prefill_mfma should take for a step: 32 (half the shared-memory
+    reads per matrix instruction) once that form's blocks are three times the compute units, else 16."""
+    blocks32 = library().blm_attn_prefill_blocks32(int(n_seqs), int(max_new), int(nh), int(nkv), int(hd))
+    return 32 if blocks32 >= 3 * int(compute_units) else 16
+
+
 def attn_prefill_mfma(q, q_row_stride, out, positions, cu_seqlens, block_table, kcache, vcache, page_size,
-                      n_seqs, max_new, nh, nkv, hd, scale, window=0):
+                      n_seqs, max_new, nh, nkv, hd, scale, window=0, queries=16):
     """Causal attention of packed sequences over their cached keys on the matrix cores (bfloat16).
     Rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out belong to sequence b; max_new is the most
-    rows any sequence has."""
+    rows any sequence has.  queries: 16 or 32 query rows per wavefront (attn_prefill_queries chooses)."""
     _gpu(q, out, positions, cu_seqlens, block_table, kcache, vcache)
     T = out.shape[0]
     _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
@@ -331,7 +340,7 @@ def attn_prefill_mfma(q, q_row_stride, out, positions, cu_seqlens, block_table, 
         raise KernelError("attn_prefill_mfma: the page table has fewer rows than there are sequences")
     _call("blm_attn_prefill_mfma", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           cu_seqlens.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
-          page_size, int(n_seqs), int(max_new), nh, nkv, hd, float(scale), int(window), _stream())
+          page_size, int(n_seqs), int(max_new), nh, nkv, hd, float(scale), int(window), int(queries), _stream())
     return out
 
 

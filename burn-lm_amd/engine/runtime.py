@@ -148,6 +148,8 @@ class Runtime:
         # from 33 rows on those are 1-2 % ahead at some shapes and as much behind at others)
         self.skinny_gated_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_GATED_ROWS", MFMA_SKINNY_MAX_ROWS))
         self.skinny_planes_rows = int(os.environ.get("BURN_LM_AMD_SKINNY_PLANES_ROWS", MFMA_SKINNY_MAX_ROWS))
+        # "16" or "32": query rows per wavefront of the prefill attention, whatever the step (for measurements)
+        self.prefill_queries = int(os.environ.get("BURN_LM_AMD_PREFILL_TILE", "0") or 0)
         # "0": 17 to 64 rows stay on the packed skinny kernels (for measurements)
         self.rows_ring = os.environ.get("BURN_LM_AMD_ROWS_RING") != "0"
 

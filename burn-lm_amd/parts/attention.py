@@ -119,8 +119,12 @@ class Attention(Mixer):
             rt.ops.attn_decode(qkv, qkv.shape[1], out, step.positions, step.token_seq, table, view.k, view.v,
                                view.page_size, nh, nkv, hd, self.scale, self.window, n_splits)
         elif aligned and rt.ops.attn_prefill_mfma_supported(rt.dtype, hd, view.page_size):
+            queries = rt.prefill_queries or rt.ops.attn_prefill_queries(step.n_seqs, step.max_new, nh, nkv, hd, rt.compute_units)
+            if queries == 32 and (hd % 32 or hd > 128):
+                queries = 16
             rt.ops.attn_prefill_mfma(qkv, qkv.shape[1], out, step.positions, step.cu_seqlens, table, view.k, view.v,
-                                     view.page_size, step.n_seqs, step.max_new, nh, nkv, hd, self.scale, self.window)
+                                     view.page_size, step.n_seqs, step.max_new, nh, nkv, hd, self.scale, self.window,
+                                     queries=queries)
         else:
             # the generic kernel has one wavefront per (token, head); with few tokens over long key
             # ranges the ranges are cut so that the whole chip has work

@@ -374,12 +374,21 @@ def test_attn_prefill_mfma(ops, nh, nkv, hd, window, tile, monkeypatch):
     """The matrix-core prefill kernel on packed sequences: a whole prompt from position 0 (not a
     multiple of 16 long), a chunk that continues a long past, one token on top of a past that ends at
     a page edge, a single first token; a far key stands out; unused places hold NaN.  Both forms: 16
-    queries per wavefront, and 32 (head sizes that are multiples of 32; the entry point picks it by
-    itself only for steps of many blocks, so it is forced here)."""
-    if tile == "32" and hd % 32:
-        pytest.skip("the 32-query form takes head sizes that are multiples of 32")
-    monkeypatch.setenv("BURN_LM_AMD_PREFILL_TILE", tile)
+    queries per wavefront, and 32 (head sizes that are multiples of 32; a caller picks it only for steps
+    of many blocks, so it is asked for here)."""
+    from burn_lm_amd.csrc.ops import KernelError
+    if tile == "32" and (hd % 32 or hd > 128):
+        with pytest.raises(KernelError, match="32 queries per wavefront"):
+            ops.attn_prefill_mfma(torch.zeros(16, (nh + 2 * nkv) * hd, dtype=torch.bfloat16, device="cuda"), (nh + 2 * nkv) * hd,
+                                  torch.zeros(16, nh * hd, dtype=torch.bfloat16, device="cuda"), torch.arange(16, dtype=torch.int32, device="cuda"),
+                                  torch.tensor([0, 16], dtype=torch.int32, device="cuda"), torch.zeros(1, 1, dtype=torch.int32, device="cuda"),
+                                  torch.zeros(1, nkv, 64, hd, dtype=torch.bfloat16, device="cuda"),
+                                  torch.zeros(1, nkv, hd, 64, dtype=torch.bfloat16, device="cuda"), 64, 1, 16, nh, nkv, hd, 0.1, 0, queries=32)
+        pytest.skip("the 32-query form takes head sizes 32, 64, 96 and 128 (and says so)")
     assert ops.attn_prefill_mfma_supported(torch.bfloat16, hd) and not ops.attn_prefill_mfma_supported(torch.float32, hd)
+    # which form a step takes by itself: 32 queries once that form's blocks are three times the compute units
+    assert ops.attn_prefill_queries(1, 2048, 32, 8, 64, 256) == 16 and ops.attn_prefill_queries(1, 4096, 32, 8, 64, 256) == 32
+    assert ops.attn_prefill_queries(4, 2048, 32, 8, 64, 256) == 32 and ops.attn_prefill_queries(1, 65536, 6, 1, 24, 256) == 16
     g = torch.Generator().manual_seed(15)
     lens = [150, 333, 65, 1, 40]             # length of each sequence after the step
     new = [150, 70, 1, 1, 33]                # rows this step brings
@@ -394,7 +403,7 @@ def test_attn_prefill_mfma(ops, nh, nkv, hd, window, tile, monkeypatch):
     scale = 1.0 / math.sqrt(hd)
     ops.attn_prefill_mfma(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
                           dev(torch.tensor(cu, dtype=torch.int32)), dev(table), dev(kc), dev(vc), 64, len(lens), max(new),
-                          nh, nkv, hd, scale, window)
+                          nh, nkv, hd, scale, window, queries=int(tile))
     got = out.cpu().double().reshape(T, nh, hd)
     assert torch.isfinite(got).all(), "a key beyond a sequence's length was read"
     for b in range(len(lens)):

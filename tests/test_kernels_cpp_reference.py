@@ -121,9 +121,9 @@ def test_attention(ops, ref, kind, nh, nkv, hd, window, monkeypatch):
     """The generic kernel (float32 and bfloat16), the matrix-core decode kernel with cut key ranges and the
     matrix-core prefill kernels (16 and 32 queries per wavefront): one C++ loop nest is the reference of all."""
     g = torch.Generator().manual_seed(33)
-    if kind == "prefill32":     # the form with 32 queries per wavefront, which small steps do not pick by themselves
-        monkeypatch.setenv("BURN_LM_AMD_PREFILL_TILE", "32")
-        kind = "prefill"
+    queries = 16
+    if kind == "prefill32":     # the form with 32 queries per wavefront, which a caller picks for steps of many blocks only
+        queries, kind = 32, "prefill"
     dtype = torch.float32 if kind == "generic32" else torch.bfloat16
     page, scale = 64, 1.0 / math.sqrt(hd)
     lens = [200, 65, 7]
@@ -152,7 +152,8 @@ def test_attention(ops, ref, kind, nh, nkv, hd, window, monkeypatch):
         ops.attn_decode(*args, dev(seq), dev(table), dev(k.to(dtype)), dev(v.to(dtype)), page, nh, nkv, hd, scale, window, 2)
     else:
         assert ops.attn_prefill_mfma_supported(dtype, hd, page)
-        ops.attn_prefill_mfma(*args, dev(cu), dev(table), dev(k.to(dtype)), dev(v.to(dtype)), page, len(lens), max(new), nh, nkv, hd, scale, window)
+        ops.attn_prefill_mfma(*args, dev(cu), dev(table), dev(k.to(dtype)), dev(v.to(dtype)), page, len(lens), max(new), nh, nkv, hd, scale, window,
+                              queries=queries)
     assert rel(out.float().cpu().numpy(), want) <= (1e-5 if dtype == torch.float32 else 1.2e-2)
 
 
