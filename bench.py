@@ -376,15 +376,19 @@ def main():
     layers = args.layers or full_layers
     config["num_hidden_layers"] = layers
     biggest = max(args.batch, 1 if args.no_points else 64)
+    from burn_lm_amd.csrc import build as _build
     if args.profile:
-        from burn_lm_amd.csrc import build as _build
         if _build.under_profiler() and not (_build.is_current() and _build.host_is_current()):
             print("bench.py: the kernel libraries do not match their sources; build them before profiling "
                   "(python -c 'import __graft_entry__ as g; g.build()')")
             sys.exit(2)
-    say("building the engine (random weights)")
+    # under a profiler every launch is slow (a counter run was seen to take two minutes for the 12,727 small
+    # launches of the counter-based weight stream alone): the weights then come from one launch per tensor
+    quick = bool(args.profile) and _build.under_profiler()
+    say("building the engine (random weights" + (", one launch per tensor)" if quick else ")"))
     engine = random_engine(config, seed=0, dtype=args.dtype, max_tokens=biggest * args.context,
-                           max_seqs=biggest, max_context=args.context, graphs=args.profile != "decode-loop")
+                           max_seqs=biggest, max_context=args.context, graphs=args.profile != "decode-loop",
+                           quick_weights=quick)
     say("engine built")
     cfg = engine.config
     page_size = engine.cache.page_size

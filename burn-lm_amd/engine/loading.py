@@ -83,7 +83,8 @@ def load_engine(folder, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_co
 
 
 def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_seqs=None, max_context=None,
-                  device="cuda:0", std=0.02, norm_jitter=0.0, page_size=64, graphs=True, stored_dtype=torch.bfloat16):
+                  device="cuda:0", std=0.02, norm_jitter=0.0, page_size=64, graphs=True, stored_dtype=torch.bfloat16,
+                  quick_weights=False):
     """Engine with seeded random weights made directly on the GPU: the very tensors that the
     random-weights mode writes into a folder for this configuration, seed and stored type (every
     value is a function of seed, tensor name and element index), checked and kept by the loader's
@@ -93,7 +94,8 @@ def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_s
     arch = registry.architecture_of(config)
     cfg = arch.read_config(config)
     rt = Runtime(dtype=dtype, device=device)
-    made = dict(random_tensors(arch, cfg, seed, std=std, norm_jitter=norm_jitter, dtype=stored_dtype, device=rt.device))
+    made = dict(random_tensors(arch, cfg, seed, std=std, norm_jitter=norm_jitter, dtype=stored_dtype, device=rt.device,
+                               quick=quick_weights))
     plan = arch.plan(cfg, set(made))
     model = Model(plan)
     tensors = loader.place(f"the random checkpoint of {arch.name}", made, model.tensor_specs(), dtype, rt.device,

@@ -118,9 +118,12 @@ def _initialiser(init):
 
 
 def make_tensor(name, shape, init, seed, std=0.02, norm_jitter=0.0, dtype=torch.bfloat16, device="cpu",
-                override=None):
+                override=None, quick=False):
     """One tensor of a fresh checkpoint.  override: a Range that replaces the initialiser of every
-    floating tensor (the reference's fixture), keeping the tensor's layout."""
+    floating tensor (the reference's fixture), keeping the tensor's layout.  quick: normal deviates from the
+    device's own generator in one launch per tensor instead of the counter-based stream (not reproducible
+    across devices or in a folder; for runs under a profiler, where each of the stream's thousands of small
+    launches is slow)."""
     init = _initialiser(init)
     shape = tuple(int(s) for s in shape)
     n = 1
@@ -150,6 +153,11 @@ def make_tensor(name, shape, init, seed, std=0.02, norm_jitter=0.0, dtype=torch.
     else:
         raise ValueError(f"random weights: {name} has the initialiser {init!r}, which is none of "
                          f"Normal, Ones, Range, IntegerTable or a role name")
+    if quick:
+        g = torch.Generator(device=device)
+        g.manual_seed(tensor_key(seed, name) & 0x7FFFFFFF)
+        z = torch.randn(shape, dtype=torch.float32, device=device, generator=g) * scale
+        return (z + offset if offset else z).to(dtype)
     out = torch.empty(n, dtype=dtype, device=device)
     chunk = CHUNK[torch.device(device).type]
     for a in range(0, n, chunk):
@@ -160,7 +168,7 @@ def make_tensor(name, shape, init, seed, std=0.02, norm_jitter=0.0, dtype=torch.
 
 
 def random_tensors(arch, cfg, seed: int, std: float = 0.02, norm_jitter: float = 0.0,
-                   dtype=torch.bfloat16, device="cpu", init=None, names=None):
+                   dtype=torch.bfloat16, device="cpu", init=None, names=None, quick=False):
     """Yields (name, tensor) in checkpoint order.  init: a Range for every floating tensor instead of
     the architecture's initialisers.  names: passed on to architectures that know several checkpoint
     layouts (the Llama architecture: "hf" or "meta")."""
@@ -168,7 +176,7 @@ def random_tensors(arch, cfg, seed: int, std: float = 0.02, norm_jitter: float =
         raise ValueError(f"architecture {arch.name} has no checkpoint_tensors: it cannot make random weights")
     table = arch.checkpoint_tensors(cfg) if names is None else arch.checkpoint_tensors(cfg, names=names)
     for name, (shape, how) in table.items():
-        yield name, make_tensor(name, shape, how, seed, std, norm_jitter, dtype, device, override=init)
+        yield name, make_tensor(name, shape, how, seed, std, norm_jitter, dtype, device, override=init, quick=quick)
 
 
 def write_model_folder(folder: str, config: dict, seed: int = 0, std: float = 0.02, norm_jitter: float = 0.0,
