@@ -426,7 +426,7 @@ def main():
 
     points, workload, kernels, measured = {}, {}, {}, {}
     if not args.no_points:
-        for b in (1, 64):
+        for b in (1, 32, 64):
             s, _ = time_decode(engine, sampler, b, args.context, max(20, args.steps // 2), 4)
             points[f"decode_b{b}"] = round(b / s, 1)
             points[f"decode_b{b}_ms"] = round(s * 1e3, 4)
