@@ -15,7 +15,7 @@ a batch of 8 and a context of 4096 tokens per sequence.  One JSON line is printe
 * ``roofline``: the bytes a decode step has to read (every weight it uses once and the cache of the
   live requests, as the model's own parts count them) / its time, against 8 TB/s; ``prefill``: a
   prompt of 2,048 tokens through the step function, its flops / time against the dense bf16 peak.
-* ``points``: decode at batch 1 and 64 at the same context, with their roofline fractions;
+* ``points``: decode at batch 1, 32 and 64 at the same context, with their roofline fractions;
   ``workload_512_256``: the benchmark's second workload (512-token prompts, 256 generated tokens, at
   batch 1, 8 and 64) as decoded tokens a second over the whole decode phase.
 * ``measured``: what this machine reaches with a kernel that only reads (GB/s) and one that only
