@@ -103,12 +103,15 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
     }
   }
   if (V_LATE) { AM_LOAD_VALUES(); }   // the keys' registers are free now; the values arrive during the softmax
-  float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
+  float mx = blm_max(s[0][0], s[0][1]);
+  mx = blm_max(blm_max(mx, s[0][2]), s[0][3]);
 #pragma unroll
-  for (int t = 1; t < 4; ++t) mx = fmaxf(mx, fmaxf(fmaxf(s[t][0], s[t][1]), fmaxf(s[t][2], s[t][3])));
-  mx = fmaxf(mx, __shfl_xor(mx, 16, BLM_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, BLM_WAVE));
-  const float m_new = fmaxf(m, mx * scale2);
+  for (int t = 1; t < 4; ++t) {
+    mx = blm_max(blm_max(mx, s[t][0]), s[t][1]);
+    mx = blm_max(blm_max(mx, s[t][2]), s[t][3]);
+  }
+  mx = rows_max(mx);
+  const float m_new = blm_max(m, mx * scale2);
   // m = -inf, m_new finite -> 0;  both -inf (nothing visible yet) -> 1, and every p below is 0
   const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
 #pragma unroll
@@ -156,6 +159,31 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
                                                       __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
     }
   }
+}
+
+// The page numbers of a stretch of one sequence's block table, 64 at a time in one register (lane i
+// holds entry base + i).  A loop over pages then takes the next page's number out of the register
+// instead of asking memory for it in front of the loads that need it, once per page.
+struct PageNumbers {
+  const int* table;
+  int width, base, held;
+  __device__ __forceinline__ void load(int first) {
+    base = first;
+    held = table[min(first + (int)(threadIdx.x & (BLM_WAVE - 1)), width - 1)];
+  }
+  // pi: the same in all lanes, not below the last load's first entry
+  __device__ __forceinline__ int at(int pi) {
+    if (pi - base >= BLM_WAVE) load(pi);
+    return __builtin_amdgcn_readlane(held, __builtin_amdgcn_readfirstlane(pi - base));
+  }
+};
+
+// A use of loaded fragments that the compiler cannot move or remove: their loads are issued, and
+// waited for, in front of it.
+template <int N>
+__device__ __forceinline__ void am_pin(uint4* f) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i].x), "+v"(f[i].y), "+v"(f[i].z), "+v"(f[i].w));
 }
 
 template <int HD>
@@ -245,12 +273,13 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const float scale2 = scale * 1.4426950408889634f;
-  const int* bt = block_table + (size_t)b * table_width;
+  PageNumbers pages{block_table + (size_t)b * table_width, table_width, 0, 0};
+  pages.load(blk_first);
 
   u32x4_t kreg[PER_THREAD], vreg[PER_THREAD];
 #define AM_FETCH(pi)                                                                          \
   {                                                                                           \
-    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;                          \
+    const size_t base = ((size_t)pages.at(pi) * nkv + kvh) * AM_PAGE * HD;                    \
     _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                  \
       const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                    \
       if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {                                \
@@ -281,6 +310,11 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
       attn_page<HD, false, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o); \
   }
   AM_FETCH(blk_first);
+  // The query fragments have arrived before the loop starts.  Left alone, the compiler moves their
+  // loads down to the loop's entry, and since its count of outstanding loads is merged over the loop's
+  // paths, it then waits in front of the first product of every page for all loads, the page it has
+  // just asked for included.
+  am_pin<KS>(qf);
   if (NBUF == 2) {
     AM_STAGE(0)
     __syncthreads();
@@ -369,11 +403,15 @@ __device__ __forceinline__ void attn_half32(const bf16* __restrict__ kp, const b
       s[v] = (kj <= qpos && kj >= lo) ? s[v] : -INFINITY;
     }
   }
-  float mx = s[0];
+  float mx = blm_max(s[0], s[1]);
 #pragma unroll
-  for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
-  mx = fmaxf(mx, __shfl_xor(mx, 32, BLM_WAVE));
-  const float m_new = fmaxf(m, mx * scale2);
+  for (int v = 2; v < 16; v += 2) mx = blm_max(blm_max(mx, s[v]), s[v + 1]);
+  {
+    float a, b;
+    blm_swap32(mx, a, b);
+    mx = blm_max(a, b);
+  }
+  const float m_new = blm_max(m, mx * scale2);
   const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
@@ -488,12 +526,13 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[rt][v] = 0.f;
   const float scale2 = scale * 1.4426950408889634f;
-  const int* bt = block_table + (size_t)b * table_width;
+  PageNumbers pages{block_table + (size_t)b * table_width, table_width, 0, 0};
+  pages.load(blk_first);
 
   u32x4_t kreg[PER_THREAD], vreg[PER_THREAD];
 #define AP_FETCH(pi)                                                                          \
   {                                                                                           \
-    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;                          \
+    const size_t base = ((size_t)pages.at(pi) * nkv + kvh) * AM_PAGE * HD;                    \
     _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                  \
       const int jj = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                   \
       if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || jj < CHUNKS) {                               \
@@ -523,6 +562,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
       attn_page32<HD, false, KSTR, VSTR>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o); \
   }
   AP_FETCH(blk_first);
+  am_pin<HD / 16>(qf);   // as in the 16-query kernel
   AP_STAGE(0)
   __syncthreads();
   for (int pi = blk_first; pi <= blk_last; ++pi) {
@@ -535,7 +575,11 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 #undef AP_STAGE
 #undef AP_USE
 #undef AP_FETCH
-  lsum += __shfl_xor(lsum, 32, BLM_WAVE);   // the two lanes of a query hold the sums over their own keys
+  {   // the two lanes of a query hold the sums over their own keys
+    float a, b;
+    blm_swap32(lsum, a, b);
+    lsum = a + b;
+  }
   if (!active || j >= nq) return;
   const float inv = 1.0f / lsum;
   bf16* orow = out + (size_t)row * nh * HD + (size_t)head * HD;
@@ -606,14 +650,15 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
     const int per_split = (last_page - first_page + 1 + n_splits - 1) / n_splits;
     const int p_begin = first_page + split * per_split;
     const int p_end = min(last_page + 1, p_begin + per_split);
-    const int* bt = block_table + (size_t)b * table_width;
+    PageNumbers pages{block_table + (size_t)b * table_width, table_width, 0, 0};
+    if (p_begin < p_end) pages.load(p_begin);
     uint4 qf[KS];
     load_q<HD>(q + (size_t)t * q_row_stride + (size_t)head * HD, qf);
     const float scale2 = scale * 1.4426950408889634f;
     u32x4_t kreg[PER_LANE], vreg[PER_LANE];
 #define AD_FETCH(pi)                                                                          \
   {                                                                                           \
-    const size_t base = ((size_t)bt[pi] * nkv + kvh) * AM_PAGE * HD;                          \
+    const size_t base = ((size_t)pages.at(pi) * nkv + kvh) * AM_PAGE * HD;                    \
     _Pragma("unroll") for (int i = 0; i < PER_LANE; ++i) {                                    \
       const int j = i * BLM_WAVE + lane;                                                      \
       kreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kcache + base + (size_t)j * 8));   \
@@ -632,6 +677,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   }
     int pi = p_begin + wave;
     if (pi < p_end) AD_FETCH(pi);
+    am_pin<KS>(qf);   // arrived before the loop, so that no page's first product waits for the page just asked for
     for (; pi < p_end; pi += AM_WAVES) {
       AD_STAGE()
       if (pi + AM_WAVES < p_end) AD_FETCH(pi + AM_WAVES);   // travels while this page is used

@@ -42,47 +42,94 @@ __device__ __forceinline__ float from_float<float>(float f) { return f; }
 template <>
 __device__ __forceinline__ bf16 from_float<bf16>(float f) { return bf16{f32_to_bf16_bits(f)}; }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = BLM_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, BLM_WAVE);
-  return v;
+// Maximum without the copies that quiet signalling NaNs in front of fmaxf (one instruction per operand
+// that comes out of a matrix instruction or a load); a NaN operand gives NaN.  Chains of it become
+// three-operand instructions.
+__device__ __forceinline__ float blm_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+
+// Exchanges across a wavefront without a trip through shared memory.  Inside a row of 16 lanes a
+// data-parallel move brings the partner's value; between rows the swap instructions of gfx950 do:
+// after blm_swap16(x, a, b), rows 0 and 1 hold a = row 0 of x, b = row 1 of x, rows 2 and 3 hold rows 2
+// and 3; after blm_swap32, lanes l and l + 32 both hold a = x of lane l % 32, b = x of lane l % 32 + 32.
+// Both partners get the same (a, b), so a + b or max(a, b) has the same bits in both.
+template <int CTRL>
+__device__ __forceinline__ float blm_dpp(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, 0xf, 0xf, false));
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = BLM_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, BLM_WAVE));
-  return v;
+#define BLM_DPP_XOR1 0xB1          // quad_perm [1, 0, 3, 2]
+#define BLM_DPP_XOR2 0x4E          // quad_perm [2, 3, 0, 1]
+#define BLM_DPP_HALF_MIRROR 0x141  // lane i of each 8 takes lane 7 - i: the other quad, once quads are uniform
+#define BLM_DPP_MIRROR 0x140       // lane i of each 16 takes lane 15 - i: the other half, once halves are uniform
+__device__ __forceinline__ void blm_swap16(float x, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void blm_swap32(float x, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+// over the four lanes l % 16, l % 16 + 16, + 32, + 48
+__device__ __forceinline__ float rows_max(float v) {
+  float a, b;
+  blm_swap16(v, a, b);
+  v = blm_max(a, b);
+  blm_swap32(v, a, b);
+  return blm_max(a, b);
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  float a, b;
+  blm_swap16(v, a, b);
+  v = a + b;
+  blm_swap32(v, a, b);
+  return a + b;
 }
 
-// Sum over a block of up to 1024 threads; every thread gets the result. `red` holds 17 floats.
+// Sum and maximum over a whole wavefront (all 64 lanes active); every lane gets the same bits.
+__device__ __forceinline__ float wave_sum(float v) {
+  v += blm_dpp<BLM_DPP_XOR1>(v);
+  v += blm_dpp<BLM_DPP_XOR2>(v);
+  v += blm_dpp<BLM_DPP_HALF_MIRROR>(v);
+  v += blm_dpp<BLM_DPP_MIRROR>(v);
+  return rows_sum(v);
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = blm_max(v, blm_dpp<BLM_DPP_XOR1>(v));
+  v = blm_max(v, blm_dpp<BLM_DPP_XOR2>(v));
+  v = blm_max(v, blm_dpp<BLM_DPP_HALF_MIRROR>(v));
+  v = blm_max(v, blm_dpp<BLM_DPP_MIRROR>(v));
+  return rows_max(v);
+}
+
+// Sum over a block of up to 1024 threads (whole wavefronts); every thread gets the result, the
+// wavefronts' sums added in the order of the wavefronts.  `red` holds 16 floats.  FRESH: `red` has
+// not been used in this kernel before, so nobody can still be reading it.
+template <bool FRESH = false>
 __device__ __forceinline__ float block_sum(float v, float* red) {
   const int lane = threadIdx.x & (BLM_WAVE - 1), w = threadIdx.x / BLM_WAVE;
   const int nw = (blockDim.x + BLM_WAVE - 1) / BLM_WAVE;
   v = wave_sum(v);
-  __syncthreads();  // red may still be read from an earlier call
+  if (nw == 1) return v;
+  if (!FRESH) __syncthreads();
   if (lane == 0) red[w] = v;
   __syncthreads();
-  if (w == 0) {
-    float t = lane < nw ? red[lane] : 0.f;
-    t = wave_sum(t);
-    if (lane == 0) red[16] = t;
-  }
-  __syncthreads();
-  return red[16];
+  float t = red[0];
+  for (int k = 1; k < nw; ++k) t += red[k];
+  return t;
 }
+template <bool FRESH = false>
 __device__ __forceinline__ float block_max(float v, float* red) {
   const int lane = threadIdx.x & (BLM_WAVE - 1), w = threadIdx.x / BLM_WAVE;
   const int nw = (blockDim.x + BLM_WAVE - 1) / BLM_WAVE;
   v = wave_max(v);
-  __syncthreads();
+  if (nw == 1) return v;
+  if (!FRESH) __syncthreads();
   if (lane == 0) red[w] = v;
   __syncthreads();
-  if (w == 0) {
-    float t = lane < nw ? red[lane] : -INFINITY;
-    t = wave_max(t);
-    if (lane == 0) red[16] = t;
-  }
-  __syncthreads();
-  return red[16];
+  float t = red[0];
+  for (int k = 1; k < nw; ++k) t = blm_max(t, red[k]);
+  return t;
 }
 
 // One direct load of 16 bytes per lane from global memory into shared memory at lds (the same in all

@@ -94,7 +94,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     }
     ss += v * v;
   }
-  ss = block_sum(ss, red);
+  ss = block_sum<true>(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)D + eps);
   TA* o = out + (size_t)i * D;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(512)
       for (int e = 0; e < 4; ++e) ss += v[it][e] * v[it][e];
     }
   }
-  ss = block_sum(ss, red);
+  ss = block_sum<true>(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)D + eps);
   TA* o = out + (size_t)i * D;
 #pragma unroll
