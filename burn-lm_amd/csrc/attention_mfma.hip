@@ -8,8 +8,10 @@
 //   O^T += V^T P^T      A = V^T rows (16 dims x 32 keys), B = P^T.  The probabilities a lane has
 //                       just computed are exactly the B fragment it must supply (the order of the
 //                       32 keys inside an MFMA is free as long as A and B agree), so P never moves.
-//                       V is cached transposed per page ([head_dim][64 tokens]) so that the A
-//                       fragment of V^T is two 8-byte loads.
+//                       V is cached transposed per page ([head_dim][64 tokens]), and the keys of a
+//                       page are dealt to the four 16-key tiles so that the eight keys a lane
+//                       supplies to one of these instructions are neighbours: the A fragment of V^T
+//                       is one 16-byte load (am_key_of).
 // No shared memory is needed for the products and nothing is transposed at run time.
 //
 // Prefill: the 16 query columns are 16 consecutive tokens of one head of one sequence.
@@ -17,6 +19,8 @@
 //          cut into splits that are merged afterwards (float partial results).
 // Visibility: query at position p sees keys j <= p of its sequence and, with a window w, p - j < w.
 #include <stdlib.h>
+
+#include <type_traits>
 
 #include "common.h"
 
@@ -27,6 +31,8 @@ typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
 
 #define AM_WAVES 4
 #define AM_PAGE 64
+// s_waitcnt vmcnt(0) of gfx9 (vmcnt in bits 3:0 and 15:14; the other counters left at their maxima)
+#define AM_WAIT_LOADS() __builtin_amdgcn_s_waitcnt(0x0F70)
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
 
@@ -49,16 +55,112 @@ __device__ __forceinline__ uint2 keep_first(uint2 v, int n) {
   return make_uint2((uint32_t)y, (uint32_t)(y >> 32));
 }
 
+// keep the first n (0..8) bf16 of a 16-byte group, zero the rest
+__device__ __forceinline__ uint4 keep_first(uint4 v, int n) {
+  const uint2 lo = keep_first(make_uint2(v.x, v.y), n), hi = keep_first(make_uint2(v.z, v.w), n - 4);
+  return make_uint4(lo.x, lo.y, hi.x, hi.y);
+}
+
+// Which key of a page row i (0..15) of score tile t (0..3) is: the scores of tile t leave lane group kg
+// with rows kg * 4 .. + 3, and the product with the values takes tiles 2 h and 2 h + 1 together, a lane
+// supplying its four rows of the one and then of the other.  With this order those are the keys
+// h * 32 + kg * 8 .. + 7.  The staged key page holds key am_key_of(t, i) in row t * 16 + i.
+__device__ __forceinline__ constexpr int am_key_of(int t, int i) { return (t >> 1) * 32 + (i >> 2) * 8 + (t & 1) * 4 + (i & 3); }
+// the staged row of key k of a page (the inverse)
+__device__ __forceinline__ constexpr int am_row_of(int k) {
+  return ((((k >> 5) << 1) | ((k >> 2) & 1)) << 4) | (((k >> 3) & 3) << 2) | (k & 3);
+}
+
 // One page of keys for one wavefront.  qf: B fragments of Q^T.  Lane (kg = lane / 16, c = lane % 16)
-// owns query column c.  qpos / lo: highest / lowest key this lane's query may see.  max_key: highest
-// key index any query of the tile may see (values past it may be garbage and are zeroed).
+// owns query column c.  qpos / lo: highest / lowest key this lane's query may see.  max_key: the last
+// key that the cache holds data for (values past it may be garbage and are zeroed; between a query's
+// own position and max_key they are other tokens' values, finite, and meet a probability of zero).
 // FULL: every key of the page is visible to every query of the tile, so no mask is computed.
 // The softmax runs in base 2: scale2 = scale * log2(e), m is the running maximum of s * scale2,
 // probabilities are exp2(s * scale2 - m); sums and outputs are the same as in base e.
-// KSTR / VSTR: row strides (elements) of the key page [64][KSTR] and the value page [HD][VSTR].
-// V_LATE: the values are read after the scores (pages in shared memory: short latency, fewer
-// registers); otherwise together with the keys (pages in global memory: one round trip for both).
-template <int HD, bool FULL, int KSTR, int VSTR, bool V_LATE>
+// PAGE: where the fragments of a staged page lie (one of the two layouts below); the values are read
+// after the scores, so they arrive during the softmax and the keys' registers are free by then.
+
+// Rows padded so that the 16-byte fragment reads of 16 rows meet every bank once (any head size):
+// keys [64][HD + 8], values [HD][64 + 8] (strides = 16 bytes mod 128).
+template <int HD>
+struct PaddedPage {
+  static constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 8;
+  static constexpr int K_ELEMS = AM_PAGE * KSTR, V_ELEMS = HD * VSTR;
+  // element offset of the 8 dims ks * 32 + kg * 8 .. of staged key row t * 16 + c
+  static __device__ __forceinline__ int k(int t, int ks, int c, int kg) { return (t * 16 + c) * KSTR + ks * 32 + kg * 8; }
+  // element offset of the 8 keys h * 32 + kg * 8 .. of value dim dt * 16 + c
+  static __device__ __forceinline__ int v(int dt, int h, int c, int kg) { return (dt * 16 + c) * VSTR + h * 32 + kg * 8; }
+};
+// Rows as they lie in memory (so a page can come straight from global memory, 1 KB per load
+// instruction), with the 16-byte pieces of a row permuted: piece J of row r is at place J ^ f(r).  Value
+// rows are 128 bytes (8 pieces), f(r) = (r / 2) % 8: the 16 rows of a fragment read then cover the 16
+// combinations of (r % 2, place), that is every bank.  Key rows of 64 dims likewise; key rows of 128
+// dims are 256 bytes (16 pieces, all banks once per row), f(r) = r % 16.
+template <int HD>
+struct SwizzledPage {
+  static_assert(HD == 64 || HD == 128, "rows of 128 or 256 bytes");
+  static constexpr int K_ELEMS = AM_PAGE * HD, V_ELEMS = HD * AM_PAGE;
+  static __device__ __forceinline__ int k_twist(int row) { return HD == 64 ? (row >> 1) & 7 : row & 15; }
+  static __device__ __forceinline__ int v_twist(int row) { return (row >> 1) & 7; }
+  static __device__ __forceinline__ int k(int t, int ks, int c, int kg) {
+    return (t * 16 + c) * HD + ((ks * 4 + kg) ^ k_twist(c)) * 8;   // k_twist(t * 16 + c) = k_twist(c)
+  }
+  static __device__ __forceinline__ int v(int dt, int h, int c, int kg) {
+    return (dt * 16 + c) * AM_PAGE + ((h * 4 + kg) ^ v_twist(c)) * 8;
+  }
+};
+
+// The order of the keys in a staged key page: row r holds key ORDER::key_of(r) of the page, and
+// ORDER::row_of is the inverse.
+struct TileOrder16 {   // for the 16x16x32 instruction, see am_key_of
+  static __device__ __forceinline__ constexpr int key_of(int row) { return am_key_of(row >> 4, row & 15); }
+  static __device__ __forceinline__ constexpr int row_of(int key) { return am_row_of(key); }
+};
+
+// A page straight from global memory into a SwizzledPage in shared memory, by the four wavefronts of a
+// block: wavefront w fills the 1-KB pieces w, w + 4, .. of the key page and of the value page, lane i
+// of piece L the place L * 64 + i, with the 16 bytes of global memory that the layout puts there (for
+// keys: of the key that belongs in that row).  What a lane adds to the page's address is the same in all
+// of a wavefront's pieces up to a term that all lanes share: four pieces further the staged row has
+// grown by a multiple of 16, which changes neither the twist nor a key's place among its 16 or 32.
+// The loads are invisible to the compiler (blm_dma16_to): the caller waits for them (AM_WAIT_LOADS)
+// before the barrier that hands the page over.
+template <int HD, class ORDER>
+struct DirectStage {
+  using PAGE = SwizzledPage<HD>;
+  static constexpr int PIECES = AM_PAGE * HD * 2 / 1024, PER_WAVE = PIECES / AM_WAVES;
+  static_assert(PIECES % AM_WAVES == 0, "pieces per wavefront");
+  static constexpr int K_CPR = HD / 8, V_CPR = AM_PAGE / 8;   // 16-byte pieces per row
+  static constexpr int K_RPP = BLM_WAVE / K_CPR;              // staged key rows per 1-KB piece
+  uint32_t k_lane, v_lane, k_lds0, v_lds0;
+  int wave_u;
+  // k_lds, v_lds: the first of the block's page buffers (further ones follow at PAGE::K_ELEMS / V_ELEMS)
+  __device__ __forceinline__ void init(const bf16* k_lds, const bf16* v_lds) {
+    const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+    wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int k_row = wave * K_RPP + lane / K_CPR;       // staged row that this lane fills in piece w
+    const int v_row = (wave * BLM_WAVE + lane) / V_CPR;
+    k_lane = (uint32_t)((ORDER::key_of(k_row) * K_CPR + ((lane % K_CPR) ^ PAGE::k_twist(k_row))) * 16);
+    v_lane = (uint32_t)((v_row * V_CPR + ((lane % V_CPR) ^ PAGE::v_twist(v_row))) * 16 - wave * 1024);
+    k_lds0 = (uint32_t)(uintptr_t)(blm_lds_ptr)k_lds;
+    v_lds0 = (uint32_t)(uintptr_t)(blm_lds_ptr)v_lds;
+  }
+  // base: element offset of the (page, key-value head) in the cache planes (the same in all lanes)
+  __device__ __forceinline__ void fetch(const bf16* kcache, const bf16* vcache, size_t base, int buf) const {
+    const char* kb = reinterpret_cast<const char*>(kcache + base);
+    const char* vb = reinterpret_cast<const char*>(vcache + base);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+      const int piece = wave_u + i * AM_WAVES;
+      const int k_step = (ORDER::key_of(piece * K_RPP) - ORDER::key_of(wave_u * K_RPP)) * HD * 2;
+      blm_dma16_to(kb + k_step, k_lane, k_lds0 + (uint32_t)(buf * PAGE::K_ELEMS * 2 + piece * 1024));
+      blm_dma16_to(vb + piece * 1024, v_lane, v_lds0 + (uint32_t)(buf * PAGE::V_ELEMS * 2 + piece * 1024));
+    }
+  }
+};
+
+template <int HD, bool FULL, class PAGE>
 __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf16* __restrict__ vp,
                                           const uint4* qf, int key0, int qpos, int lo, int max_key, float scale2,
                                           float& m, f32x4_t& l, f32x4_t* o) {
@@ -75,14 +177,8 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + kg * 8;
-      kf[t][ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(kp + (size_t)(t * 16 + c) * KSTR + d) : zero;
+      kf[t][ks] = (HD % 32 == 0 || d < HD) ? *reinterpret_cast<const uint4*>(kp + PAGE::k(t, ks, c, kg)) : zero;
     }
-  uint2 vf[DT][4];
-#define AM_LOAD_VALUES()                                                                                    \
-  _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) _Pragma("unroll") for (int t = 0; t < 4; ++t)           \
-      vf[dt][t] = *reinterpret_cast<const uint2*>(vp + (size_t)(dt * 16 + c) * VSTR + t * 16 + kg * 4)
-  if (!V_LATE) { AM_LOAD_VALUES(); }
-
   // scores, unscaled; the scale (> 0) goes into the exponent's multiply-add
   float s[4][4];
 #pragma unroll
@@ -97,12 +193,16 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
       if (FULL) {
         s[t][r] = acc[r];
       } else {
-        const int kj = key0 + t * 16 + kg * 4 + r;
+        const int kj = key0 + am_key_of(t, kg * 4 + r);
         s[t][r] = (kj <= qpos && kj >= lo) ? acc[r] : -INFINITY;
       }
     }
   }
-  if (V_LATE) { AM_LOAD_VALUES(); }   // the keys' registers are free now; the values arrive during the softmax
+  uint4 vf[DT][2];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) vf[dt][h] = *reinterpret_cast<const uint4*>(vp + PAGE::v(dt, h, c, kg));
   float mx = blm_max(s[0][0], s[0][1]);
   mx = blm_max(blm_max(mx, s[0][2]), s[0][3]);
 #pragma unroll
@@ -133,7 +233,6 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
   }
   m = m_new;
 
-#undef AM_LOAD_VALUES
   // O^T += V^T P^T, 32 keys (two 16-key tiles) per MFMA
   const bool tail = !FULL && key0 + AM_PAGE - 1 > max_key;   // uniform: the page holds places past the data
 #pragma unroll
@@ -149,12 +248,8 @@ __device__ __forceinline__ void attn_page(const bf16* __restrict__ kp, const bf1
                                                 __builtin_bit_cast(bf16x8_t, pf), l, 0, 0, 0);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      uint2 v0 = vf[dt][2 * h], v1 = vf[dt][2 * h + 1];
-      if (tail) {   // 0 * garbage must stay 0
-        v0 = keep_first(v0, max_key - (key0 + (2 * h) * 16 + kg * 4) + 1);
-        v1 = keep_first(v1, max_key - (key0 + (2 * h + 1) * 16 + kg * 4) + 1);
-      }
-      const uint4 va = make_uint4(v0.x, v0.y, v1.x, v1.y);
+      uint4 va = vf[dt][h];
+      if (tail) va = keep_first(va, max_key - (key0 + h * 32 + kg * 8) + 1);   // 0 * garbage must stay 0
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, va),
                                                       __builtin_bit_cast(bf16x8_t, pf), o[dt], 0, 0, 0);
     }
@@ -215,16 +310,18 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
                              float scale, int window) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
-  // row strides in shared memory: keys are read 16 bytes per lane from 16 rows (stride = 16 bytes mod
-  // 128 keeps the 32 banks apart), values 8 bytes per lane from 16 rows (stride = 8 bytes mod 128)
-  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 4;
+  // Head sizes 64 and 128: a page comes straight from global memory into shared memory, its rows'
+  // pieces permuted.  Other head sizes: through registers into padded rows.
+  constexpr bool DIRECT = HD == 64 || HD == 128;
+  using PAGE = std::conditional_t<DIRECT, SwizzledPage<DIRECT ? HD : 64>, PaddedPage<HD>>;
+  constexpr int KSTR = PaddedPage<HD>::KSTR, VSTR = PaddedPage<HD>::VSTR;
   constexpr int CHUNKS = AM_PAGE * HD / 8;              // 16-byte pieces of a page (keys and values alike)
   constexpr int PER_THREAD = (CHUNKS + AM_WAVES * BLM_WAVE - 1) / (AM_WAVES * BLM_WAVE);
   // two buffers for head sizes whose pages fit twice: the next page is written while the current
   // one is still being used, and one barrier per page is enough
   constexpr int NBUF = HD <= 128 ? 2 : 1;
-  __shared__ __align__(16) bf16 k_lds[NBUF][AM_PAGE * KSTR];
-  __shared__ __align__(16) bf16 v_lds[NBUF][HD * VSTR];   // HD * VSTR * 2 bytes is a multiple of 16
+  __shared__ __align__(16) bf16 k_lds[NBUF][PAGE::K_ELEMS];
+  __shared__ __align__(16) bf16 v_lds[NBUF][PAGE::V_ELEMS];   // a multiple of 16 bytes in either layout
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int c = lane & 15, kg = lane >> 4;
   const int G = nh / nkv;
@@ -254,6 +351,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
   const int qpos = positions[row];
   const int qpos_first = positions[row_begin + (active ? qt * 16 : 0)];
   const int qpos_last = positions[row_begin + (active ? qt * 16 + nq - 1 : 0)];
+  const int seq_last = positions[row_begin + n_b - 1];   // the cache holds data up to here: places past it may hold anything
   const int lo = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
   const int lo_tile = (window > 0 && qpos_first - window + 1 > 0) ? qpos_first - window + 1 : 0;
   const int lo_last = (window > 0 && qpos_last - window + 1 > 0) ? qpos_last - window + 1 : 0;
@@ -292,12 +390,10 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
   _Pragma("unroll") for (int i = 0; i < PER_THREAD; ++i) {                                                      \
     const int j = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                                        \
     if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || j < CHUNKS) {                                                    \
-      const int kr = j / (HD / 8), kc = j - kr * (HD / 8);           /* key row, 16-byte column */              \
-      *reinterpret_cast<u32x4_t*>(k_lds[buf] + kr * KSTR + kc * 8) = kreg[i];                                   \
+      const int kr = j / (HD / 8), kc = j - kr * (HD / 8);           /* key, 16-byte column */                  \
+      *reinterpret_cast<u32x4_t*>(k_lds[buf] + am_row_of(kr) * KSTR + kc * 8) = kreg[i];                        \
       const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8); /* value row (a dim), 16-byte column */    \
-      u32x2_t* vd = reinterpret_cast<u32x2_t*>(v_lds[buf] + vr * VSTR + vc * 8);   /* rows are 8-byte aligned */  \
-      vd[0] = u32x2_t{vreg[i].x, vreg[i].y};                                                                    \
-      vd[1] = u32x2_t{vreg[i].z, vreg[i].w};                                                                    \
+      *reinterpret_cast<u32x4_t*>(v_lds[buf] + vr * VSTR + vc * 8) = vreg[i];                                   \
     }                                                                                                           \
   }
 #define AM_USE(buf)                                                                                           \
@@ -305,10 +401,26 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
     const int key0 = pi * AM_PAGE;                                                                              \
     /* pages wholly inside every query's range need no mask */                                                  \
     if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)                                                    \
-      attn_page<HD, true, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o);  \
+      attn_page<HD, true, PAGE>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, seq_last, scale2, m, lsum, o);  \
     else                                                                                                        \
-      attn_page<HD, false, KSTR, VSTR, true>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o); \
+      attn_page<HD, false, PAGE>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, seq_last, scale2, m, lsum, o); \
   }
+  if constexpr (DIRECT) {
+    DirectStage<DIRECT ? HD : 64, TileOrder16> stage;
+    stage.init(k_lds[0], v_lds[0]);
+    auto fetch = [&](int pi, int buf) { stage.fetch(kcache, vcache, ((size_t)pages.at(pi) * nkv + kvh) * AM_PAGE * HD, buf); };
+    fetch(blk_first, 0);
+    am_pin<KS>(qf);   // see below
+    AM_WAIT_LOADS();
+    __syncthreads();
+    for (int pi = blk_first; pi <= blk_last; ++pi) {
+      const int cur = (pi - blk_first) & 1;
+      if (pi < blk_last) fetch(pi + 1, cur ^ 1);   // into the other buffer, which nobody reads now
+      AM_USE(cur)
+      AM_WAIT_LOADS();     // the compiler does not know of these loads: the wait is the program's own
+      __syncthreads();     // the next page is in place, and everybody is done with this one
+    }
+  } else {
   AM_FETCH(blk_first);
   // The query fragments have arrived before the loop starts.  Left alone, the compiler moves their
   // loads down to the loop's entry, and since its count of outstanding loads is merged over the loop's
@@ -333,6 +445,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
       if (pi < blk_last) AM_FETCH(pi + 1);   // travels while this page is used
       AM_USE(0)
     }
+  }
   }
 #undef AM_STAGE
 #undef AM_USE
@@ -365,13 +478,34 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 //                    query l % 32, the same dims); the result leaves lane (j = l % 32, hb = l / 32)
 //                    with the scores of query j for keys 8 (v / 4) + 4 hb + v % 4, v < 16, of the tile.
 //   O^T += V^T P^T   A = 32 dims x 16 keys, B = P^T.  The 16 keys of instruction n of a 32-key tile are
-//                    the ones whose scores sit in accumulator values 8 n .. 8 n + 7: lane hb supplies
-//                    keys 16 n + 4 hb .. + 3 and 16 n + 8 + 4 hb .. + 3, which are exactly those values,
-//                    so the probabilities never move; the matching V^T fragment is two 8-byte reads.
+//                    the ones whose scores sit in accumulator values 8 n .. 8 n + 7: lane hb supplies rows
+//                    16 n + 4 hb .. + 3 and 16 n + 8 + 4 hb .. + 3 of the tile, which are exactly those
+//                    values, so the probabilities never move.  The staged key page holds its keys in an
+//                    order (TileOrder32) in which these eight rows are the neighbouring keys
+//                    16 n + 8 hb .. + 7, so the matching V^T fragment is one 16-byte read.
 // The softmax of a query lives in the two lanes j and j + 32; the denominator is summed by one
 // two-element dot product with ones per pair of rounded probabilities (v_dot2c_f32_bf16).
 // ---------------------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+// Key order of the 32-query form: row r of the staged key page holds the key whose number is r with
+// bits 2 and 3 exchanged (its own inverse).
+struct TileOrder32 {
+  static __device__ __forceinline__ constexpr int key_of(int row) { return (row & ~12) | ((row & 4) << 1) | ((row & 8) >> 1); }
+  static __device__ __forceinline__ constexpr int row_of(int key) { return key_of(key); }
+};
+// Element offsets of the 32-query form's fragments in the two page layouts: the 8 dims ks * 16 + hb * 8 ..
+// of staged key row `row`, and the 8 keys piece * 8 .. of value dim `dim` (piece: 0..7).
+template <int HD>
+struct PaddedFragments32 {
+  static __device__ __forceinline__ int k(int row, int ks, int hb) { return row * PaddedPage<HD>::KSTR + ks * 16 + hb * 8; }
+  static __device__ __forceinline__ int v(int dim, int piece) { return dim * PaddedPage<HD>::VSTR + piece * 8; }
+};
+template <int HD>
+struct SwizzledFragments32 {
+  static __device__ __forceinline__ int k(int row, int ks, int hb) { return row * HD + ((ks * 2 + hb) ^ SwizzledPage<HD>::k_twist(row)) * 8; }
+  static __device__ __forceinline__ int v(int dim, int piece) { return dim * AM_PAGE + (piece ^ SwizzledPage<HD>::v_twist(dim)) * 8; }
+};
 
 // acc + lo + hi of a pair of bf16 in one instruction
 __device__ __forceinline__ float am_dot2_ones(uint32_t pair, float acc) {
@@ -379,11 +513,12 @@ __device__ __forceinline__ float am_dot2_ones(uint32_t pair, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(am_bf16x2, pair), __builtin_bit_cast(am_bf16x2, 0x3f803f80u), acc, false);
 }
 
-// One half page (32 keys from key0) for one wavefront: the softmax state advances once per 32 keys, so
-// only 16 scores per lane are alive at a time.
-template <int HD, bool FULL, int KSTR, int VSTR>
+// Half `half` of a page (32 keys from key0) for one wavefront: the softmax state advances once per 32
+// keys, so only 16 scores per lane are alive at a time.  kp, vp: the staged page; FRAG: where its
+// fragments lie.  max_key: the last key that the cache holds data for (see attn_page).
+template <int HD, bool FULL, class FRAG>
 __device__ __forceinline__ void attn_half32(const bf16* __restrict__ kp, const bf16* __restrict__ vp, const uint4* qf,
-                                            int key0, int qpos, int lo, int max_key, float scale2, float& m,
+                                            int half, int key0, int qpos, int lo, int max_key, float scale2, float& m,
                                             float& l, f32x16_t* o) {
   constexpr int KS = HD / 16, RT = HD / 32;
   const int lane = threadIdx.x & (BLM_WAVE - 1);
@@ -393,13 +528,13 @@ __device__ __forceinline__ void attn_half32(const bf16* __restrict__ kp, const b
   for (int v = 0; v < 16; ++v) s[v] = 0.f;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    const uint4 kf = *reinterpret_cast<const uint4*>(kp + (size_t)j * KSTR + ks * 16 + hb * 8);
+    const uint4 kf = *reinterpret_cast<const uint4*>(kp + FRAG::k(half * 32 + j, ks, hb));
     s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf), __builtin_bit_cast(bf16x8_t, qf[ks]), s, 0, 0, 0);
   }
   if (!FULL) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int kj = key0 + 8 * (v >> 2) + 4 * hb + (v & 3);
+      const int kj = key0 + TileOrder32::key_of(8 * (v >> 2) + 4 * hb + (v & 3));
       s[v] = (kj <= qpos && kj >= lo) ? s[v] : -INFINITY;
     }
   }
@@ -437,29 +572,25 @@ __device__ __forceinline__ void attn_half32(const bf16* __restrict__ kp, const b
     // the denominator takes the rounded probabilities, two per instruction (a dot product with ones);
     // a lane sums its own keys, the two lanes of a query are added at the end
     l = am_dot2_ones(pf.x, l); l = am_dot2_ones(pf.y, l); l = am_dot2_ones(pf.z, l); l = am_dot2_ones(pf.w, l);
-    const int kb = 16 * n + 4 * hb;   // this lane's keys of the instruction: kb .. kb + 3 and kb + 8 .. kb + 11
+    const int piece = half * 4 + n * 2 + hb;   // this lane's keys of the instruction: piece * 8 .. + 7 of the page
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const bf16* vrow = vp + (size_t)(rt * 32 + j) * VSTR + kb;
-      uint2 v0 = *reinterpret_cast<const uint2*>(vrow), v1 = *reinterpret_cast<const uint2*>(vrow + 8);
-      if (tail) {   // 0 * garbage must stay 0
-        v0 = keep_first(v0, max_key - (key0 + kb) + 1);
-        v1 = keep_first(v1, max_key - (key0 + kb + 8) + 1);
-      }
-      const uint4 va = make_uint4(v0.x, v0.y, v1.x, v1.y);
+      uint4 va = *reinterpret_cast<const uint4*>(vp + FRAG::v(rt * 32 + j, piece));
+      if (tail) va = keep_first(va, max_key - (key0 + n * 16 + hb * 8) + 1);   // 0 * garbage must stay 0
       o[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, pf), o[rt], 0, 0, 0);
     }
   }
 }
 
-template <int HD, bool FULL, int KSTR, int VSTR>
+// tile_last: the last key that any query of the tile sees
+template <int HD, bool FULL, class FRAG>
 __device__ __forceinline__ void attn_page32(const bf16* __restrict__ kp, const bf16* __restrict__ vp, const uint4* qf,
-                                            int key0, int qpos, int lo, int max_key, float scale2, float& m,
+                                            int key0, int qpos, int lo, int tile_last, int max_key, float scale2, float& m,
                                             float& l, f32x16_t* o) {
-  attn_half32<HD, FULL, KSTR, VSTR>(kp, vp, qf, key0, qpos, lo, max_key, scale2, m, l, o);
+  attn_half32<HD, FULL, FRAG>(kp, vp, qf, 0, key0, qpos, lo, max_key, scale2, m, l, o);
   // the second half of a page on the diagonal may lie wholly behind the tile's last query
-  if (FULL || key0 + 32 <= max_key)
-    attn_half32<HD, FULL, KSTR, VSTR>(kp + 32 * KSTR, vp + 32, qf, key0 + 32, qpos, lo, max_key, scale2, m, l, o);
+  if (FULL || key0 + 32 <= tile_last)
+    attn_half32<HD, FULL, FRAG>(kp, vp, qf, 1, key0 + 32, qpos, lo, max_key, scale2, m, l, o);
 }
 
 // grid (ceil(G * q_tiles32 / 4), kv heads, sequences); the block order and the page staging are those
@@ -473,11 +604,14 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
                           float scale, int window) {
   static_assert(HD % 32 == 0 && HD <= 128, "32-query prefill: head sizes 32, 64, 96, 128");
   constexpr int KS = HD / 16, RT = HD / 32, QT = 32;
-  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 4;
+  constexpr bool DIRECT = HD == 64 || HD == 128;   // as in the 16-query kernel
+  using PAGE = std::conditional_t<DIRECT, SwizzledPage<DIRECT ? HD : 64>, PaddedPage<HD>>;
+  using FRAG = std::conditional_t<DIRECT, SwizzledFragments32<DIRECT ? HD : 64>, PaddedFragments32<HD>>;
+  constexpr int KSTR = PaddedPage<HD>::KSTR, VSTR = PaddedPage<HD>::VSTR;
   constexpr int CHUNKS = AM_PAGE * HD / 8;
   constexpr int PER_THREAD = (CHUNKS + AM_WAVES * BLM_WAVE - 1) / (AM_WAVES * BLM_WAVE);
-  __shared__ __align__(16) bf16 k_lds[2][AM_PAGE * KSTR];
-  __shared__ __align__(16) bf16 v_lds[2][HD * VSTR];
+  __shared__ __align__(16) bf16 k_lds[2][PAGE::K_ELEMS];
+  __shared__ __align__(16) bf16 v_lds[2][PAGE::V_ELEMS];
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int j = lane & 31, hb = lane >> 5;
   const int G = nh / nkv;
@@ -502,6 +636,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
   const int qpos = positions[row];
   const int qpos_first = positions[row_begin + (active ? qt * QT : 0)];
   const int qpos_last = positions[row_begin + (active ? qt * QT + nq - 1 : 0)];
+  const int seq_last = positions[row_begin + n_b - 1];   // the cache holds data up to here
   const int lo = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
   const int lo_tile = (window > 0 && qpos_first - window + 1 > 0) ? qpos_first - window + 1 : 0;
   const int lo_last = (window > 0 && qpos_last - window + 1 > 0) ? qpos_last - window + 1 : 0;
@@ -546,31 +681,46 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
     const int jj = i * AM_WAVES * BLM_WAVE + threadIdx.x;                                                       \
     if (CHUNKS % (AM_WAVES * BLM_WAVE) == 0 || jj < CHUNKS) {                                                   \
       const int kr = jj / (HD / 8), kc = jj - kr * (HD / 8);                                                    \
-      *reinterpret_cast<u32x4_t*>(k_lds[buf] + kr * KSTR + kc * 8) = kreg[i];                                   \
+      *reinterpret_cast<u32x4_t*>(k_lds[buf] + TileOrder32::row_of(kr) * KSTR + kc * 8) = kreg[i];              \
       const int vr = jj / (AM_PAGE / 8), vc = jj - vr * (AM_PAGE / 8);                                          \
-      u32x2_t* vd = reinterpret_cast<u32x2_t*>(v_lds[buf] + vr * VSTR + vc * 8);                                \
-      vd[0] = u32x2_t{vreg[i].x, vreg[i].y};                                                                    \
-      vd[1] = u32x2_t{vreg[i].z, vreg[i].w};                                                                    \
+      *reinterpret_cast<u32x4_t*>(v_lds[buf] + vr * VSTR + vc * 8) = vreg[i];                                   \
     }                                                                                                           \
   }
 #define AP_USE(buf)                                                                                           \
   if (pi >= my_first && pi <= my_last) {                                                                        \
     const int key0 = pi * AM_PAGE;                                                                              \
     if (key0 + AM_PAGE - 1 <= qpos_first && key0 >= lo_last)                                                    \
-      attn_page32<HD, true, KSTR, VSTR>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o);  \
+      attn_page32<HD, true, FRAG>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, seq_last, scale2, m, lsum, o);  \
     else                                                                                                        \
-      attn_page32<HD, false, KSTR, VSTR>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, scale2, m, lsum, o); \
+      attn_page32<HD, false, FRAG>(k_lds[buf], v_lds[buf], qf, key0, qpos, lo, qpos_last, seq_last, scale2, m, lsum, o); \
   }
-  AP_FETCH(blk_first);
-  am_pin<HD / 16>(qf);   // as in the 16-query kernel
-  AP_STAGE(0)
-  __syncthreads();
-  for (int pi = blk_first; pi <= blk_last; ++pi) {
-    const int cur = (pi - blk_first) & 1;
-    if (pi < blk_last) AP_FETCH(pi + 1);   // travels while this page is used
-    AP_USE(cur)
-    if (pi < blk_last) { AP_STAGE(cur ^ 1) }   // the other buffer: nobody reads it now
-    __syncthreads();   // the next page is in place, and everybody is done with this one
+  if constexpr (DIRECT) {
+    DirectStage<DIRECT ? HD : 64, TileOrder32> stage;
+    stage.init(k_lds[0], v_lds[0]);
+    auto fetch = [&](int pi, int buf) { stage.fetch(kcache, vcache, ((size_t)pages.at(pi) * nkv + kvh) * AM_PAGE * HD, buf); };
+    fetch(blk_first, 0);
+    am_pin<HD / 16>(qf);   // as in the 16-query kernel
+    AM_WAIT_LOADS();
+    __syncthreads();
+    for (int pi = blk_first; pi <= blk_last; ++pi) {
+      const int cur = (pi - blk_first) & 1;
+      if (pi < blk_last) fetch(pi + 1, cur ^ 1);   // into the other buffer, which nobody reads now
+      AP_USE(cur)
+      AM_WAIT_LOADS();
+      __syncthreads();     // the next page is in place, and everybody is done with this one
+    }
+  } else {
+    AP_FETCH(blk_first);
+    am_pin<HD / 16>(qf);   // as in the 16-query kernel
+    AP_STAGE(0)
+    __syncthreads();
+    for (int pi = blk_first; pi <= blk_last; ++pi) {
+      const int cur = (pi - blk_first) & 1;
+      if (pi < blk_last) AP_FETCH(pi + 1);   // travels while this page is used
+      AP_USE(cur)
+      if (pi < blk_last) { AP_STAGE(cur ^ 1) }   // the other buffer: nobody reads it now
+      __syncthreads();   // the next page is in place, and everybody is done with this one
+    }
   }
 #undef AP_STAGE
 #undef AP_USE
@@ -617,7 +767,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   // padded as in the prefill kernel.  Nobody else touches a wavefront's area, so no barrier is
   // needed, and the next page travels in registers while the current one is used.  The areas serve
   // once more at the end, for the wavefronts' partial outputs.
-  constexpr int KSTR = HD + 8, VSTR = AM_PAGE + 4;
+  constexpr int KSTR = PaddedPage<HD>::KSTR, VSTR = PaddedPage<HD>::VSTR;
   constexpr int CHUNKS = AM_PAGE * HD / 8;              // 16-byte pieces of a page (keys and values alike)
   constexpr int PER_LANE = CHUNKS / BLM_WAVE;           // HD is a multiple of 16, so this is exact
   constexpr int STAGE_ELEMS = AM_PAGE * KSTR + HD * VSTR;
@@ -668,12 +818,10 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
 #define AD_STAGE()                                                                                            \
   _Pragma("unroll") for (int i = 0; i < PER_LANE; ++i) {                                                        \
     const int j = i * BLM_WAVE + lane;                                                                          \
-    const int kr = j / (HD / 8), kc = j - kr * (HD / 8);           /* key row, 16-byte column */                \
-    *reinterpret_cast<u32x4_t*>(k_lds + kr * KSTR + kc * 8) = kreg[i];                                          \
+    const int kr = j / (HD / 8), kc = j - kr * (HD / 8);           /* key, 16-byte column */                    \
+    *reinterpret_cast<u32x4_t*>(k_lds + am_row_of(kr) * KSTR + kc * 8) = kreg[i];                               \
     const int vr = j / (AM_PAGE / 8), vc = j - vr * (AM_PAGE / 8); /* value row (a dim), 16-byte column */      \
-    u32x2_t* vd = reinterpret_cast<u32x2_t*>(v_lds + vr * VSTR + vc * 8);   /* rows are 8-byte aligned */       \
-    vd[0] = u32x2_t{vreg[i].x, vreg[i].y};                                                                      \
-    vd[1] = u32x2_t{vreg[i].z, vreg[i].w};                                                                      \
+    *reinterpret_cast<u32x4_t*>(v_lds + vr * VSTR + vc * 8) = vreg[i];                                          \
   }
     int pi = p_begin + wave;
     if (pi < p_end) AD_FETCH(pi);
@@ -683,9 +831,9 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
       if (pi + AM_WAVES < p_end) AD_FETCH(pi + AM_WAVES);   // travels while this page is used
       const int key0 = pi * AM_PAGE;
       if (key0 + AM_PAGE - 1 <= pos && key0 >= lo)
-        attn_page<HD, true, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, pos, lo, pos, scale2, m, lsum, o);
+        attn_page<HD, true, PaddedPage<HD>>(k_lds, v_lds, qf, key0, pos, lo, pos, scale2, m, lsum, o);
       else
-        attn_page<HD, false, KSTR, VSTR, true>(k_lds, v_lds, qf, key0, pos, lo, pos, scale2, m, lsum, o);
+        attn_page<HD, false, PaddedPage<HD>>(k_lds, v_lds, qf, key0, pos, lo, pos, scale2, m, lsum, o);
     }
 #undef AD_FETCH
 #undef AD_STAGE
@@ -815,10 +963,11 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
               "attn_prefill_mfma: q rows must be 16-byte aligned");
   const int G = nh / nkv;
   // queries: 16 or 32 query rows per wavefront.  32 (head sizes 32, 64, 96, 128) halves the shared-memory
-  // reads per matrix instruction and is ahead once its blocks are three times the compute units: with fewer,
-  // all blocks run at once and the step lasts as long as the block with the most pages, whose pages take
-  // longer one after another than those of the 16-query form (measured at 32 heads of 64: 2,048 tokens 49.5
-  // against 43.6 us, 4,096 tokens 108 against 137 us; 24 heads of 128: 68 against 58 us, 141 against 187 us).
+  // reads per matrix instruction and is ahead where the work bounds the step (several rounds of blocks); where
+  // all blocks run at once the step lasts as long as the block with the most pages, whose pages take longer
+  // one after another than those of the 16-query form (measured at 32 heads of 64, 32 against 16 queries:
+  // 2,048 tokens 37.6 against 30.5 us, 8,192 tokens 330 against 347, four prompts of 1,024 tokens 48.9 against
+  // 37.3, 32 of them 231 against 261; 24 heads of 128: 2,048 tokens 57 against 43, 8,192 tokens 444 against 490).
   // The caller chooses (blm_attn_prefill_blocks32 gives it the number of blocks to compare).
   BLM_REQUIRE(queries == 16 || (queries == 32 && hd % 32 == 0 && hd <= 128),
               "attn_prefill_mfma: %d queries per wavefront with head_dim %d (16, or 32 with head sizes 32, 64, 96, 128)", queries, hd);

@@ -144,6 +144,10 @@ __device__ __forceinline__ void blm_dma16(const char* base, uint32_t lane_offset
   const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(blm_lds_ptr)lds);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
 }
+// the same with the address in shared memory given as the number it is (no cast of a generic pointer)
+__device__ __forceinline__ void blm_dma16_to(const char* base, uint32_t lane_offset, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
+}
 __device__ __forceinline__ void blm_dma16_lanes(const char* address, const void* lds) {
   const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(blm_lds_ptr)lds);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(address) : "memory", "m0");

@@ -316,10 +316,16 @@ def attn_prefill_mfma_supported(dtype, hd, page_size=64):
 
 
 def attn_prefill_queries(n_seqs, max_new, nh, nkv, hd, compute_units):
-    """Query rows per wavefront that attn_prefill_mfma should take for a step: 32 (half the shared-memory
-    reads per matrix instruction) once that form's blocks are three times the compute units, else 16."""
+    """Query rows per wavefront that attn_prefill_mfma should take for a step.  With 32 every key and value
+    fragment taken from shared memory serves twice the queries, which is worth 5-12 % where the step is bound
+    by the work (several rounds of blocks); with 16 a page takes a wavefront less long, which is worth 15-25 %
+    where all blocks run at once and the step lasts as long as its longest query tile.  So: 32 once that
+    form's blocks are 8 times the compute units (4 times for heads above 64, whose blocks are two to a
+    compute unit), or 2 times with a prompt of 3,072 tokens and more."""
     blocks32 = library().blm_attn_prefill_blocks32(int(n_seqs), int(max_new), int(nh), int(nkv), int(hd))
-    return 32 if blocks32 >= 3 * int(compute_units) else 16
+    rounds = 8 if hd <= 64 else 4
+    units = int(compute_units)
+    return 32 if blocks32 >= rounds * units or (max_new >= 3072 and blocks32 >= 2 * units) else 16
 
 
 def attn_prefill_mfma(q, q_row_stride, out, positions, cu_seqlens, block_table, kcache, vcache, page_size,

@@ -386,9 +386,11 @@ def test_attn_prefill_mfma(ops, nh, nkv, hd, window, tile, monkeypatch):
                                   torch.zeros(1, nkv, hd, 64, dtype=torch.bfloat16, device="cuda"), 64, 1, 16, nh, nkv, hd, 0.1, 0, queries=32)
         pytest.skip("the 32-query form takes head sizes 32, 64, 96 and 128 (and says so)")
     assert ops.attn_prefill_mfma_supported(torch.bfloat16, hd) and not ops.attn_prefill_mfma_supported(torch.float32, hd)
-    # which form a step takes by itself: 32 queries once that form's blocks are three times the compute units
+    # which form a step takes by itself: 32 queries for several rounds of blocks or a long prompt
     assert ops.attn_prefill_queries(1, 2048, 32, 8, 64, 256) == 16 and ops.attn_prefill_queries(1, 4096, 32, 8, 64, 256) == 32
     assert ops.attn_prefill_queries(4, 2048, 32, 8, 64, 256) == 32 and ops.attn_prefill_queries(1, 65536, 6, 1, 24, 256) == 16
+    assert ops.attn_prefill_queries(8, 512, 32, 8, 64, 256) == 16 and ops.attn_prefill_queries(4, 1024, 24, 8, 128, 256) == 16
+    assert ops.attn_prefill_queries(32, 512, 32, 8, 64, 256) == 32 and ops.attn_prefill_queries(2, 2048, 32, 8, 128, 256) == 32
     g = torch.Generator().manual_seed(15)
     lens = [150, 333, 65, 1, 40]             # length of each sequence after the step
     new = [150, 70, 1, 1, 33]                # rows this step brings
