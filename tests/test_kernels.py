@@ -414,6 +414,38 @@ def test_attn_prefill_mfma(ops, nh, nkv, hd, window, tile, monkeypatch):
             close(got[t], want, 1.5e-2)
 
 
+@pytest.mark.parametrize("hd", [64, 48])
+def test_attention_over_more_pages_than_a_register_holds_numbers_of(ops, hd):
+    """The matrix-core attention kernels keep 64 page numbers of a sequence in one register and load the
+    next 64 when a block walks past them.  One sequence of 70 pages with scrambled page numbers: the last
+    150 rows of its prompt (both prefill forms), and a decode token over the whole of it uncut and in three
+    pieces.  Head size 64 takes its pages straight into shared memory, 48 through registers."""
+    g = torch.Generator().manual_seed(16)
+    nh, nkv, window = 2, 1, 0
+    L, new = 70 * 64 - 21, 150
+    table, keys, values, kc, vc = _paged_case(g, [L], nkv, hd, far_key=5, n_pages=75)
+    stride = (nh + 2 * nkv) * hd
+    scale = 1.0 / math.sqrt(hd)
+    positions = list(range(L - new, L))
+    qkv = torch.randn(new, stride, generator=g).bfloat16()
+    table, kc, vc = dev(table), dev(kc), dev(vc)
+    for queries in ((16, 32) if hd % 32 == 0 else (16,)):
+        out = torch.full((new, nh * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.attn_prefill_mfma(dev(qkv), stride, out, dev(torch.tensor(positions, dtype=torch.int32)),
+                              dev(torch.tensor([0, new], dtype=torch.int32)), table, kc, vc, 64, 1, new, nh, nkv, hd, scale, window,
+                              queries=queries)
+        got = out.cpu().double().reshape(new, nh, hd)
+        assert torch.isfinite(got).all()
+        for t in (0, 1, 17, 64, 100, new - 1):
+            close(got[t], _attn_ref(qkv[t, : nh * hd].reshape(nh, hd), keys[0], values[0], positions[t], scale, window, nh // nkv), 1.5e-2)
+    for splits in (1, 3):
+        out = torch.full((1, nh * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.attn_decode(dev(qkv[-1:]), stride, out, dev(torch.tensor([L - 1], dtype=torch.int32)), dev(torch.zeros(1, dtype=torch.int32)),
+                        table, kc, vc, 64, nh, nkv, hd, scale, window, splits)
+        close(out.cpu().double().reshape(nh, hd),
+              _attn_ref(qkv[-1, : nh * hd].reshape(nh, hd), keys[0], values[0], L - 1, scale, window, nh // nkv), 1.5e-2)
+
+
 def test_attn_paged_refuses_what_it_cannot_do(ops):
     from burn_lm_amd.csrc.ops import KernelError
     z = torch.zeros(1, 3 * 258, device="cuda")
