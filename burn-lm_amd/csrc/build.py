@@ -22,7 +22,11 @@ ARCH = "gfx950"
 # packed-fp32 instructions are kept off for every device pass
 # (-Wno-inline-asm: the direct-load statements of common.h name m0 as clobbered, which the compiler
 # answers with a warning per use because it keeps that register for itself)
+# -amdgpu-kernarg-preload-count: a kernel's first 16 dwords of arguments arrive in scalar registers with
+# the wavefront instead of being loaded by its first instructions (every kernel keeps a prologue that
+# loads them for firmware that does not preload); worth 1-2.5 % of a decode step at 32 and 64 sequences.
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wno-inline-asm",
+               "-mllvm", "-amdgpu-kernarg-preload-count=16",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # The matrix-core attention takes maxima of matrix-core results; told that they are no NaNs (masked
 # scores are replaced by -infinity before any maximum, stale values are zeroed as integers) the

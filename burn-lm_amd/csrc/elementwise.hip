@@ -121,6 +121,18 @@ __device__ __forceinline__ void load4<bf16>(const bf16* p, float* v) {
   v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
   v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
 }
+// four elements as they lie in memory, and their values
+template <typename T>
+struct Raw4;
+template <>
+struct Raw4<float> { typedef float4 type; };
+template <>
+struct Raw4<bf16> { typedef uint2 type; };
+__device__ __forceinline__ void unpack4(float4 r, float* v) { v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w; }
+__device__ __forceinline__ void unpack4(uint2 r, float* v) {
+  v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+  v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+}
 template <typename T>
 __device__ __forceinline__ void store4(T* p, const float* v);
 template <>
@@ -145,6 +157,17 @@ __global__ void __launch_bounds__(512)
   const int r = rows ? rows[i] : i;
   float* hr = h + (size_t)r * D;
   const TD* dr = delta ? delta + (size_t)r * D : nullptr;
+  // The norm's weights are asked for first of all, with the row and its planes, and not behind the
+  // barrier: a second trip to memory in a row, where the kernel is nothing but latencies (a decode
+  // step's eight rows).  They are unpacked where the row's sum is complete, that is where everything
+  // asked for has arrived anyway: behind the barrier a wait for them would also wait for the store of
+  // the summed row (stores count with the loads).
+  typename Raw4<TG>::type graw[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int d = (it * blockDim.x + threadIdx.x) * 4;
+    if (d < D) graw[it] = *reinterpret_cast<const typename Raw4<TG>::type*>(gamma + d);
+  }
   float v[ITERS][4];
   float ss = 0.f;
 #pragma unroll
@@ -160,23 +183,43 @@ __global__ void __launch_bounds__(512)
           load4<TD>(dr + d, t);
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[it][e] += t[e];
-        } else for (int p0 = 0; p0 < n_planes; p0 += 4) {
+        } else {
+          // the first four on their own, so that their loads are asked for before the row of h is
+          // first used (as the loop's entry it would be waited for in front of the loop: two trips
+          // to memory in a row instead of one)
           float t[4][4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) load4<TD>(dr + (size_t)min(p0 + q, n_planes - 1) * plane_stride + d, t[q]);
+          for (int q = 0; q < 4; ++q) load4<TD>(dr + (size_t)min(q, n_planes - 1) * plane_stride + d, t[q]);
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            if (p0 + q < n_planes) {
+            if (q < n_planes) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[it][e] += t[q][e];
             }
+          for (int p0 = 4; p0 < n_planes; p0 += 4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) load4<TD>(dr + (size_t)min(p0 + q, n_planes - 1) * plane_stride + d, t[q]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (p0 + q < n_planes) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[it][e] += t[q][e];
+              }
+          }
         }
-        if (write_h) store4<float>(hr + d, v[it]);
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) ss += v[it][e] * v[it][e];
     }
   }
+  float g[ITERS][4];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it)
+    if ((it * blockDim.x + threadIdx.x) * 4 < D) {
+      unpack4(graw[it], g[it]);
+      // a use that cannot move: the unpacking stays in front of the reduction
+      asm volatile("" : "+v"(g[it][0]), "+v"(g[it][1]), "+v"(g[it][2]), "+v"(g[it][3]));
+    }
   ss = block_sum<true>(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)D + eps);
   TA* o = out + (size_t)i * D;
@@ -184,10 +227,10 @@ __global__ void __launch_bounds__(512)
   for (int it = 0; it < ITERS; ++it) {
     const int d = (it * blockDim.x + threadIdx.x) * 4;
     if (d < D) {
-      float g[4], y[4];
-      load4<TG>(gamma + d, g);
+      if (dr && write_h) store4<float>(hr + d, v[it]);
+      float y[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) y[e] = v[it][e] * inv * g[e];
+      for (int e = 0; e < 4; ++e) y[e] = v[it][e] * inv * g[it][e];
       store4<TA>(o + d, y);
     }
   }
