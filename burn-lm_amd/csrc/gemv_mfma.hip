@@ -49,14 +49,22 @@ __global__ void __launch_bounds__(MAXT)
   // weights hold there adds nothing; the weight loads are unconditional, with the k-step clamped
   // into the matrix.
   uint4 a[KSTEPS];
-  if (KEEP_A) {
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      const int k = kbase + s * 32;
-      const uint4 v = ld16(ap + (k < K ? k : K - 8));
-      a[s] = (row < M && k < K && step0 + s < group_end) ? v : zero;
-    }
+  // Every load of the activations, and of the first tile's weights behind them, is asked for before the
+  // first fragment is looked at: zeroing the fragments one by one as they are loaded waits for each in
+  // turn, and the weights, which come the long way, would start a trip to memory later.  (The weights
+  // first is worse: loads come back in order, so the first product would wait for all of them.)
+#define GV_LOAD_ACTIVATIONS()                                                         \
+  _Pragma("unroll") for (int s = 0; s < KSTEPS; ++s) {                                \
+    const int k = kbase + s * 32;                                                     \
+    a[s] = ld16(ap + (k < K ? k : K - 8));                                            \
   }
+#define GV_ZERO_ACTIVATIONS()                                                         \
+  _Pragma("unroll") for (int s = 0; s < KSTEPS; ++s) {                                \
+    const int k = kbase + s * 32;                                                     \
+    const bool keep = row < M && k < K && step0 + s < group_end;                      \
+    a[s] = make_uint4(keep ? a[s].x : 0u, keep ? a[s].y : 0u, keep ? a[s].z : 0u, keep ? a[s].w : 0u); \
+  }
+  if (KEEP_A) GV_LOAD_ACTIVATIONS()
 
   // a block takes a run of neighbouring column tiles, so that it streams one contiguous piece of the
   // packed weights (blocks that each read their own region reach a higher memory rate than blocks
@@ -83,6 +91,10 @@ __global__ void __launch_bounds__(MAXT)
 #pragma unroll
     for (int s = 0; s < HALF; ++s) wb[s] = ld16_stream(wt + woff[HALF + s]);
   }
+  __builtin_amdgcn_sched_barrier(0);
+  if (KEEP_A) GV_ZERO_ACTIVATIONS()
+#undef GV_LOAD_ACTIVATIONS
+#undef GV_ZERO_ACTIVATIONS
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const bf16* wt = Wp + ((size_t)tile * k_steps * 64 + lane) * 8;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
