@@ -20,7 +20,7 @@ turns the core's failure codes into exceptions.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -115,7 +115,8 @@ class _Tables:
 
 
 class KVGroup:
-    def __init__(self, need: KVNeed, places: List[int], n_pages: int, page_size: int, dtype, device):
+    def __init__(self, need: KVNeed, places: List[Tuple], n_pages: int, page_size: int, dtype, device):
+        # places: (place of the layer order, index among that place's needs or None if it has one) per plane
         self.need, self.places = need, places
         self.page_size = page_size
         self.n_pages = n_pages
@@ -166,9 +167,11 @@ class StateView:
 
 
 class Cache:
-    """needs[i] is what place i of the layer order keeps (KVNeed, StateNeed or None);
+    """needs[i] is what place i of the layer order keeps: a KVNeed, a StateNeed, None, or a tuple
+    of them for a block whose parts each keep something of their own (keys and values beside a
+    state, two sets of keys and values); its view is then a tuple in the same order.
     reads_from[i] is the earlier place whose keys and values place i reads instead of keeping
-    its own (or None)."""
+    its own (or None); both places then have one need each."""
 
     def __init__(self, needs: Sequence, reads_from: Sequence[Optional[int]], max_tokens: int,
                  max_seqs: int, max_context: int, page_size: int = 64, dtype=torch.bfloat16,
@@ -181,36 +184,55 @@ class Cache:
         self.n_pages = (max_tokens + page_size - 1) // page_size
         self.table_width = (max_context + page_size - 1) // page_size
         self.groups: List[KVGroup] = []
-        self.views: List = [None] * len(needs)
         self.state_tensors: List[torch.Tensor] = []
-        by_need: Dict[KVNeed, List[int]] = {}
+        # a cell is one need: (place, None) for a place with one need, (place, j) for the j-th of several
+        cells: List[Tuple] = []
         for i, need in enumerate(needs):
-            if reads_from[i] is not None:
-                continue
-            if isinstance(need, KVNeed):
-                by_need.setdefault(need, []).append(i)
-        for need, places in by_need.items():
-            g = KVGroup(need, places, self.n_pages, page_size, dtype, device)
+            if isinstance(need, (tuple, list)):
+                if reads_from[i] is not None:
+                    raise CacheError(f"place {i} of the layer order has several needs and keeps them all itself: "
+                                     f"it cannot read the cache of place {reads_from[i]}")
+                cells += [((i, j), n) for j, n in enumerate(need)]
+            else:
+                cells.append(((i, None), need))
+        for key, need in cells:
+            if need is not None and not isinstance(need, (KVNeed, StateNeed)):
+                raise CacheError(f"place {key[0]} of the layer order asks for {need!r}: a need is a KVNeed, a StateNeed, "
+                                 f"None or a tuple of them")
+        cell_views: Dict[Tuple, object] = {key: None for key, _ in cells}
+        by_need: Dict[KVNeed, List[Tuple]] = {}
+        for key, need in cells:
+            if reads_from[key[0]] is None and isinstance(need, KVNeed):
+                by_need.setdefault(need, []).append(key)
+        for need, keys in by_need.items():
+            g = KVGroup(need, keys, self.n_pages, page_size, dtype, device)
             gi = len(self.groups)
             self.groups.append(g)
-            for plane, i in enumerate(places):
-                self.views[i] = KVView(g, gi, plane, store=True)
-        for i, need in enumerate(needs):
+            for plane, key in enumerate(keys):
+                cell_views[key] = KVView(g, gi, plane, store=True)
+        for key, need in cells:
+            i = key[0]
             src = reads_from[i]
             if src is not None:
-                if not (0 <= src < i) or reads_from[src] is not None or not isinstance(self.views[src], KVView):
+                sv = cell_views.get((src, None)) if 0 <= src < i else None
+                if reads_from[src] is not None or not isinstance(sv, KVView):
                     raise CacheError(f"place {i} of the layer order reads the cache of place {src}, which must be "
                                      f"an earlier place that keeps keys and values of its own")
-                sv = self.views[src]
                 if isinstance(need, KVNeed) and (need.n_kv_heads, need.head_dim, need.v_heads, need.v_dim) != \
                         (sv.need.n_kv_heads, sv.need.head_dim, sv.need.v_heads, sv.need.v_dim):
                     raise CacheError(f"place {i} cannot read the cache of place {src}: head counts or sizes differ")
                 g = self.groups[sv.group_index]
-                self.views[i] = KVView(g, sv.group_index, g.places.index(src), store=False)
+                cell_views[key] = KVView(g, sv.group_index, g.places.index((src, None)), store=False)
             elif isinstance(need, StateNeed):
                 t = torch.zeros(max_seqs, *need.shape, dtype=need.dtype, device=device)
                 self.state_tensors.append(t)
-                self.views[i] = StateView(t)
+                cell_views[key] = StateView(t)
+        self.views: List = []
+        for i, need in enumerate(needs):
+            if isinstance(need, (tuple, list)):
+                self.views.append(tuple(cell_views[(i, j)] for j in range(len(need))))
+            else:
+                self.views.append(cell_views[(i, None)])
         lib = _core.library()
         self._lib = lib
         self._h = lib.blm_cache_new(len(self.groups), _core.ints([g.n_pages for g in self.groups]),
@@ -226,7 +248,7 @@ class Cache:
         place of the order reads its group's keys and values (a place that shares another's cache
         reads them again), all of them or the last window."""
         total = 0
-        for v in self.views:
+        for v in (c for v in self.views for c in (v if isinstance(v, tuple) else (v,))):
             if isinstance(v, KVView):
                 keys = min(length, v.need.window) if v.need.window > 0 else length
                 total += (v.need.n_kv_heads * v.need.head_dim + v.need.v_heads * v.need.v_dim) * keys * v.k.element_size()

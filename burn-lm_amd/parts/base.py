@@ -24,7 +24,9 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
   projection followed by ``encode_and_store`` and which an encoding may fuse.
 * ``Block.roles`` (role -> family of the parts it arranges), ``Block.cache_need()`` and
   ``Block.forward(h, delta, step, view) -> delta``: runs its parts; the returned delta has not
-  been added to ``h`` yet (the next norm adds it, in float32).
+  been added to ``h`` yet (the next norm adds it, in float32).  A block with several parts that
+  each keep something (an attention beside a mixer with a state) returns a tuple of needs and
+  gets a tuple of views in the same order.
 """
 from __future__ import annotations
 
@@ -160,7 +162,8 @@ class Block:
     family each is (the registry's families: mixer, feed_forward, norm); the model builder makes the
     part a layer plan names for every role and hands the block the mapping role -> part.  The parts
     are also reachable as attributes (``self.mixer`` ...).  A block whose cache need is not simply
-    that of a role called ``mixer`` overrides ``cache_need``."""
+    that of a role called ``mixer`` overrides ``cache_need``; it may return a tuple of needs, one for
+    each of its parts that keeps something, and ``forward`` then gets a tuple of views in that order."""
     roles: Dict[str, str] = {}
 
     def __init__(self, parts: Dict[str, Part]):

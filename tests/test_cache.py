@@ -274,3 +274,29 @@ def test_advance_needs_reserved_pages():
         c.advance(a, 16)          # 21 tokens need a second page of 16
     c.advance(a, 11)              # the reserved page holds 16
     assert c.length(a) == 16
+
+
+def test_a_place_with_several_needs_gets_a_view_for_each():
+    kv, wide = KVNeed(2, 8), KVNeed(2, 8, window=32)
+    c = make([(kv, StateNeed((6,))), kv, (wide, kv, None), None], max_tokens=128)
+    assert isinstance(c.views[0], tuple) and isinstance(c.views[0][0], KVView) and isinstance(c.views[0][1], StateView)
+    assert isinstance(c.views[1], KVView) and c.views[3] is None
+    w, k, nothing = c.views[2]
+    assert isinstance(w, KVView) and isinstance(k, KVView) and nothing is None
+    full = next(g for g in c.groups if g.need.window == 0)
+    assert len(c.groups) == 2 and full.k_storage.shape[0] == 3           # three cells keep every key: three planes
+    planes = {v.k.data_ptr() for v in (c.views[0][0], c.views[1], k)}
+    assert len(planes) == 3 and w.group_index != k.group_index
+    # one step's pages serve every cell of a group; a state is zeroed when its slot opens
+    s = c.open()
+    c.views[0][1].tensor[s] += 3
+    c.reserve([(s, 40)]); c.advance(s, 40)
+    assert c.bytes_read(40) == (3 * 40 + 32) * 2 * (2 * 8) * c.views[1].k.element_size()
+    c.close(s)
+    assert c.open() == s and float(c.views[0][1].tensor[s].abs().sum()) == 0.0
+    with pytest.raises(CacheError, match="several needs"):
+        make([kv, (kv, StateNeed((2,)))], [None, 0])
+    with pytest.raises(CacheError, match="keeps keys and values of its own"):
+        make([(kv, StateNeed((2,))), kv], [None, 0])                    # a place with several needs lends none
+    with pytest.raises(CacheError, match="a need is"):
+        make([(kv, "keys")])

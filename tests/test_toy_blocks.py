@@ -181,3 +181,160 @@ def test_a_plan_that_names_a_role_its_block_does_not_have_is_refused(tmp_path):
     del plan.layers[0].parts["post_ffn_norm"]
     with pytest.raises(ValueError, match="lacks"):
         Model(plan)
+
+
+# ---- a block whose two mixers each keep something: keys and values beside a fixed-size state ----------------------
+
+HYBRID = dict(architectures=["ToyHybridLM"], width=80, inner=112, heads=5, kv_heads=5, head_dim=16, vocab=131, eps=1e-6,
+              theta=5000.0, decay=0.7, max_positions=256)
+
+
+def register_hybrid():
+    import math
+    from burn_lm_amd import registry
+    from burn_lm_amd.models.plan import LayerPlan, ModelPlan, Place
+    from burn_lm_amd.parts.base import Block, Mixer, PartSpec, StateNeed, TensorSpec
+
+    class RunningSumMixer(Mixer):
+        """params: width, decay.  names: w.  s_t = decay * s_{t-1} + x_t W, one float32 vector per sequence."""
+
+        def tensor_specs(self):
+            return {self.names["w"]: TensorSpec((self.params["width"],) * 2)}
+
+        def cache_need(self):
+            return StateNeed((self.params["width"],), torch.float32)
+
+        def bind(self, tensors, rt):
+            self.rt, self.w, self.a = rt, tensors[self.names["w"]], float(self.params["decay"])
+
+        def forward(self, x, step, view):
+            u = self.rt.linear(x, self.w).float()
+            out = torch.empty_like(u)
+            row = 0
+            for slot, n in zip(step.host_slots, step.host_new):
+                s = view.tensor[slot]
+                for t in range(row, row + n):
+                    s = self.a * s + u[t]
+                    out[t] = s
+                view.tensor[slot] = s
+                row += n
+            return out
+
+    class HybridBlock(Block):
+        """h = x + attention(norm(x)) + memory(norm(x)); y = h + ffn(ffn_norm(h)).  Both mixers keep
+        something for every sequence, so the block asks the cache for two things."""
+        roles = {"norm": "norm", "attention": "mixer", "memory": "mixer", "ffn_norm": "norm", "feed_forward": "feed_forward"}
+
+        def cache_need(self):
+            return (self.attention.cache_need(), self.memory.cache_need())
+
+        def forward(self, h, delta, step, view):
+            keys_and_values, state = view
+            x = self.norm.add_norm(h, delta)
+            planes = []
+            for d in (self.attention.forward(x, step, keys_and_values), self.memory.forward(x, step, state)):
+                planes += list(d.float()) if d.dim() == 3 else [d.float()]
+            x = self.ffn_norm.add_norm(h, torch.stack(planes).contiguous())
+            return self.feed_forward.forward(x, step)
+
+    def plan(cfg, names=None):
+        D = cfg["width"]
+        norm = lambda n: PartSpec("rmsnorm", dict(width=D, eps=cfg["eps"]), dict(weight=n))
+        attn = lambda i: PartSpec("attention", dict(width=D, heads=cfg["heads"], kv_heads=cfg["kv_heads"],
+                                                    head_dim=cfg["head_dim"], scale=1 / math.sqrt(cfg["head_dim"])),
+                                  dict(q=f"l{i}.q", k=f"l{i}.k", v=f"l{i}.v", o=f"l{i}.o"))
+        ffn = lambda i: PartSpec("swiglu", dict(width=D, inner=cfg["inner"]),
+                                 dict(gate=f"l{i}.gate", up=f"l{i}.up", down=f"l{i}.down"))
+        layers = [LayerPlan("toy_hybrid", position="rope", norm=norm("l0.n1"), attention=attn(0),
+                            memory=PartSpec("toy_running_sum", dict(width=D, decay=cfg["decay"]), dict(w="l0.w")),
+                            ffn_norm=norm("l0.n2"), feed_forward=ffn(0)),
+                  LayerPlan("pre_norm", position="rope", mixer_norm=norm("l1.n1"), mixer=attn(1), ffn_norm=norm("l1.n2"),
+                            feed_forward=ffn(1))]
+        # the hybrid layer runs twice; each run keeps keys, values and a state of its own
+        return ModelPlan(vocab_size=cfg["vocab"], width=D, max_positions=cfg["max_positions"],
+                         embedding=PartSpec("table", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         layers=layers, order=[Place(0), Place(1), Place(0)], final_norm=norm("norm"),
+                         head=PartSpec("linear", dict(vocab=cfg["vocab"], width=D), dict(weight="emb")),
+                         positions={"rope": PartSpec("rope", dict(head_dim=cfg["head_dim"], theta=cfg["theta"],
+                                                                  pairing="interleaved", scaling=None))})
+
+    def checkpoint_tensors(cfg):
+        D, hd, I = cfg["width"], cfg["head_dim"], cfg["inner"]
+        t = {"emb": ((cfg["vocab"], D), "table"), "norm": ((D,), "norm"), "l0.w": ((D, D), "matrix")}
+        for i in (0, 1):
+            t.update({f"l{i}.n1": ((D,), "norm"), f"l{i}.n2": ((D,), "norm"),
+                      f"l{i}.q": ((cfg["heads"] * hd, D), "matrix"), f"l{i}.k": ((cfg["kv_heads"] * hd, D), "matrix"),
+                      f"l{i}.v": ((cfg["kv_heads"] * hd, D), "matrix"), f"l{i}.o": ((D, cfg["heads"] * hd), "matrix"),
+                      f"l{i}.gate": ((I, D), "matrix"), f"l{i}.up": ((I, D), "matrix"), f"l{i}.down": ((D, I), "matrix")})
+        return t
+
+    registry.register_part("mixer", "toy_running_sum", RunningSumMixer)
+    registry.register_part("block", "toy_hybrid", HybridBlock)
+    registry.register_architecture(registry.Architecture("ToyHybridLM", read_config=lambda d: d, plan=plan,
+                                                         checkpoint_tensors=checkpoint_tensors))
+
+
+def hybrid_plain(tokens, w):
+    c = HYBRID
+    freqs = P.rope_base_frequencies(c["head_dim"], c["theta"])
+    attn = lambda x, i: P.attention_layer(x, w[f"l{i}.q"], w[f"l{i}.k"], w[f"l{i}.v"], w[f"l{i}.o"],
+                                          c["heads"], c["kv_heads"], c["head_dim"], freqs)
+    n = lambda x, name: P.rms_norm(x, w[name], c["eps"])
+    ffn = lambda x, i: P.swiglu_feed_forward(x, w[f"l{i}.gate"], w[f"l{i}.up"], w[f"l{i}.down"])
+
+    def running_sum(x):
+        u = x @ w["l0.w"].T
+        s, outs = np.zeros(c["width"]), []
+        for t in range(u.shape[1]):
+            s = c["decay"] * s + u[0, t]
+            outs.append(s)
+        return np.stack(outs)[None]
+
+    def hybrid(h):
+        x = n(h, "l0.n1")
+        h = h + attn(x, 0) + running_sum(x)
+        return h + ffn(n(h, "l0.n2"), 0)
+
+    h = hybrid(w["emb"][np.asarray(tokens)][None])
+    h = h + attn(n(h, "l1.n1"), 1)
+    h = h + ffn(n(h, "l1.n2"), 1)
+    h = hybrid(h)
+    return (n(h, "norm") @ w["emb"].T)[0]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_a_block_whose_two_mixers_keep_keys_and_values_and_a_state(tmp_path, dtype, tol):
+    import burn_lm_amd
+    from burn_lm_amd.cache.cache import KVView, StateView
+    from burn_lm_amd.engine.loading import load_engine
+    from burn_lm_amd.weights import safetensors_io as st
+    register_hybrid()
+    folder = burn_lm_amd.write_random_model(str(tmp_path), HYBRID, seed=9, std=0.1, norm_jitter=0.1)
+    f = st.open_folder(folder)
+    w = {n: f[n].tensor(n).double().numpy() for n in f}
+    eng = load_engine(folder, dtype=dtype, max_tokens=768, max_seqs=3)
+    views = eng.cache.views
+    assert [type(v) for v in views] == [tuple, KVView, tuple]
+    for v in (views[0], views[2]):
+        assert isinstance(v[0], KVView) and isinstance(v[1], StateView)
+    # three places keep keys and values of one shape: one group, three planes; two states of their own
+    assert len(eng.cache.groups) == 1 and eng.cache.groups[0].k_storage.shape[0] == 3
+    assert views[0][1].tensor.data_ptr() != views[2][1].tensor.data_ptr()
+    rng = np.random.default_rng(12)
+    for batch in ([70, 9, 33], [41, 100]):            # the second batch takes the slots and pages of the first
+        reqs = [[int(x) for x in rng.integers(0, HYBRID["vocab"], L)] for L in batch]
+        want = [hybrid_plain(r, w) for r in reqs]
+        slots = [eng.open() for _ in reqs]
+        cut = [len(r) - 4 for r in reqs]
+        got = eng.step([(s, r[:k], [0, k - 1]) for s, r, k in zip(slots, reqs, cut)]).double().cpu().numpy()
+        for i, k in enumerate(cut):
+            for j, p in enumerate((0, k - 1)):
+                assert np.abs(got[2 * i + j] - want[i][p]).max() / np.abs(want[i]).max() <= tol, (dtype, batch, i, p)
+        for j in range(4):
+            got = eng.step([(s, [r[k + j]], [0]) for s, r, k in zip(slots, reqs, cut)]).double().cpu().numpy()
+            for i in range(len(reqs)):
+                assert np.abs(got[i] - want[i][cut[i] + j]).max() / np.abs(want[i]).max() <= tol, (dtype, batch, i, cut[i] + j)
+        for s in slots:
+            eng.close(s)
+        assert eng.cache.pages_in_use() == 0
