@@ -37,14 +37,22 @@ def decode_splits(pages: int, blocks: int, head_dim: int, compute_units: int = 2
     wavefront and (for heads up to 64) three: a merge costs three trips through device-coherent memory in a
     row, about 3 us, a further page per wavefront about 2 (us per call, cut in two / uncut, 32 heads of 64
     in 8 groups: 8 pages at batch 1 7.1 / 6.6, at batch 8 8.1 / 7.0; 11 pages 7.9 / 8.0 and 9.0 / 8.4;
-    16 pages, cut in four, 7.3 / 10.2; heads of 128: 8 pages 11.1 / 11.1, 11 pages 12.8 / 13.7)."""
+    16 pages, cut in four, 7.3 / 10.2; heads of 128: 8 pages 11.1 / 11.1, 11 pages 12.8 / 13.7).  Where a
+    range is cut although the blocks are few, it is cut down to two pages per piece, not four (one
+    compute unit brings a page of wide heads, 32 KB, no faster than 60 GB/s: heads of 128 at batch 1,
+    11 pages: 2 pieces 13.0, uncut 11.1, 6 pieces 10.4; 16 pages: 4 pieces 12.1, 8 pieces 10.7; heads of 64,
+    16 pages: 4 pieces 7.9, 8 pieces 7.3), and ranges of up to 16 pages stay whole from a block for every
+    fourth compute unit on (heads of 128, 11 pages at batch 8: uncut 12.3, in two 14.0; 16 pages at batch
+    16: 16.9 / 18.5; heads of 64, 16 pages at batch 8: 9.1 / 10.0)."""
     if blocks >= compute_units or pages <= (12 if head_dim <= 64 else 8):
+        return 1
+    if pages <= 16 and blocks * 4 >= compute_units:
         return 1
     target = compute_units * DECODE_TARGET_PER_UNIT if head_dim <= 64 else max(1, compute_units * DECODE_TARGET_PER_UNIT // 2)
     least = max(1, int(compute_units * DECODE_MIN_PER_UNIT))
     n = min(max(1, pages // 8), (target + blocks - 1) // blocks, DECODE_MAX_PIECES)
     if blocks * n < least:
-        n = max(n, min(max(1, pages // 4), (least + blocks - 1) // blocks))
+        n = max(n, min(max(1, pages // 2), (least + blocks - 1) // blocks, DECODE_MAX_PIECES))
     return max(1, n)
 
 

@@ -156,7 +156,7 @@ def test_tokenizers_for_the_command_line(tmp_path):
 
 def test_decode_attention_split_rule():
     """How many pieces a sequence's pages are cut into for the decode attention: never more pieces
-    than pages, pieces of at least eight pages (four while the chip would be mostly idle), no more
+    than pages, pieces of at least eight pages (two while the chip would be mostly idle), no more
     blocks than the target."""
     from burn_lm_amd.parts.attention import decode_splits
     # the targets follow the chip: on half as many compute units, half as many pieces
@@ -167,14 +167,19 @@ def test_decode_attention_split_rule():
     assert decode_splits(64, 8, 128) == 16 and decode_splits(64, 64, 128) == 4      # wide heads: half the blocks
     assert decode_splits(1, 8, 64) == 1 and decode_splits(3, 8, 64) == 1 and decode_splits(8, 8, 64) == 1
     # short ranges stay whole: up to two pages per wavefront, three with heads up to 64
-    assert decode_splits(12, 8, 64) == 1 and decode_splits(13, 8, 64) == 3 and decode_splits(8, 8, 128) == 1 and decode_splits(12, 8, 128) == 3
+    assert decode_splits(12, 8, 64) == 1 and decode_splits(13, 8, 64) == 6 and decode_splits(8, 8, 128) == 1 and decode_splits(12, 8, 128) == 6
+    # 11 and 16 pages of wide heads at batch 1, 2, 4, 8, 16: two pages a piece while blocks are few, whole from 64 blocks on
+    assert [decode_splits(11, b * 8, 128) for b in (1, 2, 4, 8, 16)] == [5, 5, 4, 1, 1]
+    assert [decode_splits(16, b * 8, 128) for b in (1, 2, 4, 8, 16)] == [8, 8, 4, 1, 1]
+    assert [decode_splits(16, b * 8, 64) for b in (1, 2, 4, 8, 16)] == [8, 8, 4, 1, 1]
+    assert decode_splits(17, 64, 64) == 2                                           # beyond 16 pages the range is cut again
     assert decode_splits(2048, 8, 64) == 32 and decode_splits(512, 8, 64) == 32     # a long context at batch 1: the cap
     for pages in (1, 2, 5, 8, 9, 31, 64, 100, 1000):
         for blocks in (1, 3, 8, 64, 500, 5000):
             for hd in (64, 128):
                 n = decode_splits(pages, blocks, hd)
                 assert 1 <= n <= pages
-                assert n == 1 or pages // n >= 4
+                assert n == 1 or pages // n >= 2
 
 
 def test_command_line_random_models_delete(tmp_path, monkeypatch, capsys):
