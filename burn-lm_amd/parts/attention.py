@@ -14,8 +14,9 @@ import torch
 
 from .base import KVNeed, Mixer, TensorSpec
 
-# Blocks the decode attention aims for when it cuts the key ranges into pieces, per compute unit: two
-# (one where heads are wider than 64), at least half a block, and no cutting from one block per unit on.
+# Blocks the decode attention aims for when it cuts the key ranges into pieces: one round of at most one
+# block per compute unit, at least half of them busy, and no cutting from one block per unit on.
+# (DECODE_TARGET_PER_UNIT is what the generic kernel's one-wavefront blocks aim for.)
 DECODE_TARGET_PER_UNIT = 2
 DECODE_MIN_PER_UNIT = 0.5
 DECODE_MAX_PIECES = 32
@@ -24,11 +25,16 @@ DECODE_MAX_PIECES = 32
 def decode_splits(pages: int, blocks: int, head_dim: int, compute_units: int = 256) -> int:
     """Into how many pieces the decode attention cuts a sequence's pages.  Every piece is a block of
     four wavefronts that take pages in turn, and the pieces' results are merged by the last block to
-    finish, so a piece should hold two pages per wavefront (eight), or one (four) while that leaves
-    fewer than half a block per compute unit; and there is no point in more blocks than the chip takes at
-    once (pages of wide heads hold more bytes: half as many blocks reach the same memory rate).
+    finish, so a piece should hold two pages per wavefront (eight), or down to two pages in all while
+    that leaves fewer than half the compute units busy; and all blocks should run in one round, at most
+    one per compute unit: a second, partial round costs more than longer pieces do (us per call at a
+    context of 4,096, blocks in brackets; heads of 64, batch 6: 4 pieces (192) 13.8, 5 (240) 14.0, 6 (288)
+    16.2, 8 (384) 14.9, 10 (480) 14.5; batch 10: 3 (240) 18.5, 4 (320) 21.2, 6 (480) 18.9, 7 (560) 21.5;
+    batch 24: whole (192) 32.3, 3 (576) 41.6; heads of 128, whose blocks fill a compute unit's shared
+    memory alone: batch 10: 3 (240) 32.8, 4 (320) 44.0; batch 20: whole (160) 54.0, 2 (320) 71.9; the
+    same at contexts of 2,048 and 16,384).
     Measured at context 4096, head_dim 64, ms per step: batch 1: 16 pieces 0.870, 8: 0.880, 64: 1.002;
-    batch 2: 8 pieces 0.909, 16: 0.928; batch 4: 8 pieces 0.961, 16: 0.988; batch 8: 8 pieces best.
+    batch 2: 8 pieces 0.909, 16: 0.928; batch 4: 8 pieces 0.961, 16: 0.988; batch 8: 4 and 8 pieces equal.
     Never more than DECODE_MAX_PIECES: at batch 1 and a context of 32,768 the kernel takes 18.6 us with
     32 pieces, 22.3 with 64 and 31.4 with 128 (every piece costs its look-ups, its partial result and
     its arrival; the merge reads them all).  And no cutting at all once every compute unit has a block:
@@ -48,9 +54,8 @@ def decode_splits(pages: int, blocks: int, head_dim: int, compute_units: int = 2
         return 1
     if pages <= 16 and blocks * 4 >= compute_units:
         return 1
-    target = compute_units * DECODE_TARGET_PER_UNIT if head_dim <= 64 else max(1, compute_units * DECODE_TARGET_PER_UNIT // 2)
     least = max(1, int(compute_units * DECODE_MIN_PER_UNIT))
-    n = min(max(1, pages // 8), (target + blocks - 1) // blocks, DECODE_MAX_PIECES)
+    n = min(max(1, pages // 8), max(1, compute_units // blocks), DECODE_MAX_PIECES)
     if blocks * n < least:
         n = max(n, min(max(1, pages // 2), (least + blocks - 1) // blocks, DECODE_MAX_PIECES))
     return max(1, n)

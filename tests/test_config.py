@@ -162,7 +162,13 @@ def test_decode_attention_split_rule():
     # the targets follow the chip: on half as many compute units, half as many pieces
     assert decode_splits(64, 8, 64, compute_units=128) == 8 and decode_splits(64, 64, 64, compute_units=64) == 1
     # context 4096 (64 pages), 8 key-value heads: batch 1, 2, 4, 8, 16, 64
-    assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 32, 64)] == [16, 8, 8, 8, 4, 1, 1]
+    assert [decode_splits(64, b * 8, 64) for b in (1, 2, 4, 8, 16, 32, 64)] == [16, 8, 8, 4, 2, 1, 1]
+    # all blocks in one round, at most one per compute unit, also where the batch is no power of two
+    assert [decode_splits(64, b * 8, 64) for b in (3, 5, 6, 7, 10, 12, 14, 20, 24)] == [8, 6, 5, 4, 3, 2, 2, 1, 1]
+    assert [decode_splits(256, b * 8, 128) for b in (3, 5, 6, 10, 20)] == [10, 6, 5, 3, 1]
+    for b in range(1, 40):
+        for pages in (20, 64, 256, 2048):
+            assert b * 8 * decode_splits(pages, b * 8, 64) <= 256 or decode_splits(pages, b * 8, 64) == 1
     assert decode_splits(256, 32 * 8, 64) == 1                                      # every compute unit has a block: no cutting
     assert decode_splits(64, 8, 128) == 16 and decode_splits(64, 64, 128) == 4      # wide heads: half the blocks
     assert decode_splits(1, 8, 64) == 1 and decode_splits(3, 8, 64) == 1 and decode_splits(8, 8, 64) == 1
