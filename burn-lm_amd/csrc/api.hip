@@ -18,4 +18,4 @@ int blm_fail(const char* fmt, ...) {
 extern "C" const char* blm_last_error() { return g_error; }
 
 // ABI version: bumped when an entry point's signature changes, checked by the Python loader.
-extern "C" int blm_abi_version() { return 23; }
+extern "C" int blm_abi_version() { return 24; }

@@ -310,19 +310,54 @@ extern "C" int blm_gemv_mfma_supported(int M, int N, int K) {
   return (N >= 1 && K >= 8 && K % 8 == 0 && K <= blm_gemv_mfma_group_limit(M)) ? 1 : 0;
 }
 
+// The launch geometry of the product for M rows of [N, K] in k_groups groups of K: k-steps per
+// wavefront, wavefronts per block, and blocks per group.  A block takes a run of neighbouring column
+// tiles; enough blocks to fill the chip, few enough that a block uses its activations more than once,
+// and only blocks that have a tile.
+struct GemvGeometry {
+  int ksteps, waves, blocks;
+};
+static GemvGeometry gemv_geometry(int M, int N, int K, int k_groups) {
+  const int n_tiles = (N + 15) / 16;
+  const int k_steps = (K + 31) / 32;
+  const int steps_per_group = (k_steps + k_groups - 1) / k_groups;
+  GemvGeometry g{0, 0, 0};
+  int cap;
+  if (M > 16) {
+    g.ksteps = steps_per_group > 64 ? 16 : 8;   // more than 2048 of K per group: two row tiles at most
+    g.waves = (steps_per_group + g.ksteps - 1) / g.ksteps;   // at most 8 by the group limit
+    cap = 256 / k_groups;
+  } else {
+    g.waves = plan_k(steps_per_group * 32, &g.ksteps);
+    cap = (g.waves > 4 ? 256 : 512) / k_groups;
+  }
+  int blocks = n_tiles < cap ? n_tiles : (cap > 0 ? cap : 1);
+  const int tiles_per_block = (n_tiles + blocks - 1) / blocks;
+  g.blocks = (n_tiles + tiles_per_block - 1) / tiles_per_block;   // the kernel derives the same tiles per block from it
+  return g;
+}
+
+// Blocks (over all groups) and wavefronts per block that blm_gemv_mfma launches; 0 if K does not fit.
+extern "C" int blm_gemv_mfma_geometry(int M, int N, int K, int k_groups, int* blocks, int* waves) {
+  if (M < 1 || M > 64 || N < 1 || K < 8 || k_groups < 1 || k_groups > 64) return 0;
+  const int per_group = ((K + 31) / 32 + k_groups - 1) / k_groups * 32;
+  if (per_group > blm_gemv_mfma_group_limit(M)) return 0;
+  const GemvGeometry g = gemv_geometry(M, N, K, k_groups);
+  *blocks = g.blocks * k_groups;
+  *waves = g.waves;
+  return 1;
+}
+
 template <typename TC>
 static int launch_mfma(const void* A, const void* Wp, void* C, int M, int N, int K, int lda, int ldc, int c_mode,
                        int k_groups, hipStream_t stream) {
   const int n_tiles = (N + 15) / 16;
   const int k_steps = (K + 31) / 32;
   const int steps_per_group = (k_steps + k_groups - 1) / k_groups;
+  const GemvGeometry geo = gemv_geometry(M, N, K, k_groups);
   if (M > 16) {
     const int mt = (M + 15) / 16;
-    const int ks = steps_per_group > 64 ? 16 : 8;   // more than 2048 of K per group: two row tiles at most
-    const int waves = (steps_per_group + ks - 1) / ks;   // at most 8 by the group limit
-    int blocks = n_tiles;
-    const int cap = 256 / k_groups;
-    if (blocks > cap) blocks = cap > 0 ? cap : 1;
+    const int ks = geo.ksteps, waves = geo.waves, blocks = geo.blocks;
     dim3 grid(blocks, k_groups), block(waves * BLM_WAVE);
     const size_t smem = (size_t)waves * mt * 256 * sizeof(float);
 #define BLM_GR(MT, KS, PF)                                                                                      \
@@ -336,12 +371,7 @@ static int launch_mfma(const void* A, const void* Wp, void* C, int M, int N, int
     BLM_LAUNCH_CHECK("gemv_mfma_rows");
     return 0;
   }
-  int ksteps = 0;
-  const int waves = plan_k(steps_per_group * 32, &ksteps);
-  // enough blocks to fill the chip, few enough that a block reuses its activations
-  int blocks = n_tiles;
-  const int cap = (waves > 4 ? 256 : 512) / k_groups;
-  if (blocks > cap) blocks = cap > 0 ? cap : 1;
+  const int ksteps = geo.ksteps, waves = geo.waves, blocks = geo.blocks;
   dim3 grid(blocks, k_groups), block(waves * BLM_WAVE);
   const size_t smem = (size_t)waves * 256 * sizeof(float);
 #define BLM_GM(KS, MAXT, KEEP)                                                                                  \

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 23
+ABI_VERSION = 24
 _lib = None
 _lock = threading.Lock()
 
@@ -48,6 +48,7 @@ _SIGNATURES = {
     "blm_gemv_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_void_p],
     "blm_gemv_mfma_supported": [_c_int, _c_int, _c_int],
+    "blm_gemv_mfma_geometry": [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
     "blm_gemm_mfma_init": [],
     "blm_gemm_rows_init": [],
     "blm_gemm_rows": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -421,6 +422,14 @@ def gemv_mfma_supported(M, N, K):
 def gemv_mfma_group_limit(M):
     """The largest K that one K-group of gemv_mfma may span for M rows (0: M out of range)."""
     return int(library().blm_gemv_mfma_group_limit(int(M)))
+
+
+def gemv_mfma_geometry(M, N, K, groups=1):
+    """(blocks over all groups, wavefronts per block) that gemv_mfma launches for M rows of a [N, K]
+    matrix in that many groups of K, or None if a group's stretch of K is beyond what it takes."""
+    blocks, waves = ctypes.c_int(0), ctypes.c_int(0)
+    ok = library().blm_gemv_mfma_geometry(int(M), int(N), int(K), int(groups), ctypes.byref(blocks), ctypes.byref(waves))
+    return (blocks.value, waves.value) if ok else None
 
 
 def pack_weight(w, gated=False):

@@ -42,6 +42,11 @@ MFMA_SKINNY_MAX_ROWS = 64
 RING_GROUP_K = 2048
 # The shortest K a group keeps when a short K is cut for more blocks.
 RING_MIN_GROUP_K = 512
+# Numbers of groups that a skinny product's K may be cut into, the longest stretch of K a group gets where a
+# finer cut is to be had, and the least share of the compute units that the last round of blocks should keep busy.
+GROUP_CHOICES = (1, 2, 3, 4, 6, 8, 12, 16)
+GROUP_MAX_K = 4096
+GROUP_MIN_FILL = 0.6
 # 65 to 256 rows: the longest K at which the row-ring product with a block for every 64 rows still beats the
 # library's and the matrix-core kernel's planes (measured: ahead at 1536, 2048 and 2560, behind at 3072 and 4096).
 RING_MID_K = 2560
@@ -171,20 +176,34 @@ class Runtime:
         return LinearWeight(w, packable, gated)
 
     def k_groups(self, N, K, M=1):
-        """Into how many groups a skinny product's K is cut so that a narrow output still gives
-        every compute unit two blocks: groups * (N / 16) tiles should reach twice the compute units and a
-        group should span at most RING_GROUP_K of K, but keeps at least RING_MIN_GROUP_K (measured at the
-        1B shape: the output projection in 4 groups of 512 is 0.8 % of a step faster than in 2); and a
-        group must fit what the kernel takes for M rows."""
-        tiles = (N + 15) // 16
-        g = 1
-        while g < 8 and K // (g * 2) >= RING_MIN_GROUP_K and (tiles * g < 2 * self.compute_units or K // g > RING_GROUP_K):
-            g *= 2
-        limit = ops.gemv_mfma_group_limit(M)
-        steps = (K + 31) // 32
-        while g < 64 and (steps + g - 1) // g * 32 > limit:
-            g *= 2
-        return g
+        """Into how many groups a skinny product's K is cut: the fewest whose stretch of K is at most
+        GROUP_MAX_K (beyond it a wavefront re-reads its activations for every tile) and whose blocks fill
+        at least GROUP_MIN_FILL of their last round on the compute units.  Every block streams its stretch
+        of the weights at what one unit can bring, so the product takes as long as the unit with the most
+        blocks, and a number of blocks just above a multiple of the units leaves most of the chip idle for
+        a block's time; few groups of many wavefronts do better than many of few, and every group is a plane
+        that the next norm has to add.  Product and norm together, us at 8 rows (blocks x wavefronts in
+        brackets): [4096, 14336] in 4 groups (256x7) 25.1, in 8 (512x4) 28.1; [3072, 3072] in 1 (192x6) 9.4,
+        in 4 (384x2) 10.2; [2560, 11008] in 3 (240x8) 15.7, in 8 (432x3) 17.6, in 16 (512x2) 19.9; [1536, 6144]
+        in 2 (192x6) 9.4, in 8 (384x2) 11.2; [2048, 8192] in 2 (256x8) 11.4, in 3 (192x6) 12.0, in 4 (512x4) 11.3;
+        [2048, 2048] in 1 (128x4) 7.1, in 2 (256x2) 6.6; [8192, 8192] in 2 (256x8) 30.7, in 4 (512x4) 29.8."""
+        best, best_fill = None, -1.0
+        for g in GROUP_CHOICES:
+            if g > 1 and K // g < RING_MIN_GROUP_K:
+                break
+            geometry = ops.gemv_mfma_geometry(M, N, K, g)
+            if geometry is None or -(-K // g) > GROUP_MAX_K:
+                continue
+            blocks = geometry[0]
+            fill = blocks / (-(-blocks // self.compute_units) * self.compute_units)
+            if fill >= GROUP_MIN_FILL:
+                return g
+            if fill > best_fill:
+                best, best_fill = g, fill
+        if best is not None:
+            return best
+        # no grouping within the bounds: the coarsest one the kernel takes
+        return next((g for g in (1, 2, 4, 8, 16, 32, 64) if ops.gemv_mfma_geometry(M, N, K, g) is not None), 64)
 
     def rows_plan(self, N, K):
         """(groups of K, columns per block) for a product of 17 to 64 rows that may come as partial planes."""

@@ -324,8 +324,12 @@ def test_wide_layers_take_the_grouped_products(tmp_path):
                rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False)
     rt = Runtime(torch.bfloat16, "cuda:0")
     assert rt.compute_units == 256
-    assert rt.k_groups(2048, 2048) == 4 and rt.k_groups(2048, 4096) == 4 and rt.k_groups(6144, 2048) == 2
-    assert rt.k_groups(2048, 8192) == 4 and rt.k_groups(16384, 2048) == 1 and rt.k_groups(4096, 4096) == 2
+    # the fewest groups of at most 4096 of K whose blocks fill most of a round of the compute units
+    assert rt.k_groups(2048, 2048) == 2 and rt.k_groups(2048, 4096) == 2 and rt.k_groups(6144, 2048) == 1
+    assert rt.k_groups(2048, 8192) == 2 and rt.k_groups(16384, 2048) == 1 and rt.k_groups(4096, 4096) == 1
+    assert rt.k_groups(3072, 3072) == 1 and rt.k_groups(3072, 8192) == 2 and rt.k_groups(4096, 14336) == 4
+    assert rt.k_groups(2560, 11008) == 3 and rt.k_groups(96, 96) == 1 and rt.k_groups(2048, 100000) == 8
+    assert rt.k_groups(2048, 8192, 40) == 4 and rt.k_groups(4096, 14336, 40) == 8     # more rows: shorter groups
     folder = make_folder(tmp_path / "wide", cfg, seed=5, std=0.03)
     plain = P.load_model_folder(folder)
     reqs = [random_tokens(200 + i, 300, n) for i, n in enumerate([20, 9, 41])]

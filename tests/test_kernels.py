@@ -568,7 +568,8 @@ def test_gemv_mfma(ops, out_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,groups", [(8, 2048, 8192, 2), (3, 100, 2048, 2), (16, 48, 4104, 4), (1, 40, 8192, 8),
-                                          (64, 2048, 8192, 4), (24, 100, 8200, 8), (40, 48, 3000, 2), (33, 64, 14336, 8)])
+                                          (64, 2048, 8192, 4), (24, 100, 8200, 8), (40, 48, 3000, 2), (33, 64, 14336, 8),
+                                          (8, 2560, 11008, 3), (5, 72, 2600, 3), (16, 3072, 8192, 6), (2, 56, 12296, 12)])
 def test_gemv_mfma_partial_products_are_summed_by_the_norm(ops, M, N, K, groups):
     """K cut into groups handled by different blocks: each plane holds a partial product, their sum is
     the product, and the residual add in front of a norm takes the planes as they are."""
@@ -598,6 +599,15 @@ def test_gemv_mfma_partial_products_are_summed_by_the_norm(ops, M, N, K, groups)
     out2 = torch.empty(2, N, dtype=torch.bfloat16, device="cuda")
     ops.add_rmsnorm(hd2, planes, dev(gamma), 1e-5, out2, rows=dev(rows), write_h=False)
     assert torch.equal(out2.cpu(), out.cpu()[rows.long()]) and torch.equal(hd2.cpu(), h)
+
+
+def test_gemv_mfma_says_how_many_blocks_it_launches(ops):
+    """The routing counts on it: blocks over all groups and wavefronts per block, only blocks that have a tile."""
+    assert ops.gemv_mfma_geometry(8, 2048, 2048, 1) == (128, 4) and ops.gemv_mfma_geometry(8, 2048, 2048, 4) == (512, 4)
+    assert ops.gemv_mfma_geometry(8, 3072, 8192, 4) == (384, 4) and ops.gemv_mfma_geometry(8, 3072, 8192, 8) == (512, 2)
+    assert ops.gemv_mfma_geometry(8, 4096, 14336, 4) == (256, 7) and ops.gemv_mfma_geometry(1, 128256, 2048, 1) == (501, 4)
+    assert ops.gemv_mfma_geometry(40, 2048, 8192, 2) is None and ops.gemv_mfma_geometry(40, 2048, 8192, 4) == (256, 8)
+    assert ops.gemv_mfma_geometry(8, 48, 64, 1) == (3, 1)
 
 
 @pytest.mark.parametrize("M,I,K", [(8, 176, 64), (3, 384, 144), (16, 8, 520), (5, 1000, 2048), (1, 64, 4104), (4, 20000, 2048),
