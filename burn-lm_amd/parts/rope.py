@@ -10,6 +10,10 @@ Pairing: the reference pairs adjacent lanes ``(2i, 2i+1)`` and permutes Hugging 
 into that order when it imports them (nn/llama/import.rs:94-127).  ``pairing="half"`` pairs
 ``(i, i + head_dim/2)`` instead, which is the same function on un-permuted Hugging Face rows,
 so such checkpoints load without a re-layout.
+
+``rotary_dim`` (default: all of head_dim) turns only the first that many lanes of every head, with
+``theta_i = theta^(-2i/rotary_dim)``, and passes the rest through: the table holds angle zero for
+their pairs, so the kernels need not know (pairs of "half" are then ``(i, i + rotary_dim/2)``).
 """
 from __future__ import annotations
 
@@ -23,21 +27,26 @@ from .base import PositionEncoding
 PAIRING = {"interleaved": 0, "half": 1}
 
 
-def rope_frequencies(head_dim, theta, scaling=None):
-    """float64 [head_dim/2].  scaling: None or (factor, low_freq_factor, high_freq_factor, old_context)."""
-    i = np.arange(0, head_dim, 2, dtype=np.float64)
-    f = np.power(float(theta), -i / head_dim)
+def rope_frequencies(head_dim, theta, scaling=None, rotary_dim=None):
+    """float64 [head_dim/2].  scaling: None or (factor, low_freq_factor, high_freq_factor, old_context).
+    rotary_dim: lanes of a head that turn (default all); the pairs beyond them get frequency zero."""
+    turning = head_dim if rotary_dim is None else int(rotary_dim)
+    i = np.arange(0, turning, 2, dtype=np.float64)
+    f = np.power(float(theta), -i / turning)
     if scaling is not None:
         factor, low, high, old = (float(v) for v in scaling)
         wavelen = 2.0 * math.pi / f
         smooth = (old / wavelen - low) / (high - low)
         mid = (1.0 - smooth) * f / factor + smooth * f
         f = np.where(wavelen < old / high, f, np.where(wavelen > old / low, f / factor, mid))
+    if turning < head_dim:
+        f = np.concatenate([f, np.zeros((head_dim - turning) // 2)])
     return f
 
 
 class RotaryEncoding(PositionEncoding):
-    """params: head_dim, theta, scaling (None or 4 numbers), pairing ("half" | "interleaved")."""
+    """params: head_dim, theta, scaling (None or 4 numbers), pairing ("half" | "interleaved"),
+    rotary_dim (optional: the lanes of a head that turn, an even number up to head_dim)."""
     graph_safe = True
 
 
@@ -47,7 +56,10 @@ class RotaryEncoding(PositionEncoding):
         if self.params["pairing"] not in PAIRING:
             raise ValueError(f"rotary pairing {self.params['pairing']!r} unknown; one of {list(PAIRING)}")
         self.pairing = PAIRING[self.params["pairing"]]
-        self.freqs = rope_frequencies(self.head_dim, self.params["theta"], self.params.get("scaling"))
+        self.rotary_dim = int(self.params.get("rotary_dim") or self.head_dim)
+        if self.rotary_dim % 2 or not 2 <= self.rotary_dim <= self.head_dim or self.head_dim % 2:
+            raise ValueError(f"rotary_dim must be an even number from 2 to head_dim = {self.head_dim}, got {self.rotary_dim}")
+        self.freqs = rope_frequencies(self.head_dim, self.params["theta"], self.params.get("scaling"), self.rotary_dim)
         self._shared = {"table": None, "n_positions": 0}    # one table for this encoding and its adjacent-pair twin
         self._twin = None
 
@@ -75,14 +87,22 @@ class RotaryEncoding(PositionEncoding):
             twin.bind({}, self.rt)
             twin._shared = self._shared
             self._twin = twin
-        hd = self.head_dim
+        hd, rd = self.head_dim, self.rotary_dim
 
         def permute(w, n):
-            return w.reshape(n, 2, hd // 2, w.shape[1]).transpose(1, 2).reshape(n * hd, w.shape[1]).contiguous()
+            heads = w.reshape(n, hd, w.shape[1])
+            turning = heads[:, :rd].reshape(n, 2, rd // 2, w.shape[1]).transpose(1, 2).reshape(n, rd, w.shape[1])
+            return torch.cat([turning, heads[:, rd:]], dim=1).reshape(n * hd, w.shape[1]).contiguous()
 
         return permute(w_q, heads), permute(w_k, kv_heads), self._twin
 
+    def _check_pairs(self):
+        if self.pairing == PAIRING["half"] and self.rotary_dim < self.head_dim:
+            raise ValueError("pairs half the turning lanes apart exist only as adjacent pairs on permuted rows: "
+                             "bind the projections through for_projection and use the encoding it hands back")
+
     def encode_and_store(self, qkv, step, view, heads, kv_heads, head_dim, store=True):
+        self._check_pairs()
         if step.max_position >= self.n_positions:
             raise ValueError(f"position {step.max_position} is past the rotary table of {self.n_positions}")
         self.rt.ops.rope_kv_write(qkv, step.positions, step.token_seq, view.block_table(step), self.table,
@@ -95,6 +115,7 @@ class RotaryEncoding(PositionEncoding):
         exists for it; otherwise the three steps apart.  Which geometry suits which sizes is the
         runtime's answer (Runtime.qkv_plan); what is checked here is only what the rotation itself needs."""
         rt = self.rt
+        self._check_pairs()
         M, K = x.shape
         n_qkv = (heads + 2 * kv_heads) * head_dim
         plan = rt.qkv_plan(M, n_qkv, K) if hasattr(rt, "qkv_plan") else None

@@ -129,6 +129,79 @@ def test_attention_part(rt, pairing, heads, kv_heads, hd):
             assert rel(torch.cat(outs[i]), want[i]) <= TOL[rt.dtype], f"sequence {i}, cuts {cuts}"
 
 
+@pytest.mark.parametrize("pairing,heads,kv_heads,hd,turning", [("interleaved", 4, 2, 32, 8), ("half", 6, 3, 24, 16),
+                                                               ("half", 2, 1, 64, 32), ("interleaved", 3, 1, 48, 46)])
+def test_attention_part_with_only_part_of_each_head_rotated(rt, pairing, heads, kv_heads, hd, turning):
+    """rotary_dim: the first `turning` lanes of every head turn by theta^(-2i/turning), the rest pass through.  The plain side
+    rotates those lanes itself (adjacent pairs, or pairs half the turning lanes apart) and leaves the others alone; a prompt step of
+    unequal sequences, then single tokens."""
+    from burn_lm_amd import registry
+    from burn_lm_amd.cache.cache import Cache
+    from burn_lm_amd.engine.batch import build_step
+    D = 64
+    t, tn = weights(rt, 5, q=(heads * hd, D), k=(kv_heads * hd, D), v=(kv_heads * hd, D), o=(D, heads * hd))
+    rope = registry.part("position", "rope")(dict(head_dim=hd, theta=10000.0, pairing=pairing, scaling=None, rotary_dim=turning), {})
+    rope.bind({}, rt)
+    rope.prepare(256, rt)
+    assert rope.freqs.shape == (hd // 2,) and np.all(rope.freqs[turning // 2:] == 0)
+    np.testing.assert_allclose(rope.freqs[: turning // 2], P.rope_base_frequencies(turning, 10000.0), rtol=1e-12)
+    attn = registry.part("mixer", "attention")(
+        dict(width=D, heads=heads, kv_heads=kv_heads, head_dim=hd, scale=1 / math.sqrt(hd), window=0, position=rope),
+        dict(q="q", k="k", v="v", o="o"))
+    attn.bind(on_gpu(t), rt)
+    freqs = P.rope_base_frequencies(turning, 10000.0)
+
+    def turn(x, pos):     # x [heads, T, hd]
+        a = pos[:, None] * freqs[None, :]
+        c, s = np.cos(a), np.sin(a)
+        head, tail = x[..., :turning], x[..., turning:]
+        out = np.empty_like(head)
+        if pairing == "interleaved":
+            e, o = head[..., 0::2], head[..., 1::2]
+            out[..., 0::2], out[..., 1::2] = e * c - o * s, e * s + o * c
+        else:
+            lo, hi = head[..., : turning // 2], head[..., turning // 2:]
+            out[..., : turning // 2], out[..., turning // 2:] = lo * c - hi * s, lo * s + hi * c
+        return np.concatenate([out, tail], axis=-1)
+
+    def plain(x):
+        T = x.shape[0]
+        pos = np.arange(T, dtype=np.float64)
+        q = (x @ tn["q"].T).reshape(T, heads, hd).swapaxes(0, 1)
+        k = (x @ tn["k"].T).reshape(T, kv_heads, hd).swapaxes(0, 1)
+        v = (x @ tn["v"].T).reshape(T, kv_heads, hd).swapaxes(0, 1)
+        o = P.scaled_attention(turn(q, pos)[None], turn(k, pos)[None], v[None], P.hidden_mask(T, T))[0]
+        return o.swapaxes(0, 1).reshape(T, heads * hd) @ tn["o"].T
+
+    g = torch.Generator().manual_seed(8)
+    lens = [70, 3, 33]
+    xs = [(torch.randn(n, D, generator=g)).to(rt.dtype) for n in lens]
+    want = [plain(x.double().numpy()) for x in xs]
+    cache = Cache([attn.cache_need()], [None], 1024, 8, 256, PAGE, rt.dtype, rt.device)
+    slots = [cache.open() for _ in lens]
+    first = [n - 2 for n in lens]
+    outs = [[], [], []]
+    for chunk in range(3):
+        entries = [(s, [0] * (first[i] if chunk == 0 else 1), []) for i, s in enumerate(slots)]
+        cache.reserve([(s, len(tk)) for s, tk, _ in entries])
+        step = build_step(entries, cache, rt.device)
+        at = [0 if chunk == 0 else first[i] + chunk - 1 for i in range(3)]
+        x = torch.cat([xs[i][at[i]: at[i] + len(entries[i][1])] for i in range(3)]).to("cuda")
+        y = attn.forward(x, step, cache.views[0])
+        o = 0
+        for i in range(3):
+            n = len(entries[i][1])
+            outs[i].append(y[o:o + n]); o += n
+            cache.advance(slots[i], n)
+    for i in range(3):
+        assert rel(torch.cat(outs[i]), want[i]) <= TOL[rt.dtype], f"sequence {i}"
+    with pytest.raises(ValueError, match="rotary_dim"):
+        registry.part("position", "rope")(dict(head_dim=16, theta=1e4, pairing="half", rotary_dim=7), {}).bind({}, rt)
+    if pairing == "half":
+        with pytest.raises(ValueError, match="for_projection"):
+            rope.encode_and_store(None, None, None, heads, kv_heads, hd)
+
+
 def test_swiglu_part(rt):
     from burn_lm_amd import registry
     t, tn = weights(rt, 4, g=(200, 72), u=(200, 72), d=(72, 200))
