@@ -137,6 +137,7 @@ class Runtime:
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible to this process; burn-lm_amd has no CPU path")
         self.ops = ops
+        self._k_groups = {}     # (N, K, M) -> groups of K, as chosen once (see k_groups)
         ops.library()  # fail now, loudly, if the kernel library cannot be had
         ops.arrival_counters(self.device)   # allocated here, before any graph capture can be open
         ops.gemm_mfma_init(self.device)     # likewise: a function attribute is set once per device
@@ -187,6 +188,12 @@ class Runtime:
         in 4 (384x2) 10.2; [2560, 11008] in 3 (240x8) 15.7, in 8 (432x3) 17.6, in 16 (512x2) 19.9; [1536, 6144]
         in 2 (192x6) 9.4, in 8 (384x2) 11.2; [2048, 8192] in 2 (256x8) 11.4, in 3 (192x6) 12.0, in 4 (512x4) 11.3;
         [2048, 2048] in 1 (128x4) 7.1, in 2 (256x2) 6.6; [8192, 8192] in 2 (256x8) 30.7, in 4 (512x4) 29.8."""
+        known = self._k_groups.get((N, K, M))
+        if known is None:
+            known = self._k_groups[(N, K, M)] = self._choose_k_groups(N, K, M)
+        return known
+
+    def _choose_k_groups(self, N, K, M):
         best, best_fill = None, -1.0
         for g in GROUP_CHOICES:
             if g > 1 and K // g < RING_MIN_GROUP_K:
