@@ -118,7 +118,7 @@ def workload_hbm_frac(engine, batch, steps_per_second, prompt_len=512, generated
     return round((c["weight_bytes"] + c["cache_bytes"]) * steps_per_second / 1e9 / HBM_PEAK_GBS, 4)
 
 
-def other_shape(name, dtype, batch, context, steps, prefill_tokens):
+def other_shape(name, dtype, batch, context, steps, warmup, prefill_tokens):
     """Decode at `batch` and a prefill of `prefill_tokens` for another preset with all its layers: flat
     figures for the record's `shapes` block."""
     import torch
@@ -126,7 +126,7 @@ def other_shape(name, dtype, batch, context, steps, prefill_tokens):
     from burn_lm_amd.engine.loading import random_engine
     from burn_lm_amd.sampling.sampler import Sampler
     engine = random_engine(preset(name), seed=0, dtype=dtype, max_tokens=batch * context, max_seqs=batch, max_context=context)
-    sec, _ = time_decode(engine, Sampler(temperature=0.0), batch, context, steps, 4)
+    sec, _ = time_decode(engine, Sampler(temperature=0.0), batch, context, steps, warmup)
     roof = decode_roofline(engine, batch, context, steps, sec)
     psec = time_prefill(engine, prefill_tokens, reps=3)
     pflops = engine.model.step_costs([0], [prefill_tokens], 1)["flops"]
@@ -446,7 +446,7 @@ def main():
         del engine      # its storage goes back before the wider shapes are built
         torch.cuda.empty_cache()
         for name in ("llama3.2-3b", "llama3.1-8b"):
-            shapes.update(other_shape(name, args.dtype, args.batch, args.context, 24, T))
+            shapes.update(other_shape(name, args.dtype, args.batch, args.context, args.steps, args.warmup, T))   # timed as the headline is
         shapes.update(reference_bench_shapes(args.dtype))
     else:
         roof = decode_roofline(engine, args.batch, args.context, args.steps, sec)
