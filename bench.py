@@ -42,6 +42,9 @@ def random_prompts(engine, n, length, seed=0):
     return [[int(t) for t in rng.integers(0, engine.vocab_size, length)] for _ in range(n)]
 
 
+SETTLE_S = float(os.environ.get('BENCH_SETTLE', '0'))
+
+
 def time_decode(engine, sampler, batch, context, steps, warmup):
     """-> (seconds per step over `steps` steps, median seconds of the single steps).  The batch runs
     through the generation loop: its prompts end `warmup + steps + 2` tokens before the context."""
@@ -57,6 +60,9 @@ def time_decode(engine, sampler, batch, context, steps, warmup):
             return
         seen[0] += 1        # token 1 comes from the prompt step, token 1 + k from decode step k
         k = seen[0] - 1
+        if k == 0 and SETTLE_S > 0:
+            torch.cuda.synchronize()
+            time.sleep(SETTLE_S)
         if k in (warmup, warmup + steps):
             torch.cuda.synchronize()
             marks[k] = time.perf_counter()

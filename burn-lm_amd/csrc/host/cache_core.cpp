@@ -27,10 +27,26 @@ struct BlmPool {
   std::vector<char> out;        // out[p]: page p is held by somebody
 };
 
+// The pages are handed out in a fixed scrambled order, not 0, 1, 2, ...: sequences that get their pages in
+// one go would otherwise lie at equal distances of a power of two in memory (64 pages of 64 KB: 4 MB), and the
+// blocks of a decode attention, which read the same page number of every sequence at the same time, then
+// meet in the same memory channels (measured at a context of 4,096: batch 8 16.3 us a layer against 14.5 with
+// scattered pages, batch 32 48.2 against 42.3, batch 64 94.4 against 82.8; heads of 128 at batch 64 185
+// against 162).  A cache that has served a while is scattered anyway; this makes a fresh one so.
 static void pool_init(BlmPool& p, int n_pages) {
   p.n_pages = n_pages;
   p.free_list.resize(n_pages);
-  for (int i = 0; i < n_pages; ++i) p.free_list[i] = n_pages - 1 - i;   // page 0 first
+  for (int i = 0; i < n_pages; ++i) p.free_list[i] = i;
+  unsigned long long state = 0x9E3779B97F4A7C15ull;   // splitmix64 with a fixed seed: the same order in every run
+  for (int i = n_pages - 1; i > 0; --i) {
+    state += 0x9E3779B97F4A7C15ull;
+    unsigned long long z = state;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    const int j = (int)(z % (unsigned long long)(i + 1));
+    std::swap(p.free_list[i], p.free_list[j]);
+  }
   p.out.assign(n_pages, 0);
 }
 
